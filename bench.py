@@ -1,0 +1,161 @@
+"""Headline benchmark: 4-bit blockwise quantize + dequantize of a 16384 x 16384 fp32 tensor
+(268,435,456 elements, 1 GiB; 99% N(0,1) + 1% outliers of sigma 10; linear-2 table, block 64)
+on one MI355X, reported as achieved HBM GB/s over the algorithmic bytes.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+One "step" = one quantize launch + one dequantize launch over the whole tensor, inputs
+resident in HBM.  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for p in (str(ROOT), str(ROOT / "low-bit-shampoo_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0
+ORDER = 16384
+BLOCK = 64
+BITS = 4
+BYTES_PER_ELEMENT = 4 + BITS / 8 + 4 / BLOCK      # fp32 in/out + packed code + share of the fp32 maximum
+
+
+def stress_tensor(torch, order, seed=0):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn(order, order, device="cuda", generator=g)
+    mask = torch.rand(order, order, device="cuda", generator=g) < 0.01
+    x[mask] *= 10.0
+    return x
+
+
+def cpu_baseline(torch, x_slice, code):
+    """The reference's CPU code path (per-segment torch loop) on a bounded sample: 256 rows of
+    the same tensor viewed as a 2048 x 2048 matrix (identical segments)."""
+    from oracle import quant_loop_torch as QL
+    order = 2048
+    t0 = time.perf_counter()
+    out, absmax = QL.quantize_loop(x_slice, code, order, BLOCK, BITS)
+    QL.dequantize_loop(out, code, order, absmax, BLOCK, BITS)
+    dt = time.perf_counter() - t0
+    nbytes = 2 * BYTES_PER_ELEMENT * order * order
+    return {
+        "value": nbytes / dt / 1e9,
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": "rows 0-255 of the same tensor viewed as 2048x2048 (4,194,304 elements, 65,536 segments), "
+                  "quantize+dequantize with the per-segment torch loop of the reference's CPU path",
+        "seconds": dt,
+        "host_cpus": os.cpu_count(),
+        "torch_threads": torch.get_num_threads(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
+
+    import torch
+    import qtensor.functional as F
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU.")
+    if F.lib is None:
+        sys.exit("libqtensor_hip.so is missing; run `python -c 'import __graft_entry__ as g; g.build()'`.")
+
+    code_host = F.create_linear_map(True, BITS, 2)
+    code = code_host.cuda()
+    x = stress_tensor(torch, ORDER)
+    n = ORDER * ORDER
+    out = torch.empty(n * BITS // 8, dtype=torch.uint8, device="cuda")
+    absmax = torch.empty(n // BLOCK, dtype=torch.float32, device="cuda")
+    back = torch.empty(ORDER, ORDER, dtype=torch.float32, device="cuda")
+
+    def step():
+        F.quantize_blockwise(x, code, ORDER, absmax=absmax, out=out, blocksize=BLOCK, bits=BITS)
+        F.dequantize_blockwise(out, code, ORDER, absmax, out=back, blocksize=BLOCK, bits=BITS)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+
+    # per-kernel durations with events on the launch stream (torch's current stream)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    for e0, e1, e2 in ev:
+        e0.record()
+        F.quantize_blockwise(x, code, ORDER, absmax=absmax, out=out, blocksize=BLOCK, bits=BITS)
+        e1.record()
+        F.dequantize_blockwise(out, code, ORDER, absmax, out=back, blocksize=BLOCK, bits=BITS)
+        e2.record()
+    torch.cuda.synchronize()
+    q_ms = sum(e0.elapsed_time(e1) for e0, e1, _ in ev) / args.steps
+    d_ms = sum(e1.elapsed_time(e2) for _, e1, e2 in ev) / args.steps
+
+    algo = BYTES_PER_ELEMENT * n                     # per launch, same for quantize and dequantize
+    value = 2 * algo / (ms_per_step * 1e-3) / 1e9
+    q_gbs = algo / (q_ms * 1e-3) / 1e9
+    d_gbs = algo / (d_ms * 1e-3) / 1e9
+    result = {
+        "metric": "quant+dequant HBM GB/s",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "16384x16384 fp32 (99% N(0,1), 1% sigma-10 outliers), 4-bit linear-2 table, "
+                        "blocksize 64: blockwise quantize then dequantize of the whole tensor",
+            "elements": n,
+            "algorithmic_bytes_per_step": int(2 * algo),
+        },
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "quantize_flat_kernel<float,4,64,false,true>",
+            "achieved": round(q_gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(q_gbs / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "avg_launch_ms": round(q_ms, 4),
+            "algorithmic_bytes_per_launch": int(algo),
+        },
+        "dequantize": {
+            "kernel": "dequantize_flat_kernel<float,4,false>",
+            "achieved": round(d_gbs, 1),
+            "frac": round(d_gbs / HBM_PEAK_GBS, 4),
+            "avg_launch_ms": round(d_ms, 4),
+        },
+    }
+    if not args.no_cpu_baseline:
+        x_slice = x.view(-1)[: 2048 * 2048].cpu()
+        result["cpu_baseline"] = cpu_baseline(torch, x_slice, code_host)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,94 @@
+/*
+ * qtensor_hip.h -- C ABI of libqtensor_hip.so, the gfx950 replacement of the reference's
+ * libqtensor_cuda{XY}.so.
+ *
+ * All pointers are DEVICE pointers on the caller's current HIP device (the code table
+ * included).  The library never allocates, frees or retains caller memory, never
+ * synchronises the device, and is re-entrant.  Matrices are order x order, row-major,
+ * contiguous.  Quantisation segments are row pieces of `blocksize` consecutive elements
+ * (the last piece of a row is shorter when blocksize does not divide order);
+ * absmax[row * ceil(order/blocksize) + piece].  4-bit codes pack two per byte over the
+ * FLAT element stream, first element in the HIGH nibble, an odd tail padded with 0.
+ *
+ * Arithmetic is that of the reference's CPU path (qtensor/functional.py:526-746), NOT of
+ * its CUDA kernels: true fp32 division by the segment maximum, nearest table entry by two
+ * fp32-rounded distances with ties to the lower index, index 0 for all-zero segments,
+ * +0.0 when dequantizing a zero-maximum segment.
+ *
+ * The 16 unsuffixed entry points have exactly the names and argument order that the
+ * reference binds with ctypes (cudaC_python/csrc/pythonInterface.cpp:27-52, bound at
+ * qtensor/functional.py:17-60, called at :155, :211, :282, :343).  They launch on the
+ * null stream, as the reference's `<<<grid, threads>>>` launches do
+ * (cudaC_python/csrc/ops.cu:13).  Each has a `_stream` twin taking a hipStream_t as the
+ * last argument.  blocksize must be one of 64,128,256,512,1024,2048 and order >= 1;
+ * order*order must be below 2^31.  A violated precondition or a failed launch is
+ * reported on stderr and through qtensor_hip_last_error(); nothing is launched then.
+ * (The reference prints and calls exit(1), cudaC_python/csrc/ops.cuh:20-26.)
+ */
+#ifndef QTENSOR_HIP_H
+#define QTENSOR_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *qtensor_stream_t; /* a hipStream_t; NULL = the null stream */
+typedef uint16_t qtensor_bf16;  /* raw bfloat16 bits */
+
+/* Library/version probe; returns 10000*major + 100*minor + patch. */
+int qtensor_hip_version(void);
+/* 0 if the last call on this host thread succeeded, else a nonzero code; the text is in
+ * qtensor_hip_last_error_string().  Reading clears nothing; the next call resets it. */
+int qtensor_hip_last_error(void);
+const char *qtensor_hip_last_error_string(void);
+
+/* Replaces pythonInterface.cpp:29-33 (called from functional.py:155). */
+void cquantize_blockwise_8bit_fp32(float *A, float *code, int order, float *absmax, unsigned char *out, int blocksize);
+void cquantize_blockwise_8bit_bf16(qtensor_bf16 *A, float *code, int order, float *absmax, unsigned char *out, int blocksize);
+void cquantize_blockwise_4bit_fp32(float *A, float *code, int order, float *absmax, unsigned char *out, int blocksize);
+void cquantize_blockwise_4bit_bf16(qtensor_bf16 *A, float *code, int order, float *absmax, unsigned char *out, int blocksize);
+
+/* Replaces pythonInterface.cpp:35-39 (called from functional.py:211). */
+void cdequantize_blockwise_8bit_fp32(unsigned char *A, float *code, int order, float *absmax, float *out, int blocksize);
+void cdequantize_blockwise_8bit_bf16(unsigned char *A, float *code, int order, float *absmax, qtensor_bf16 *out, int blocksize);
+void cdequantize_blockwise_4bit_fp32(unsigned char *A, float *code, int order, float *absmax, float *out, int blocksize);
+void cdequantize_blockwise_4bit_bf16(unsigned char *A, float *code, int order, float *absmax, qtensor_bf16 *out, int blocksize);
+
+/* Replaces pythonInterface.cpp:41-45 (called from functional.py:282).  diag[order] receives
+ * the exact fp32 diagonal; the diagonal counts as 0 for the segment maxima and codes. */
+void cquantize_blockwise_diagreal_8bit_fp32(float *A, float *code, int order, float *absmax, float *diag, unsigned char *out, int blocksize);
+void cquantize_blockwise_diagreal_8bit_bf16(qtensor_bf16 *A, float *code, int order, float *absmax, float *diag, unsigned char *out, int blocksize);
+void cquantize_blockwise_diagreal_4bit_fp32(float *A, float *code, int order, float *absmax, float *diag, unsigned char *out, int blocksize);
+void cquantize_blockwise_diagreal_4bit_bf16(qtensor_bf16 *A, float *code, int order, float *absmax, float *diag, unsigned char *out, int blocksize);
+
+/* Replaces pythonInterface.cpp:47-51 (called from functional.py:343).  out[i,i] = diag[i]. */
+void cdequantize_blockwise_diagreal_8bit_fp32(unsigned char *A, float *code, int order, float *absmax, float *diag, float *out, int blocksize);
+void cdequantize_blockwise_diagreal_8bit_bf16(unsigned char *A, float *code, int order, float *absmax, float *diag, qtensor_bf16 *out, int blocksize);
+void cdequantize_blockwise_diagreal_4bit_fp32(unsigned char *A, float *code, int order, float *absmax, float *diag, float *out, int blocksize);
+void cdequantize_blockwise_diagreal_4bit_bf16(unsigned char *A, float *code, int order, float *absmax, float *diag, qtensor_bf16 *out, int blocksize);
+
+/* The same sixteen with an explicit stream (no counterpart in the reference, whose launches
+ * are pinned to the null stream; these let the host mirror follow torch's current stream). */
+void cquantize_blockwise_8bit_fp32_stream(float *A, float *code, int order, float *absmax, unsigned char *out, int blocksize, qtensor_stream_t stream);
+void cquantize_blockwise_8bit_bf16_stream(qtensor_bf16 *A, float *code, int order, float *absmax, unsigned char *out, int blocksize, qtensor_stream_t stream);
+void cquantize_blockwise_4bit_fp32_stream(float *A, float *code, int order, float *absmax, unsigned char *out, int blocksize, qtensor_stream_t stream);
+void cquantize_blockwise_4bit_bf16_stream(qtensor_bf16 *A, float *code, int order, float *absmax, unsigned char *out, int blocksize, qtensor_stream_t stream);
+void cdequantize_blockwise_8bit_fp32_stream(unsigned char *A, float *code, int order, float *absmax, float *out, int blocksize, qtensor_stream_t stream);
+void cdequantize_blockwise_8bit_bf16_stream(unsigned char *A, float *code, int order, float *absmax, qtensor_bf16 *out, int blocksize, qtensor_stream_t stream);
+void cdequantize_blockwise_4bit_fp32_stream(unsigned char *A, float *code, int order, float *absmax, float *out, int blocksize, qtensor_stream_t stream);
+void cdequantize_blockwise_4bit_bf16_stream(unsigned char *A, float *code, int order, float *absmax, qtensor_bf16 *out, int blocksize, qtensor_stream_t stream);
+void cquantize_blockwise_diagreal_8bit_fp32_stream(float *A, float *code, int order, float *absmax, float *diag, unsigned char *out, int blocksize, qtensor_stream_t stream);
+void cquantize_blockwise_diagreal_8bit_bf16_stream(qtensor_bf16 *A, float *code, int order, float *absmax, float *diag, unsigned char *out, int blocksize, qtensor_stream_t stream);
+void cquantize_blockwise_diagreal_4bit_fp32_stream(float *A, float *code, int order, float *absmax, float *diag, unsigned char *out, int blocksize, qtensor_stream_t stream);
+void cquantize_blockwise_diagreal_4bit_bf16_stream(qtensor_bf16 *A, float *code, int order, float *absmax, float *diag, unsigned char *out, int blocksize, qtensor_stream_t stream);
+void cdequantize_blockwise_diagreal_8bit_fp32_stream(unsigned char *A, float *code, int order, float *absmax, float *diag, float *out, int blocksize, qtensor_stream_t stream);
+void cdequantize_blockwise_diagreal_8bit_bf16_stream(unsigned char *A, float *code, int order, float *absmax, float *diag, qtensor_bf16 *out, int blocksize, qtensor_stream_t stream);
+void cdequantize_blockwise_diagreal_4bit_fp32_stream(unsigned char *A, float *code, int order, float *absmax, float *diag, float *out, int blocksize, qtensor_stream_t stream);
+void cdequantize_blockwise_diagreal_4bit_bf16_stream(unsigned char *A, float *code, int order, float *absmax, float *diag, qtensor_bf16 *out, int blocksize, qtensor_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QTENSOR_HIP_H */

@@ -36,7 +36,9 @@ static float canonical_nan(void) {
     return c.f;
 }
 
-/* fp32 <- bf16 (exact) and bf16 <- fp32 (round to nearest even; NaN kept quiet). */
+/* fp32 <- bf16 (exact) and bf16 <- fp32 (round to nearest even; every NaN becomes 0x7FC0,
+ * torch's scalar cast in functional.py:671 does the same; its vectorised cast yields another
+ * NaN pattern, so comparisons treat all NaNs alike). */
 float qo_bf16_to_f32(uint16_t h) {
     union { uint32_t u; float f; } c;
     c.u = ((uint32_t)h) << 16;
@@ -46,7 +48,7 @@ float qo_bf16_to_f32(uint16_t h) {
 uint16_t qo_f32_to_bf16(float x) {
     union { uint32_t u; float f; } c;
     c.f = x;
-    if ((c.u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((c.u >> 16) | 0x0040u);
+    if ((c.u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)0x7fc0u;
     uint32_t lsb = (c.u >> 16) & 1u;
     c.u += 0x7fffu + lsb;
     return (uint16_t)(c.u >> 16);

@@ -74,11 +74,12 @@ def dynamic_map(signed: bool = True, total_bits: int = 8, power: int = 1) -> np.
 
 # --------------------------------------------------------------------------- bf16
 def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
-    """Round-to-nearest-even float32 -> bfloat16, returned as uint16 bit patterns."""
+    """Round-to-nearest-even float32 -> bfloat16, returned as uint16 bit patterns; every NaN
+    becomes 0x7FC0 like torch's CPU cast."""
     u = np.ascontiguousarray(x, dtype=F32).view(np.uint32).astype(np.uint64)
     nan = (u & 0x7FFFFFFF) > 0x7F800000
     r = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
-    r = np.where(nan, (u >> 16) | 0x40, r)
+    r = np.where(nan, 0x7FC0, r)
     return r.astype(np.uint16)
 
 

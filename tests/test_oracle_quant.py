@@ -290,15 +290,18 @@ def test_python_scalar_form_agrees(code_maps, order):
 def test_bf16_round_trip_helpers_match_torch():
     rng = np.random.default_rng(0)
     x = np.concatenate([rng.standard_normal(4096).astype(F32) * F32(10.0) ** rng.integers(-20, 20, 4096),
-                        np.array([0.0, -0.0, np.inf, -np.inf, 1.00390625, 1.01171875], F32)]).astype(F32)
+                        np.array([0.0, -0.0, np.inf, -np.inf, 1.00390625, 1.01171875, np.nan, -np.nan], F32)]).astype(F32)
     mine = Q.f32_to_bf16_bits(x)
     theirs = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
-    assert np.array_equal(mine, theirs)
-    assert np.array_equal(Q.bf16_bits_to_f32(mine), torch.from_numpy(x).to(torch.bfloat16).float().numpy())
+    finite = ~np.isnan(x)
+    assert np.array_equal(mine[finite], theirs[finite])
+    # NaN payloads differ between torch's scalar and vectorised casts; any NaN is a NaN
+    assert np.all(np.isnan(Q.bf16_bits_to_f32(mine[~finite]))) and np.all(mine[~finite] == 0x7FC0)
+    assert np.array_equal(Q.bf16_bits_to_f32(mine), torch.from_numpy(x).to(torch.bfloat16).float().numpy(), equal_nan=True)
     lib = Q.c_lib()
     lib.qo_f32_to_bf16.restype = np.ctypeslib.ctypes.c_uint16
     lib.qo_f32_to_bf16.argtypes = [np.ctypeslib.ctypes.c_float]
-    assert all(lib.qo_f32_to_bf16(float(v)) == int(m) for v, m in zip(x[:512], mine[:512]))
+    assert all(lib.qo_f32_to_bf16(float(v)) == int(m) for v, m in zip(x[-520:], mine[-520:]))
 
 
 def test_bf16_output_rounding(code_maps):
