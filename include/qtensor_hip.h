@@ -88,6 +88,19 @@ void cdequantize_blockwise_diagreal_8bit_bf16_stream(unsigned char *A, float *co
 void cdequantize_blockwise_diagreal_4bit_fp32_stream(unsigned char *A, float *code, int order, float *absmax, float *diag, float *out, int blocksize, qtensor_stream_t stream);
 void cdequantize_blockwise_diagreal_4bit_bf16_stream(unsigned char *A, float *code, int order, float *absmax, float *diag, qtensor_bf16 *out, int blocksize, qtensor_stream_t stream);
 
+/* ---- self check and calibration (no counterpart in the reference) ------------------------
+ * The flat-path quantizer replaces IEEE division by the segment maximum a with r = rcp(a) refined
+ * by one Newton step and q = fma(fma(-x*r, a, x), r, x*r).  This entry point compares both
+ * with IEEE division on the device for every divisor bit pattern lo_bits, lo_bits+stride, ...
+ * <= hi_bits (0x21800000 = 2^-60 <= lo <= hi <= 0x5d800000 = 2^60), x_per_a pseudo-random
+ * numerators each.  counts (device, 3 x uint64, zeroed by the caller) receives
+ * {reciprocal mismatches, quotient mismatches, pairs tried}. */
+void qtensor_hip_check_fast_division(uint32_t lo_bits, uint32_t hi_bits, uint32_t stride, int x_per_a,
+                                     unsigned long long *counts, qtensor_stream_t stream);
+/* Plain device copy of n floats (n divisible by 4, 16-byte aligned): a kernel of exactly known
+ * HBM traffic (4n bytes read, 4n written) against which profiler byte counters are scaled. */
+void qtensor_hip_copy_f32(const float *src, float *dst, unsigned long long n, qtensor_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -2,7 +2,7 @@
 # Builds qtensor/libqtensor_hip.so for gfx950 (cross-compiles without a GPU).
 set -euo pipefail
 here="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
-out="${here}/../qtensor/libqtensor_hip.so"
+out="${QT_OUT:-${here}/../qtensor/libqtensor_hip.so}"
 HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
 # -ffp-contract=off: the nearest-entry rule needs two separately rounded fp32 subtractions.
 # packed-fp32-ops is switched off for the device pass on this pool.

@@ -4,86 +4,137 @@
 // then rounded to the output type; the diagreal form overwrites the diagonal with diag[]
 // (qtensor/functional.py:618-688 and :738-746 of the reference).
 //
-// flat path (blocksize divides order): one lane turns 2 bytes (4-bit) or 4 bytes (8-bit) of
-// codes into one 16-byte (fp32) or 8-byte (bf16) store, so the store stream -- eight ninths of
-// the traffic -- is perfectly coalesced.  general path: one thread per code byte.
+// flat path (blocksize divides order): codes are fetched 16 bytes per lane, turned around in
+// LDS, and written out as fully coalesced 16-byte (fp32) or 8-byte (bf16) stores per lane -- the
+// store stream is eight ninths of the traffic.  general path: one thread per code byte.
 #include "qt_common.h"
 
 namespace qt {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kUnroll = 4;
+#ifndef QT_D_THREADS
+#define QT_D_THREADS 256
+#endif
+#ifndef QT_D_BLOCKS_PER_CU
+#define QT_D_BLOCKS_PER_CU 3
+#endif
+#ifndef QT_D_CHUNKED
+#define QT_D_CHUNKED 0
+#endif
+constexpr int kThreads = 256;             // general-path kernel
+constexpr int kFlatThreads = QT_D_THREADS;
+constexpr int kFlatBlocksPerCU = QT_D_BLOCKS_PER_CU;
+constexpr int kSuper = 2048;              // elements a wave turns around per step
 
 template <typename T> struct Vec4Store;
 template <> struct Vec4Store<float> {
+    template <bool STREAM>
     static __device__ __forceinline__ void store(float *base, uint32_t k, float4 y) {
-        *reinterpret_cast<float4 *>(base + k) = y;
+        store_f32x4<STREAM>(base + k, y);
     }
     static __device__ __forceinline__ void store1(float *base, size_t k, float y) { base[k] = y; }
 };
 template <> struct Vec4Store<uint16_t> {
+    template <bool STREAM>
     static __device__ __forceinline__ void store(uint16_t *base, uint32_t k, float4 y) {
         uint2 w;
         w.x = (uint32_t)float_to_bf16_bits(y.x) | ((uint32_t)float_to_bf16_bits(y.y) << 16);
         w.y = (uint32_t)float_to_bf16_bits(y.z) | ((uint32_t)float_to_bf16_bits(y.w) << 16);
-        *reinterpret_cast<uint2 *>(base + k) = w;
+        store_u32x2<STREAM>(base + k, w);
     }
     static __device__ __forceinline__ void store1(uint16_t *base, size_t k, float y) { base[k] = float_to_bf16_bits(y); }
 };
 
-template <typename T, int BITS, bool DIAG>
-__global__ __launch_bounds__(kThreads) void dequantize_flat_kernel(
-    const uint8_t *__restrict__ q, const float *__restrict__ code, uint32_t n_vec, uint32_t bs_shift,
+// Flat path.  Per step a wave takes 2048 consecutive elements: their packed codes arrive with
+// one 16-byte (4-bit) or two 16-byte (8-bit) loads per lane and the segment maxima with one
+// 4-byte load on the first lanes; both are parked in the wave's private LDS area and read back
+// in the order that makes every one of the 8 output stores a fully coalesced 1 KiB (fp32) run.
+// The loads of the next step are issued before the stores of the current one.
+template <typename T, int BITS, bool DIAG, bool STREAM>
+__global__ __launch_bounds__(kFlatThreads) void dequantize_flat_kernel(
+    const uint8_t *__restrict__ q, const float *__restrict__ code, uint32_t n_super, uint32_t bs_shift,
     FastDiv row_div, const float *__restrict__ absmax, const float *__restrict__ diag, T *__restrict__ out) {
     constexpr int NCODE = 1 << BITS;
+    constexpr int kWaves = kFlatThreads / 64;
+    constexpr int CODE_VECS = BITS == 4 ? 1 : 2;            // uint4 loads per lane per step
     __shared__ float s_code[NCODE];
-    for (int i = threadIdx.x; i < NCODE; i += kThreads) s_code[i] = code[i];
+    __shared__ uint4 s_stage[kWaves][CODE_VECS * 64];
+    __shared__ float s_scale[kWaves][32];
+    for (int i = threadIdx.x; i < NCODE; i += kFlatThreads) s_code[i] = code[i];
     __syncthreads();
 
-    const uint32_t stride = gridDim.x * kThreads;
-    for (uint32_t base = blockIdx.x * kThreads + threadIdx.x; base < n_vec; base += stride * kUnroll) {
-        uint32_t packed[kUnroll];
-        float scale[kUnroll];
+    const uint32_t lane = threadIdx.x & 63u, w = threadIdx.x >> 6;
+    const uint32_t wave = blockIdx.x * kWaves + w;
+    const uint32_t n_waves = gridDim.x * kWaves;
+#if QT_D_CHUNKED
+    const uint32_t per = (n_super + n_waves - 1) / n_waves;
+    uint32_t st = wave * per;
+    const uint32_t end = min(st + per, n_super);
+    const uint32_t step = 1;
+#else
+    uint32_t st = wave;
+    const uint32_t end = n_super;
+    const uint32_t step = n_waves;
+#endif
+    if (st >= end) return;
+    const uint32_t last = end - 1;
+    const uint32_t seg_per_super = (uint32_t)kSuper >> bs_shift;   // 32 .. 1
+    const uint4 *q16 = reinterpret_cast<const uint4 *>(q);
+
+    uint4 c[CODE_VECS];
+    float a = 0.0f;
+    auto fetch = [&](uint32_t s) {
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const uint32_t i = base + (uint32_t)u * stride;
-            if (i < n_vec) {
-                packed[u] = BITS == 4 ? (uint32_t) reinterpret_cast<const uint16_t *>(q)[i]
-                                      : reinterpret_cast<const uint32_t *>(q)[i];
-                scale[u] = absmax[(i << 2) >> bs_shift];
-            }
+        for (int v = 0; v < CODE_VECS; ++v) c[v] = load_u32x4<STREAM>(q16 + (size_t)s * (CODE_VECS * 64) + v * 64 + lane);
+        if (lane < seg_per_super) a = absmax[s * seg_per_super + lane];
+    };
+    fetch(st);
+    const uint16_t *stage16 = reinterpret_cast<const uint16_t *>(&s_stage[w][0]);
+    const uint32_t *stage32 = reinterpret_cast<const uint32_t *>(&s_stage[w][0]);
+
+    for (; st < end; st += step) {
+#pragma unroll
+        for (int v = 0; v < CODE_VECS; ++v) s_stage[w][v * 64 + lane] = c[v];
+        if (lane < seg_per_super) s_scale[w][lane] = a;
+        fetch(min(st + step, last));
+        wave_lds_sync();
+
+        const uint32_t k4_0 = st * (uint32_t)(kSuper / 4) + lane;   // index of this lane's first 4-vector
+        uint32_t row = 0, col4 = 0;
+        if (DIAG) {
+            row = fastdiv(k4_0, row_div);
+            col4 = k4_0 - row * row_div.divisor;
         }
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const uint32_t i = base + (uint32_t)u * stride;
-            if (i >= n_vec) break;
+        for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t v4 = j * 64u + lane;                 // 4-vector inside the step
             uint32_t id0, id1, id2, id3;
             if (BITS == 4) {
-                id0 = (packed[u] >> 4) & 15u; id1 = packed[u] & 15u;
-                id2 = (packed[u] >> 12) & 15u; id3 = (packed[u] >> 8) & 15u;
+                const uint32_t p = stage16[v4];
+                id0 = (p >> 4) & 15u; id1 = p & 15u; id2 = (p >> 12) & 15u; id3 = (p >> 8) & 15u;
             } else {
-                id0 = packed[u] & 255u; id1 = (packed[u] >> 8) & 255u;
-                id2 = (packed[u] >> 16) & 255u; id3 = packed[u] >> 24;
+                const uint32_t p = stage32[v4];
+                id0 = p & 255u; id1 = (p >> 8) & 255u; id2 = (p >> 16) & 255u; id3 = p >> 24;
             }
-            const float a = scale[u];
+            const float scale = s_scale[w][(v4 << 2) >> bs_shift];
             float4 y;
-            if (a == 0.0f) {
+            if (scale == 0.0f) {
                 y = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             } else {
-                y = make_float4(s_code[id0] * a, s_code[id1] * a, s_code[id2] * a, s_code[id3] * a);
+                y = make_float4(s_code[id0] * scale, s_code[id1] * scale, s_code[id2] * scale, s_code[id3] * scale);
             }
             if (DIAG) {
-                const uint32_t row = fastdiv(i, row_div);
-                const uint32_t col4 = i - row * row_div.divisor;
                 if ((row >> 2) == col4) {
                     const float d = diag[row];
                     const uint32_t e = row & 3u;
                     if (e == 0) y.x = d; else if (e == 1) y.y = d; else if (e == 2) y.z = d; else y.w = d;
                 }
+                col4 += 64u;
+                while (col4 >= row_div.divisor) { col4 -= row_div.divisor; ++row; }
             }
-            Vec4Store<T>::store(out, i << 2, y);
+            Vec4Store<T>::template store<STREAM>(out, (k4_0 + j * 64u) << 2, y);
         }
+        wave_lds_sync();   // the staging area is rewritten at the top of the next step
     }
 }
 
@@ -144,12 +195,20 @@ void dequantize_dispatch(const uint8_t *q, const float *code, int order_i, const
     }
     const uint32_t order = (uint32_t)order_i, bs = (uint32_t)blocksize;
     const uint32_t total = order * order;
-    const bool flat = order % bs == 0 && is_aligned(out, 4 * sizeof(T)) && is_aligned(q, BITS == 4 ? 2 : 4) && is_aligned(absmax, 4);
+    const bool flat = order % bs == 0 && is_aligned(out, 4 * sizeof(T)) && is_aligned(q, 16) && is_aligned(absmax, 4);
     if (flat) {
-        const uint32_t n_vec = total / 4;
-        const uint32_t blocks = (n_vec + kThreads * kUnroll - 1) / (kThreads * kUnroll);
-        hipLaunchKernelGGL((dequantize_flat_kernel<T, BITS, DIAG>), dim3(capped_grid(blocks, 16)), dim3(kThreads), 0, stream,
-                           q, code, n_vec, (uint32_t)bs_shift, make_fastdiv(order / 4), absmax, diag, out);
+        constexpr uint32_t kWaves = kFlatThreads / 64;
+        const uint32_t n_super = total / kSuper;
+        const uint32_t blocks = (n_super + kWaves - 1) / kWaves;
+        const dim3 grid(capped_grid(blocks, kFlatBlocksPerCU));
+        // Outputs far beyond the 256 MB last-level cache are written with the streaming hint.
+        if (total >= (1u << 25)) {
+            hipLaunchKernelGGL((dequantize_flat_kernel<T, BITS, DIAG, true>), grid, dim3(kFlatThreads), 0, stream,
+                               q, code, n_super, (uint32_t)bs_shift, make_fastdiv(order / 4), absmax, diag, out);
+        } else {
+            hipLaunchKernelGGL((dequantize_flat_kernel<T, BITS, DIAG, false>), grid, dim3(kFlatThreads), 0, stream,
+                               q, code, n_super, (uint32_t)bs_shift, make_fastdiv(order / 4), absmax, diag, out);
+        }
     } else {
         const uint32_t nb = (order + bs - 1) / bs;
         const uint32_t n_bytes = (total * BITS + 7) / 8;

@@ -2,8 +2,8 @@
 //
 // Two paths:
 //  * flat path -- blocksize divides order.  The matrix is then a flat stream of whole segments
-//    (segment s = elements [s*BS, (s+1)*BS), absmax index s).  Each lane owns one 16-byte vector
-//    per 256-element slice, the segment maximum is a DPP butterfly over 16/32/64 lanes, the
+//    (segment s = elements [s*BS, (s+1)*BS), absmax index s).  A wave takes 2048 elements per
+//    step as 8 coalesced 16-byte loads per lane, the segment maximum is a DPP butterfly, the
 //    quotient is a correctly rounded fp32 division (one exact reciprocal per segment, then the
 //    multiply / residual-fma / correction-fma sequence), and the index is a threshold count
 //    done either through a bucket table in LDS (large inputs) or a binary search in LDS.
@@ -13,22 +13,34 @@
 // Arithmetic follows qtensor/functional.py:526-615 and :703-735 of the reference.
 #include "qt_common.h"
 #include "qt_tables.h"
+#include "qt_divide.h"
 
 namespace qt {
 namespace {
 
-constexpr int kThreads = 256;
+#ifndef QT_Q_THREADS
+#define QT_Q_THREADS 256
+#endif
+#ifndef QT_Q_BLOCKS_PER_CU
+#define QT_Q_BLOCKS_PER_CU 3
+#endif
+constexpr int kThreads = 256;            // general-path kernels
+constexpr int kFlatThreads = QT_Q_THREADS;
+constexpr int kFlatBlocksPerCU = QT_Q_BLOCKS_PER_CU;
+constexpr int kStep = 2048;              // elements a wave takes per step on the flat path
 
-template <typename T> struct Vec4Loader;
-template <> struct Vec4Loader<float> {
-    static __device__ __forceinline__ float4 load(const float *base, uint32_t k) {
-        return *reinterpret_cast<const float4 *>(base + k);
+template <typename T> struct ElementLoader;
+template <> struct ElementLoader<float> {
+    template <bool STREAM>
+    static __device__ __forceinline__ float4 load4(const float *base, uint32_t k) {
+        return load_f32x4<STREAM>(base + k);
     }
     static __device__ __forceinline__ float load1(const float *base, size_t k) { return base[k]; }
 };
-template <> struct Vec4Loader<uint16_t> {
-    static __device__ __forceinline__ float4 load(const uint16_t *base, uint32_t k) {
-        const uint2 w = *reinterpret_cast<const uint2 *>(base + k);
+template <> struct ElementLoader<uint16_t> {
+    template <bool STREAM>
+    static __device__ __forceinline__ float4 load4(const uint16_t *base, uint32_t k) {
+        const uint2 w = load_u32x2<STREAM>(base + k);
         return make_float4(__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u),
                            __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u));
     }
@@ -45,117 +57,180 @@ __device__ __forceinline__ uint32_t exact_index(float x, uint32_t amax_bits, con
     return t.perm[count_thresholds<NCODE>(q, t.thr)];
 }
 
-// Correctly rounded x / a for a in [2^-60, 2^60] and |x/a| >= 2^-40 (or x == 0), given
-// r = fl(1/a): q0 = fl(x*r) is within one ulp, the residual x - q0*a is exact in fp32, and one
-// more fma lands on the correctly rounded quotient (Markstein's division theorem).
-__device__ __forceinline__ float quotient(float x, float a, float r) {
-    const float q0 = x * r;
-    const float rem = __builtin_fmaf(-q0, a, x);
-    return __builtin_fmaf(rem, r, q0);
+// Bucket of a quotient known to satisfy |q| <= 1 (no upper clamp needed).
+__device__ __forceinline__ int lut_bucket_unit(float q) {
+    const uint32_t b = __float_as_uint(q);
+    int fb = (int)((b & 0x7fffffffu) >> kLutShift) - kLutBias;
+    fb = max(fb, 0);
+    return kLutPerSign + (fb ^ ((int)b >> 31));
 }
 
 template <int NCODE, bool USE_LUT>
 __device__ __forceinline__ uint32_t fast_index(float x, float a, float r, const CodeTables<NCODE> &t, const uint2 *lut) {
     const float q = quotient(x, a, r);
     if (USE_LUT) {
-        const uint2 e = lut[lut_bucket(q)];
+        const uint2 e = lut[lut_bucket_unit(q)];
         return e.y + (uint32_t)!(q < __uint_as_float(e.x));
     }
     return (uint32_t)count_thresholds<NCODE>(q, t.thr);
 }
 
-// One wave handles TILE = max(BS, 256) consecutive elements per iteration; VPT 16-byte
-// vectors per lane.  Segment = G lanes when BS <= 256, the whole wave otherwise.
-template <typename T, int BITS, int BS, bool DIAG, bool USE_LUT>
-__global__ __launch_bounds__(kThreads) void quantize_flat_kernel(
-    const T *__restrict__ A, const float *__restrict__ code, uint32_t n_tiles, FastDiv row_div,
+// Per-wave staging area: packed codes of one step in element order, and its segment maxima.
+template <int BITS>
+struct WaveStage {
+    uint4 codes[BITS == 4 ? 64 : 128];
+    float maxima[32];
+};
+
+// One step of a wave = 2048 consecutive elements, fetched as J = 8 fully coalesced 16-byte
+// loads per lane (vector j of lane L covers elements 256 j + 4 L .. +3).  A segment is G = BS/4
+// lanes of one vector for BS <= 256, and JS = BS/256 whole vectors of the wave above that.  The
+// packed codes and the maxima are parked in LDS so that they leave as one contiguous 1 KiB
+// (4-bit) or 2 KiB (8-bit) run and one run of 2048/BS floats per step.
+template <typename T, int BITS, int BS, bool DIAG, bool USE_LUT, bool STREAM>
+struct FlatQuantizer {
+    static constexpr int NCODE = 1 << BITS;
+    static constexpr int J = 8;
+    static constexpr int JS = BS > 256 ? BS / 256 : 1;
+    static constexpr int G = BS >= 256 ? 64 : BS / 4;
+    static constexpr int SEGS = kStep / BS;
+
+    const T *__restrict__ A;
+    float *__restrict__ absmax;
+    float *__restrict__ diag;
+    uint8_t *__restrict__ out;
+    const CodeTables<NCODE> &tab;
+    const uint2 *lut;
+    WaveStage<BITS> &stage;
+    FastDiv row_div;                                        // by order/4
+    bool fast_ok, ascending;
+    uint32_t lane;
+
+    struct Step {
+        float4 v[J];
+    };
+
+    __device__ __forceinline__ void load(Step &s, uint32_t step) const {
+        const uint32_t k0 = step * (uint32_t)kStep + lane * 4u;
+#pragma unroll
+        for (int j = 0; j < J; ++j) s.v[j] = ElementLoader<T>::template load4<STREAM>(A, k0 + (uint32_t)j * 256u);
+    }
+
+    __device__ __forceinline__ void process(Step &s, uint32_t step) const {
+        if (DIAG) {
+            const uint32_t k4 = step * (uint32_t)(kStep / 4) + lane;
+            uint32_t row = fastdiv(k4, row_div);
+            uint32_t col4 = k4 - row * row_div.divisor;
+#pragma unroll
+            for (int j = 0; j < J; ++j) {
+                if ((row >> 2) == col4) {                   // this vector holds element (row, row)
+                    const uint32_t e = row & 3u;
+                    float4 &v = s.v[j];
+                    diag[row] = e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w;
+                    if (e == 0) v.x = 0.0f; else if (e == 1) v.y = 0.0f; else if (e == 2) v.z = 0.0f; else v.w = 0.0f;
+                }
+                col4 += 64u;
+                while (col4 >= row_div.divisor) { col4 -= row_div.divisor; ++row; }
+            }
+        }
+
+        uint16_t *stage16 = reinterpret_cast<uint16_t *>(stage.codes);
+        uint32_t *stage32 = reinterpret_cast<uint32_t *>(stage.codes);
+#pragma unroll
+        for (int jg = 0; jg < J; jg += JS) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int jj = 0; jj < JS; ++jj) {
+                const float4 v = s.v[jg + jj];
+                m = max(max(m, max(abs_bits(v.x), abs_bits(v.y))), max(abs_bits(v.z), abs_bits(v.w)));
+            }
+            m = group_max_u32<G>(m);
+
+            // 2^-60 <= amax <= 2^60, else (zero, huge, tiny, inf, NaN) take the exact route
+            const bool special = !fast_ok || (m - kFastDivLo) > (kFastDivHi - kFastDivLo);
+            uint32_t idx[JS][4];
+            if (__any(special)) {
+                if (m > 0x7f800000u) m = 0x7fc00000u;       // any NaN in the segment -> canonical NaN
+#pragma unroll
+                for (int jj = 0; jj < JS; ++jj) {
+                    const float4 v = s.v[jg + jj];
+                    idx[jj][0] = exact_index<NCODE>(v.x, m, tab);
+                    idx[jj][1] = exact_index<NCODE>(v.y, m, tab);
+                    idx[jj][2] = exact_index<NCODE>(v.z, m, tab);
+                    idx[jj][3] = exact_index<NCODE>(v.w, m, tab);
+                }
+            } else {
+                const float amax = __uint_as_float(m);
+                const float r = exact_reciprocal(amax);
+#pragma unroll
+                for (int jj = 0; jj < JS; ++jj) {
+                    const float4 v = s.v[jg + jj];
+                    idx[jj][0] = fast_index<NCODE, USE_LUT>(v.x, amax, r, tab, lut);
+                    idx[jj][1] = fast_index<NCODE, USE_LUT>(v.y, amax, r, tab, lut);
+                    idx[jj][2] = fast_index<NCODE, USE_LUT>(v.z, amax, r, tab, lut);
+                    idx[jj][3] = fast_index<NCODE, USE_LUT>(v.w, amax, r, tab, lut);
+                }
+                if (!ascending) {
+#pragma unroll
+                    for (int jj = 0; jj < JS; ++jj)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) idx[jj][e] = tab.perm[idx[jj][e]];
+                }
+            }
+            if ((lane & (G - 1)) == 0) stage.maxima[(jg * 256 + (int)lane * 4) / BS] = __uint_as_float(m);
+#pragma unroll
+            for (int jj = 0; jj < JS; ++jj) {
+                const uint32_t *i = idx[jj];
+                if (BITS == 4)
+                    stage16[(jg + jj) * 64 + lane] = (uint16_t)(((i[0] << 4) | i[1]) | (((i[2] << 4) | i[3]) << 8));
+                else
+                    stage32[(jg + jj) * 64 + lane] = i[0] | (i[1] << 8) | (i[2] << 16) | (i[3] << 24);
+            }
+        }
+        wave_lds_sync();
+        uint4 *dst = reinterpret_cast<uint4 *>(out + (size_t)step * (kStep * BITS / 8));
+        dst[lane] = stage.codes[lane];
+        if (BITS == 8) dst[64 + lane] = stage.codes[64 + lane];
+        if (lane < SEGS) absmax[step * (uint32_t)SEGS + lane] = stage.maxima[lane];
+        wave_lds_sync();                                    // the next step rewrites the staging area
+    }
+};
+
+template <typename T, int BITS, int BS, bool DIAG, bool USE_LUT, bool STREAM>
+__global__ __launch_bounds__(kFlatThreads) void quantize_flat_kernel(
+    const T *__restrict__ A, const float *__restrict__ code, uint32_t n_steps, FastDiv row_div,
     float *__restrict__ absmax, float *__restrict__ diag, uint8_t *__restrict__ out) {
-    constexpr int NCODE = 1 << BITS;
-    constexpr int TILE = BS > 256 ? BS : 256;
-    constexpr int VPT = TILE / 256;
-    constexpr int G = BS >= 256 ? 64 : BS / 4;
+    using Q = FlatQuantizer<T, BITS, BS, DIAG, USE_LUT, STREAM>;
+    constexpr int NCODE = Q::NCODE;
+    constexpr int kWaves = kFlatThreads / 64;
 
     __shared__ CodeTables<NCODE> tab;
     __shared__ uint2 lut_mem[USE_LUT ? kLutEntries : 1];
+    __shared__ WaveStage<BITS> stages[kWaves];
     uint2 *lut = USE_LUT ? lut_mem : nullptr;
     build_code_tables<NCODE>(code, tab, lut);
     const int flags = tab.flags;
-    const bool fast_ok = (flags & kFlagLut) != 0;
-    const bool ascending = (flags & kFlagAscending) != 0;
 
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wave = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
-    const uint32_t n_waves = gridDim.x * (kThreads / 64);
-
-    for (uint32_t tile = wave; tile < n_tiles; tile += n_waves) {
-        const uint32_t k0 = tile * (uint32_t)TILE + lane * 4u;
-        float4 v[VPT];
-#pragma unroll
-        for (int j = 0; j < VPT; ++j) v[j] = Vec4Loader<T>::load(A, k0 + (uint32_t)j * 256u);
-
-        if (DIAG) {
-#pragma unroll
-            for (int j = 0; j < VPT; ++j) {
-                const uint32_t k4 = (k0 + (uint32_t)j * 256u) >> 2;
-                const uint32_t row = fastdiv(k4, row_div);
-                const uint32_t col4 = k4 - row * row_div.divisor;
-                if ((row >> 2) == col4) {
-                    const uint32_t e = row & 3u;
-                    const float d = e == 0 ? v[j].x : e == 1 ? v[j].y : e == 2 ? v[j].z : v[j].w;
-                    diag[row] = d;
-                    if (e == 0) v[j].x = 0.0f; else if (e == 1) v[j].y = 0.0f; else if (e == 2) v[j].z = 0.0f; else v[j].w = 0.0f;
-                }
-            }
-        }
-
-        uint32_t m = 0;
-#pragma unroll
-        for (int j = 0; j < VPT; ++j)
-            m = max(max(m, max(abs_bits(v[j].x), abs_bits(v[j].y))), max(abs_bits(v[j].z), abs_bits(v[j].w)));
-        m = group_max_u32<G>(m);
-        if (m > 0x7f800000u) m = 0x7fc00000u;   // any NaN in the segment -> canonical NaN
-        const float amax = __uint_as_float(m);
-        if ((lane & (G - 1)) == 0) absmax[tile * (uint32_t)(TILE / BS) + lane / G] = amax;
-
-        // 2^-60 <= amax <= 2^60, else (zero, huge, tiny, inf, NaN) take the exact route
-        const bool special = !fast_ok || (m - 0x21800000u) > (0x5d800000u - 0x21800000u);
-        uint32_t idx[VPT][4];
-        if (__any(special)) {
-#pragma unroll
-            for (int j = 0; j < VPT; ++j) {
-                idx[j][0] = exact_index<NCODE>(v[j].x, m, tab);
-                idx[j][1] = exact_index<NCODE>(v[j].y, m, tab);
-                idx[j][2] = exact_index<NCODE>(v[j].z, m, tab);
-                idx[j][3] = exact_index<NCODE>(v[j].w, m, tab);
-            }
-        } else {
-            const float r = 1.0f / amax;
-#pragma unroll
-            for (int j = 0; j < VPT; ++j) {
-                idx[j][0] = fast_index<NCODE, USE_LUT>(v[j].x, amax, r, tab, lut);
-                idx[j][1] = fast_index<NCODE, USE_LUT>(v[j].y, amax, r, tab, lut);
-                idx[j][2] = fast_index<NCODE, USE_LUT>(v[j].z, amax, r, tab, lut);
-                idx[j][3] = fast_index<NCODE, USE_LUT>(v[j].w, amax, r, tab, lut);
-            }
-            if (!ascending) {
-#pragma unroll
-                for (int j = 0; j < VPT; ++j)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) idx[j][e] = tab.perm[idx[j][e]];
-            }
-        }
-
-#pragma unroll
-        for (int j = 0; j < VPT; ++j) {
-            const uint32_t k = k0 + (uint32_t)j * 256u;
-            if (BITS == 4) {
-                const uint32_t h = ((idx[j][0] << 4) | idx[j][1]) | (((idx[j][2] << 4) | idx[j][3]) << 8);
-                *reinterpret_cast<uint16_t *>(out + (k >> 1)) = (uint16_t)h;
-            } else {
-                const uint32_t w = idx[j][0] | (idx[j][1] << 8) | (idx[j][2] << 16) | (idx[j][3] << 24);
-                *reinterpret_cast<uint32_t *>(out + k) = w;
-            }
-        }
+    const uint32_t w = threadIdx.x >> 6;
+    const Q q{A, absmax, diag, out, tab, lut, stages[w], row_div, (flags & kFlagLut) != 0,
+              (flags & kFlagAscending) != 0, threadIdx.x & 63u};
+    const uint32_t n_waves = gridDim.x * kWaves;
+    uint32_t step = blockIdx.x * kWaves + w;
+    if (step >= n_steps) return;
+    // Two register buffers in ping-pong: the loads of the next step are in flight while the
+    // current one is processed.  Look-ahead indices are clamped so every load is unconditional.
+    const uint32_t last = n_steps - 1;
+    typename Q::Step a, b;
+    q.load(a, step);
+    while (true) {
+        q.load(b, min(step + n_waves, last));
+        q.process(a, step);
+        step += n_waves;
+        if (step >= n_steps) break;
+        q.load(a, min(step + n_waves, last));
+        q.process(b, step);
+        step += n_waves;
+        if (step >= n_steps) break;
     }
 }
 
@@ -174,7 +249,7 @@ __global__ __launch_bounds__(kThreads) void segment_max_kernel(
         const size_t row0 = (size_t)r * order;
         uint32_t m = 0;
         for (uint32_t c = c0 + lane; c < c1; c += 64u) {
-            float x = Vec4Loader<T>::load1(A, row0 + c);
+            float x = ElementLoader<T>::load1(A, row0 + c);
             if (DIAG && c == r) { diag[r] = x; x = 0.0f; }
             m = max(m, abs_bits(x));
         }
@@ -202,7 +277,7 @@ __global__ __launch_bounds__(kThreads) void encode_kernel(
             uint32_t id = 0;
             if (k < total) {
                 const uint32_t r = k / order, c = k - r * order;
-                float x = Vec4Loader<T>::load1(A, k);
+                float x = ElementLoader<T>::load1(A, k);
                 if (DIAG && r == c) x = 0.0f;
                 id = exact_index<NCODE>(x, __float_as_uint(absmax[r * nb + c / bs]), tab);
             }
@@ -220,21 +295,24 @@ int grid_for(uint32_t work_items_per_block_unit, int blocks_per_cu) {
 
 template <typename T, int BITS, int BS, bool DIAG>
 void launch_flat(const T *A, const float *code, uint32_t order, float *absmax, float *diag, uint8_t *out, hipStream_t stream) {
-    constexpr uint32_t TILE = BS > 256 ? BS : 256;
+    constexpr uint32_t kWaves = kFlatThreads / 64;
     const uint32_t total = order * order;
-    const uint32_t n_tiles = total / TILE;
+    const uint32_t n_steps = total / kStep;
     const FastDiv rd = make_fastdiv(order / 4);
-    const uint32_t blocks_needed = (n_tiles + 3) / 4;
+    const uint32_t blocks_needed = (n_steps + kWaves - 1) / kWaves;
+    const int grid = grid_for(blocks_needed, kFlatBlocksPerCU);
     // The bucket table costs a few microseconds of set-up per workgroup; it pays from about
-    // a million elements on.
-    if (total >= (1u << 20)) {
-        const int grid = grid_for(blocks_needed, 5);
-        hipLaunchKernelGGL((quantize_flat_kernel<T, BITS, BS, DIAG, true>), dim3(grid), dim3(kThreads), 0, stream,
-                           A, code, n_tiles, rd, absmax, diag, out);
+    // a million elements on.  Inputs far beyond the 256 MB last-level cache are read with the
+    // streaming hint.
+    if (total >= (1u << 25)) {
+        hipLaunchKernelGGL((quantize_flat_kernel<T, BITS, BS, DIAG, true, true>), dim3(grid), dim3(kFlatThreads), 0, stream,
+                           A, code, n_steps, rd, absmax, diag, out);
+    } else if (total >= (1u << 20)) {
+        hipLaunchKernelGGL((quantize_flat_kernel<T, BITS, BS, DIAG, true, false>), dim3(grid), dim3(kFlatThreads), 0, stream,
+                           A, code, n_steps, rd, absmax, diag, out);
     } else {
-        const int grid = grid_for(blocks_needed, 8);
-        hipLaunchKernelGGL((quantize_flat_kernel<T, BITS, BS, DIAG, false>), dim3(grid), dim3(kThreads), 0, stream,
-                           A, code, n_tiles, rd, absmax, diag, out);
+        hipLaunchKernelGGL((quantize_flat_kernel<T, BITS, BS, DIAG, false, false>), dim3(grid), dim3(kFlatThreads), 0, stream,
+                           A, code, n_steps, rd, absmax, diag, out);
     }
 }
 
@@ -267,7 +345,7 @@ void quantize_dispatch(const T *A, const float *code, int order_i, float *absmax
         return;
     }
     const uint32_t order = (uint32_t)order_i, bs = (uint32_t)blocksize;
-    const bool flat = order % bs == 0 && is_aligned(A, 4 * sizeof(T)) && is_aligned(out, 4) && is_aligned(absmax, 4);
+    const bool flat = order % bs == 0 && is_aligned(A, 4 * sizeof(T)) && is_aligned(out, 16) && is_aligned(absmax, 4);
     if (flat) {
         switch (blocksize) {
             case 64: launch_flat<T, BITS, 64, DIAG>(A, code, order, absmax, diag, out, stream); break;
