@@ -24,6 +24,9 @@ ORDER = 16384
 BLOCK = 64
 BITS = 4
 BYTES_PER_ELEMENT = 4 + BITS / 8 + 4 / BLOCK      # fp32 in/out + packed code + share of the fp32 maximum
+# HBM bytes per launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE on this workload, scaled by
+# the library's plain copy kernel (summary: profiles/quantize_dequantize_16384sq_4bit_bs64_hbm_traffic.txt)
+MEASURED_TRAFFIC = {"quantize": 1225662500, "dequantize": 1225738000}
 
 
 def stress_tensor(torch, order, seed=0):
@@ -143,17 +146,18 @@ def main():
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "roofline": {
             "bound": "hbm",
-            "kernel": "quantize_flat_kernel<float,4,64,false,true>",
+            "kernel": "quantize_flat_kernel<float,4,64,false,true,true>",
             "achieved": round(q_gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(q_gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC["quantize"],
             "avg_launch_ms": round(q_ms, 4),
             "algorithmic_bytes_per_launch": int(algo),
         },
         "dequantize": {
-            "kernel": "dequantize_flat_kernel<float,4,false>",
+            "kernel": "dequantize_flat_kernel<float,4,false,true>",
+            "traffic": MEASURED_TRAFFIC["dequantize"],
             "achieved": round(d_gbs, 1),
             "frac": round(d_gbs / HBM_PEAK_GBS, 4),
             "avg_launch_ms": round(d_ms, 4),
