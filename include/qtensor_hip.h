@@ -101,6 +101,62 @@ void qtensor_hip_check_fast_division(uint32_t lo_bits, uint32_t hi_bits, uint32_
  * HBM traffic (4n bytes read, 4n written) against which profiler byte counters are scaled. */
 void qtensor_hip_copy_f32(const float *src, float *dst, unsigned long long n, qtensor_stream_t stream);
 
+/* ---- batched fp32 products on the matrix cores with fused (de)quantization --------------------
+ * Replaces, for a whole batch of equally shaped problems in one launch, what the reference
+ * does as separate torch calls per matrix:
+ *   P = dequantize(Pq); P @ G and G @ P        optimizers/shampoo2.py:255-268, shampoo1.py:224-237
+ *   G @ G.T, G.T @ G, L.mul_(b).add_(S, alpha=1-b) on the dequantized statistic
+ *                                              optimizers/shampoo1.py:164-178, shampoo2.py:185-199
+ *   the matmuls and max|M - I| of the coupled Newton inverse root
+ *                                              optimizers/matrix_functions.py:127-140
+ * C[b] = epilogue(opA(A[b]) * opB(B[b])), b = 0..batch-1, all matrices row-major fp32 unless
+ * quantized.  A quantized operand is a square matrix in the layout of cquantize_blockwise_*
+ * with blocksize dividing its order (diag optional); 4-bit codes need 4-byte, 8-bit codes
+ * 8-byte alignment. */
+typedef struct {
+    const void *base;           /* entry b lives at base + b * stride elements ...            */
+    const void *const *list;    /* ... unless list != NULL: then at list[b] (device array)    */
+    long long stride;
+} qtensor_batch_ptr;
+
+typedef struct {
+    qtensor_batch_ptr codes;    /* uint8                                                      */
+    qtensor_batch_ptr absmax;   /* float                                                      */
+    qtensor_batch_ptr diag;     /* float; both pointers NULL = plain form without diagonal    */
+    int order;
+    int bs_shift;               /* log2(blocksize), 6..11                                     */
+} qtensor_quant_ref;
+
+enum { QTENSOR_DENSE = 0, QTENSOR_DENSE_T = 1, QTENSOR_QUANT4 = 2, QTENSOR_QUANT8 = 3 };
+enum { QTENSOR_EPI_STORE = 0, QTENSOR_EPI_AXPBY_DENSE = 1, QTENSOR_EPI_AXPBY_QUANT4 = 2,
+       QTENSOR_EPI_AXPBY_QUANT8 = 3, QTENSOR_EPI_NEWTON = 4 };
+
+typedef struct {
+    int M, N, K, batch;
+    int kind_a;                 /* DENSE: A is M x K (lda); DENSE_T: stored K x M (lda); QUANT*: Aq, M == K   */
+    int kind_b;                 /* DENSE: B is K x N (ldb); DENSE_T: stored N x K (ldb); QUANT*: Bq, K == N   */
+    int epilogue;
+    struct {
+        int M_, N_, K_;         /* ignored (overwritten from the fields above)                 */
+        qtensor_batch_ptr A; int lda;
+        qtensor_batch_ptr B; int ldb;
+        qtensor_quant_ref Aq, Bq;
+        qtensor_batch_ptr C; int ldc;
+        float alpha, beta;      /* AXPBY: C = beta * E + alpha * (A B)                          */
+        qtensor_batch_ptr E; int lde;
+        qtensor_quant_ref Eq;   /* AXPBY_QUANT*: E is this quantized M x M matrix               */
+        qtensor_batch_ptr T; int ldt;   /* NEWTON: T = (1 - w) I + w (A B), besides C = A B     */
+        float newton_w;
+        float *err;             /* NEWTON: err[b] = max(err[b], max |A B - I|); caller zeroes   */
+        const int *skip;        /* optional device array: skip[b] != 0 leaves entry b untouched */
+        const float *code;      /* code table of the quantized operands / addend               */
+    } args;
+} qtensor_gemm_desc;
+
+/* Combinations built: (QUANT*, DENSE, STORE), (DENSE, QUANT*, STORE), (DENSE, DENSE_T, STORE|AXPBY_*),
+ * (DENSE_T, DENSE, STORE|AXPBY_*), (DENSE, DENSE, STORE|AXPBY_DENSE|NEWTON); anything else is an error. */
+void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,480 @@
+// fp32 matrix products on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32), with blockwise
+// quantized operands expanded on their way into LDS and the Shampoo epilogues fused in.
+//
+// What the reference does with separate steps
+//   P = dequantize(Pq);  out = P @ G            (optimizers/shampoo2.py:255-268, shampoo1.py:224-237)
+//   S = G @ G.T;  L = dequantize(Lq);  L.mul_(b).add_(S, alpha=1-b)   (shampoo1.py:164-178)
+//   the matmuls of the coupled Newton iteration  (optimizers/matrix_functions.py:131-140)
+// is done here as one launch per product over a whole batch of equally shaped problems.
+//
+// C[b] = epilogue( opA(A[b]) * opB(B[b]) ), b = blockIdx.z.  Row-major everywhere.
+//   operand kinds: dense (k contiguous for A, n contiguous for B), dense transposed, or a
+//   square 4/8-bit blockwise-quantized matrix (flat layout: blocksize divides the order).
+//   epilogues: plain store | beta * E + alpha * acc with E dense or quantized |
+//              Newton: C = acc, T = (1 - w) I + w * acc, err = max |acc - I|.
+//
+// Tiling: workgroup = 4 waves in a 2 x 2 grid, block tile BM x BN x 16, each wave owns
+// (BM/2) x (BN/2) as 32 x 32 MFMA blocks.  Both operand tiles sit in LDS as [row][k] with an odd
+// row stride so the per-lane fragment reads (row = lane % 32, k = lane / 32) hit 32 different
+// banks.  Global loads for tile t+1 are issued before the MFMAs of tile t.
+#include "qt_common.h"
+
+#include <type_traits>
+
+namespace qt {
+
+enum OperandKind : int { kDense = 0, kDenseT = 1, kQuant4 = 2, kQuant8 = 3 };
+enum EpilogueKind : int { kStore = 0, kAxpbyDense = 1, kAxpbyQuant4 = 2, kAxpbyQuant8 = 3, kNewton = 4 };
+
+// One matrix argument over the batch: either base + b * stride, or list[b] when list != nullptr.
+struct BatchPtr {
+    const void *base;
+    const void *const *list;
+    long long stride;   // in elements of the pointee type
+};
+
+struct QuantRef {       // a square blockwise-quantized matrix per batch entry
+    BatchPtr codes;     // uint8
+    BatchPtr absmax;    // float
+    BatchPtr diag;      // float, base == nullptr and list == nullptr: plain (no exact diagonal)
+    int order;
+    int bs_shift;       // log2(blocksize)
+};
+
+struct GemmArgs {
+    int M, N, K;
+    BatchPtr A; int lda;          // dense A: M x K (lda) or, transposed, K x M (lda)
+    BatchPtr B; int ldb;          // dense B: K x N (ldb) or, transposed, N x K (ldb)
+    QuantRef Aq, Bq;              // used when the operand kind is quantized
+    BatchPtr C; int ldc;
+    float alpha, beta;
+    BatchPtr E; int lde;          // dense addend for kAxpbyDense
+    QuantRef Eq;                  // quantized addend for kAxpbyQuant*
+    BatchPtr T; int ldt;          // kNewton: second output
+    float newton_w;               // kNewton: T = (1 - w) I + w acc
+    float *err;                   // kNewton: err[b] = max |acc - I| (must be zeroed by the caller)
+    const int *skip;              // optional: skip[b] != 0 -> this batch entry is left untouched
+    const float *code;            // code table for quantized operands / addend
+};
+
+namespace {
+
+constexpr int BK = 16;
+constexpr uint32_t kDies = 8;          // accelerator dies (XCDs) of an MI355X
+constexpr int LDS_STRIDE = BK + 1;
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <typename T>
+__device__ __forceinline__ const T *batch_ptr(const BatchPtr &p, int b) {
+    return p.list ? reinterpret_cast<const T *>(p.list[b]) : reinterpret_cast<const T *>(p.base) + (long long)b * p.stride;
+}
+
+__device__ __forceinline__ bool has_ptr(const BatchPtr &p) { return p.base != nullptr || p.list != nullptr; }
+inline bool has_host_ptr(const BatchPtr &p) { return p.base != nullptr || p.list != nullptr; }
+
+// Dequantized element (r, c) of a flat-layout quantized matrix.
+template <int BITS>
+__device__ __forceinline__ float dequant_element(const uint8_t *codes, const float *absmax, const float *diag,
+                                                 const float *s_code, int order, int bs_shift, int r, int c) {
+    if (diag != nullptr && r == c) return diag[r];
+    const long long k = (long long)r * order + c;
+    uint32_t id;
+    if (BITS == 8) id = codes[k];
+    else { const uint32_t byte = codes[k >> 1]; id = (k & 1) ? (byte & 15u) : (byte >> 4); }
+    const float a = absmax[k >> bs_shift];
+    return a == 0.0f ? 0.0f : s_code[id] * a;
+}
+
+// ---- tile loaders: global -> registers -> LDS ([row][k], row stride LDS_STRIDE) -------------
+// Every loader covers ROWS x BK elements with 256 threads and keeps them in registers between
+// `fetch` (global loads, issued early) and `commit` (LDS stores, after the barrier).
+
+// Dense, k contiguous in memory: element (row, k) at base[row * ld + k].
+template <int ROWS>
+struct LoadKContig {
+    static constexpr int VEC = ROWS * BK / 4 / 256;          // float4 per thread
+    float4 v[VEC];
+    __device__ __forceinline__ void fetch(const float *base, int ld, int row0, int k0, int rows, int K, bool vec_ok) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const int f = threadIdx.x + i * 256;
+            const int r = f >> 2, kq = (f & 3) << 2;
+            const int gr = row0 + r, gk = k0 + kq;
+            float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (gr < rows) {
+                const float *p = base + (long long)gr * ld + gk;
+                if (vec_ok && gk + 3 < K) x = *reinterpret_cast<const float4 *>(p);
+                else {
+                    if (gk < K) x.x = p[0];
+                    if (gk + 1 < K) x.y = p[1];
+                    if (gk + 2 < K) x.z = p[2];
+                    if (gk + 3 < K) x.w = p[3];
+                }
+            }
+            v[i] = x;
+        }
+    }
+    __device__ __forceinline__ void commit(float *lds) const {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const int f = threadIdx.x + i * 256;
+            const int r = f >> 2, kq = (f & 3) << 2;
+            float *d = lds + r * LDS_STRIDE + kq;
+            d[0] = v[i].x; d[1] = v[i].y; d[2] = v[i].z; d[3] = v[i].w;
+        }
+    }
+};
+
+// Dense, row index contiguous in memory: element (row, k) at base[k * ld + row].
+template <int ROWS>
+struct LoadRowContig {
+    static constexpr int VEC = ROWS * BK / 4 / 256;
+    float4 v[VEC];
+    __device__ __forceinline__ void fetch(const float *base, int ld, int row0, int k0, int rows, int K, bool vec_ok) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const int f = threadIdx.x + i * 256;
+            const int kk = f / (ROWS / 4), rq = (f % (ROWS / 4)) << 2;
+            const int gk = k0 + kk, gr = row0 + rq;
+            float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (gk < K) {
+                const float *p = base + (long long)gk * ld + gr;
+                if (vec_ok && gr + 3 < rows) x = *reinterpret_cast<const float4 *>(p);
+                else {
+                    if (gr < rows) x.x = p[0];
+                    if (gr + 1 < rows) x.y = p[1];
+                    if (gr + 2 < rows) x.z = p[2];
+                    if (gr + 3 < rows) x.w = p[3];
+                }
+            }
+            v[i] = x;
+        }
+    }
+    __device__ __forceinline__ void commit(float *lds) const {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const int f = threadIdx.x + i * 256;
+            const int kk = f / (ROWS / 4), rq = (f % (ROWS / 4)) << 2;
+            float *d = lds + rq * LDS_STRIDE + kk;
+            d[0] = v[i].x; d[LDS_STRIDE] = v[i].y; d[2 * LDS_STRIDE] = v[i].z; d[3 * LDS_STRIDE] = v[i].w;
+        }
+    }
+};
+
+// Quantized square matrix (order x order, flat layout).  ALONG_K: the tile's k runs along the
+// matrix columns (left factor); otherwise the tile's rows run along the matrix columns (right
+// factor).  Each thread expands 8 consecutive codes of one matrix row.
+template <int ROWS, int BITS, bool ALONG_K>
+struct LoadQuant {
+    static constexpr int TOTAL = ROWS * BK / 8;              // 8-element groups in the tile
+    static constexpr int GROUPS = (TOTAL + 255) / 256;       // per thread
+    float v[GROUPS][8];
+    __device__ __forceinline__ bool active(int g) const { return (int)threadIdx.x + g * 256 < TOTAL; }
+    __device__ __forceinline__ void locate(int g, int &mr, int &mc) const {
+        const int f = threadIdx.x + g * 256;
+        if (ALONG_K) { mr = f >> 1; mc = (f & 1) << 3; }                    // tile row = matrix row, 2 groups per row
+        else { mr = f / (ROWS / 8); mc = (f % (ROWS / 8)) << 3; }           // tile k = matrix row
+    }
+    __device__ __forceinline__ void fetch(const QuantRef &q, int b, const float *s_code, int row0, int k0) {
+        const uint8_t *codes = batch_ptr<uint8_t>(q.codes, b);
+        const float *absmax = batch_ptr<float>(q.absmax, b);
+        const float *diag = has_ptr(q.diag) ? batch_ptr<float>(q.diag, b) : nullptr;
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            if (!active(g)) continue;
+            int tr, tc;
+            locate(g, tr, tc);
+            const int mr = ALONG_K ? row0 + tr : k0 + tr;     // matrix row
+            const int mc = ALONG_K ? k0 + tc : row0 + tc;     // first matrix column of the group
+            if (mr < q.order && mc < q.order) {               // order is a multiple of 64: whole group inside
+                const long long k = (long long)mr * q.order + mc;
+                const float a = absmax[k >> q.bs_shift];
+                uint32_t id[8];
+                if (BITS == 4) {
+                    const uint32_t w = *reinterpret_cast<const uint32_t *>(codes + (k >> 1));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t byte = (w >> (8 * e)) & 255u;
+                        id[2 * e] = byte >> 4;
+                        id[2 * e + 1] = byte & 15u;
+                    }
+                } else {
+                    const uint2 w = *reinterpret_cast<const uint2 *>(codes + k);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) { id[e] = (w.x >> (8 * e)) & 255u; id[4 + e] = (w.y >> (8 * e)) & 255u; }
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[g][e] = a == 0.0f ? 0.0f : s_code[id[e]] * a;
+                if (diag != nullptr && mr >= mc && mr < mc + 8) v[g][mr - mc] = diag[mr];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[g][e] = 0.0f;
+            }
+        }
+    }
+    __device__ __forceinline__ void commit(float *lds) const {
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            if (!active(g)) continue;
+            int tr, tc;
+            locate(g, tr, tc);
+            if (ALONG_K) {
+                float *d = lds + tr * LDS_STRIDE + tc;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) d[e] = v[g][e];
+            } else {
+                float *d = lds + tc * LDS_STRIDE + tr;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) d[e * LDS_STRIDE] = v[g][e];
+            }
+        }
+    }
+};
+
+template <int BM, int BN, int KA, int KB, int EPI>
+__global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
+    constexpr int WM = BM / 2, WN = BN / 2, MI = WM / 32, NI = WN / 32;
+    // Workgroups are dealt round-robin to the 8 accelerator dies, each with its own L2.  Renumber
+    // them so that every die works through one contiguous run of (batch entry, tile row, tile
+    // column): the tiles that share operand panels then share an L2 as well.
+    const int tiles_n = (args.N + BN - 1) / BN, tiles_m = (args.M + BM - 1) / BM;
+    const uint32_t total = gridDim.x;
+    const uint32_t die = blockIdx.x % kDies, slot = blockIdx.x / kDies;
+    const uint32_t per = total / kDies, extra = total % kDies;
+    uint32_t id = die * per + min(die, extra) + slot;
+    const int tile_n = id % tiles_n;
+    id /= tiles_n;
+    const int tile_m = id % tiles_m;
+    const int b = id / tiles_m;
+    if (args.skip != nullptr && args.skip[b] != 0) return;
+
+    __shared__ float s_a[2][BM * LDS_STRIDE];
+    __shared__ float s_b[2][BN * LDS_STRIDE];
+    __shared__ float s_code[256];
+    constexpr bool kNeedCode = KA >= kQuant4 || KB >= kQuant4 || EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8;
+    if (kNeedCode) {
+        constexpr int NCODE = (KA == kQuant8 || KB == kQuant8 || EPI == kAxpbyQuant8) ? 256 : 16;
+        if ((int)threadIdx.x < NCODE) s_code[threadIdx.x] = args.code[threadIdx.x];
+        __syncthreads();
+    }
+
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+
+    const float *A = (KA < kQuant4) ? batch_ptr<float>(args.A, b) : nullptr;
+    const float *B = (KB < kQuant4) ? batch_ptr<float>(args.B, b) : nullptr;
+    const bool a_vec = KA < kQuant4 && (args.lda & 3) == 0 && is_aligned16(A);
+    const bool b_vec = KB < kQuant4 && (args.ldb & 3) == 0 && is_aligned16(B);
+
+    typename std::conditional<KA == kDense, LoadKContig<BM>,
+        typename std::conditional<KA == kDenseT, LoadRowContig<BM>,
+            LoadQuant<BM, KA == kQuant4 ? 4 : 8, true>>::type>::type la;
+    typename std::conditional<KB == kDense, LoadRowContig<BN>,
+        typename std::conditional<KB == kDenseT, LoadKContig<BN>,
+            LoadQuant<BN, KB == kQuant4 ? 4 : 8, false>>::type>::type lb;
+
+    auto fetch = [&](int k0) {
+        if constexpr (KA < kQuant4) la.fetch(A, args.lda, m0, k0, args.M, args.K, a_vec);
+        else la.fetch(args.Aq, b, s_code, m0, k0);
+        if constexpr (KB < kQuant4) lb.fetch(B, args.ldb, n0, k0, args.N, args.K, b_vec);
+        else lb.fetch(args.Bq, b, s_code, n0, k0);
+    };
+
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // Pipeline: tile t is multiplied out of one LDS buffer while tile t+1 (already in registers,
+    // its loads were issued a whole tile earlier) is written to the other buffer half-way through
+    // the MFMA stream and the loads of tile t+2 are issued right after.  One barrier per tile.
+    const int n_tiles = (args.K + BK - 1) / BK;
+    fetch(0);
+    la.commit(s_a[0]);
+    lb.commit(s_b[0]);
+    if (n_tiles > 1) fetch(BK);
+    __syncthreads();
+    const int frag_row = lane & 31, frag_k = lane >> 5;
+    for (int t = 0; t < n_tiles; ++t) {
+        const int cur = t & 1;
+        const float *pa = s_a[cur] + (wm + frag_row) * LDS_STRIDE + frag_k;
+        const float *pb = s_b[cur] + (wn + frag_row) * LDS_STRIDE + frag_k;
+        // fragments for step ks+1 are read from LDS before the MFMAs of step ks are issued
+        float fa[2][MI], fb[2][NI];
+#pragma unroll
+        for (int i = 0; i < MI; ++i) fa[0][i] = pa[i * 32 * LDS_STRIDE];
+#pragma unroll
+        for (int j = 0; j < NI; ++j) fb[0][j] = pb[j * 32 * LDS_STRIDE];
+#pragma unroll
+        for (int ks = 0; ks < BK / 2; ++ks) {
+            const int now = ks & 1, nxt = now ^ 1;
+            if (ks + 1 < BK / 2) {
+#pragma unroll
+                for (int i = 0; i < MI; ++i) fa[nxt][i] = pa[i * 32 * LDS_STRIDE + 2 * (ks + 1)];
+#pragma unroll
+                for (int j = 0; j < NI; ++j) fb[nxt][j] = pb[j * 32 * LDS_STRIDE + 2 * (ks + 1)];
+            }
+            if (ks == BK / 4 && t + 1 < n_tiles) {
+                la.commit(s_a[cur ^ 1]);
+                lb.commit(s_b[cur ^ 1]);
+                if (t + 2 < n_tiles) fetch((t + 2) * BK);
+            }
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[now][i], fb[now][j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
+    float *C = const_cast<float *>(batch_ptr<float>(args.C, b));
+    float local_err = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int col = n0 + wn + j * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (row >= args.M || col >= args.N) continue;
+                float y = acc[i][j][r];
+                if (EPI == kAxpbyDense) {
+                    const float *E = batch_ptr<float>(args.E, b);
+                    y = args.beta * E[(long long)row * args.lde + col] + args.alpha * y;
+                } else if (EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8) {
+                    const float e = dequant_element<EPI == kAxpbyQuant4 ? 4 : 8>(
+                        batch_ptr<uint8_t>(args.Eq.codes, b), batch_ptr<float>(args.Eq.absmax, b),
+                        has_ptr(args.Eq.diag) ? batch_ptr<float>(args.Eq.diag, b) : nullptr, s_code, args.Eq.order,
+                        args.Eq.bs_shift, row, col);
+                    // same two roundings as tensor.mul_(beta).add_(S, alpha=1-beta)
+                    y = __builtin_fmaf(args.alpha, y, args.beta * e);
+                } else if (EPI == kNewton) {
+                    const float eye = row == col ? 1.0f : 0.0f;
+                    local_err = fmaxf(local_err, fabsf(y - eye));
+                    float *T = const_cast<float *>(batch_ptr<float>(args.T, b));
+                    T[(long long)row * args.ldt + col] = (1.0f - args.newton_w) * eye + args.newton_w * y;
+                }
+                C[(long long)row * args.ldc + col] = y;
+            }
+        }
+    if (EPI == kNewton) {
+        uint32_t e = group_max_u32<64>(__float_as_uint(local_err));   // non-negative floats order like their bits
+        if (lane == 0) atomicMax(reinterpret_cast<unsigned int *>(args.err) + b, e);
+    }
+}
+
+
+template <int BM, int BN, int KA, int KB, int EPI>
+void launch_gemm(const GemmArgs &a, int batch, hipStream_t stream) {
+    const long long blocks = (long long)((a.N + BN - 1) / BN) * ((a.M + BM - 1) / BM) * batch;
+    if (blocks > 0x7fffffffLL) { set_error(kBadArgument, "gemm: too many tiles (%lld)", blocks); return; }
+    hipLaunchKernelGGL((gemm_kernel<BM, BN, KA, KB, EPI>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+}
+
+bool valid_quant(const QuantRef &q, int bits, const char *what) {
+    const int bs = 1 << q.bs_shift;
+    if (q.bs_shift < 6 || q.bs_shift > 11 || q.order < bs || q.order % bs != 0) {
+        set_error(kBadArgument, "gemm: %s: quantized matrices need blocksize in 64..2048 dividing the order (order %d, blocksize %d)",
+                  what, q.order, bs);
+        return false;
+    }
+    if (!has_host_ptr(q.codes) || !has_host_ptr(q.absmax)) {
+        set_error(kNullPointer, "gemm: %s: null codes/absmax pointer", what);
+        return false;
+    }
+    (void)bits;
+    return true;
+}
+
+}  // namespace
+}  // namespace qt
+
+// Flat C description of one batched product (see include/qtensor_hip.h for the field meanings).
+struct qtensor_gemm_desc {
+    int M, N, K, batch;
+    int kind_a, kind_b, epilogue;
+    qt::GemmArgs args;
+};
+
+extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
+    using namespace qt;
+    clear_error();
+    hipStream_t stream = (hipStream_t)stream_v;
+    if (!d) { set_error(kNullPointer, "gemm: null descriptor"); return; }
+    GemmArgs a = d->args;
+    a.M = d->M; a.N = d->N; a.K = d->K;
+    if (d->M < 1 || d->N < 1 || d->K < 1 || d->batch < 1 || d->batch > 65535) {
+        set_error(kBadArgument, "gemm: need M, N, K >= 1 and 1 <= batch <= 65535 (got %d %d %d, batch %d)", d->M, d->N, d->K, d->batch);
+        return;
+    }
+    const int ka = d->kind_a, kb = d->kind_b, ep = d->epilogue;
+    if (ka < kDense || ka > kQuant8 || kb < kDense || kb > kQuant8 || ep < kStore || ep > kNewton) {
+        set_error(kBadArgument, "gemm: unknown operand or epilogue kind (%d, %d, %d)", ka, kb, ep);
+        return;
+    }
+    if (!has_host_ptr(a.C) || a.ldc < d->N) { set_error(kBadArgument, "gemm: bad C (ldc %d < N %d or null)", a.ldc, d->N); return; }
+    if (ka < kQuant4) {
+        const int need = ka == kDense ? d->K : d->M;
+        if (!has_host_ptr(a.A) || a.lda < need) { set_error(kBadArgument, "gemm: bad A (lda %d < %d or null)", a.lda, need); return; }
+    } else {
+        if (!valid_quant(a.Aq, ka == kQuant4 ? 4 : 8, "A")) return;
+        if (a.Aq.order != d->M || d->K != d->M) { set_error(kBadArgument, "gemm: quantized A must be square with M == K == order"); return; }
+    }
+    if (kb < kQuant4) {
+        const int need = kb == kDense ? d->N : d->K;
+        if (!has_host_ptr(a.B) || a.ldb < need) { set_error(kBadArgument, "gemm: bad B (ldb %d < %d or null)", a.ldb, need); return; }
+    } else {
+        if (!valid_quant(a.Bq, kb == kQuant4 ? 4 : 8, "B")) return;
+        if (a.Bq.order != d->N || d->K != d->N) { set_error(kBadArgument, "gemm: quantized B must be square with K == N == order"); return; }
+    }
+    if (ep == kAxpbyDense && (!has_host_ptr(a.E) || a.lde < d->N)) { set_error(kBadArgument, "gemm: bad dense addend"); return; }
+    if (ep == kAxpbyQuant4 || ep == kAxpbyQuant8) {
+        if (!valid_quant(a.Eq, ep == kAxpbyQuant4 ? 4 : 8, "addend")) return;
+        if (a.Eq.order != d->M || d->M != d->N) { set_error(kBadArgument, "gemm: quantized addend must be M x N square of its order"); return; }
+    }
+    if (ep == kNewton && (!has_host_ptr(a.T) || a.ldt < d->N || !a.err)) { set_error(kBadArgument, "gemm: Newton epilogue needs T and err"); return; }
+    const bool need_code = ka >= kQuant4 || kb >= kQuant4 || ep == kAxpbyQuant4 || ep == kAxpbyQuant8;
+    if (need_code && !a.code) { set_error(kNullPointer, "gemm: code table missing"); return; }
+
+    // 128 x 128 tiles when that still gives every compute unit work, else 64 x 64 (quantized
+    // operands always use a 128-wide tile on their side).
+    const long long big_tiles = (long long)((d->M + 127) / 128) * ((d->N + 127) / 128) * d->batch;
+    const bool big = big_tiles >= compute_units();
+    const int combo = ka * 100 + kb * 10 + ep;
+#define QT_GEMM_CASE(KA, KB, EP)                                                                             \
+    case (KA) * 100 + (KB) * 10 + (EP):                                                                      \
+        if (big) launch_gemm<128, 128, KA, KB, EP>(a, d->batch, stream);                                     \
+        else if ((KA) >= kQuant4) launch_gemm<128, 64, KA, KB, EP>(a, d->batch, stream);                     \
+        else if ((KB) >= kQuant4) launch_gemm<64, 128, KA, KB, EP>(a, d->batch, stream);                     \
+        else launch_gemm<64, 64, KA, KB, EP>(a, d->batch, stream);                                           \
+        break;
+    switch (combo) {
+        QT_GEMM_CASE(kQuant4, kDense, kStore)
+        QT_GEMM_CASE(kQuant8, kDense, kStore)
+        QT_GEMM_CASE(kDense, kQuant4, kStore)
+        QT_GEMM_CASE(kDense, kQuant8, kStore)
+        QT_GEMM_CASE(kDense, kDenseT, kStore)
+        QT_GEMM_CASE(kDense, kDenseT, kAxpbyDense)
+        QT_GEMM_CASE(kDense, kDenseT, kAxpbyQuant4)
+        QT_GEMM_CASE(kDense, kDenseT, kAxpbyQuant8)
+        QT_GEMM_CASE(kDenseT, kDense, kStore)
+        QT_GEMM_CASE(kDenseT, kDense, kAxpbyDense)
+        QT_GEMM_CASE(kDenseT, kDense, kAxpbyQuant4)
+        QT_GEMM_CASE(kDenseT, kDense, kAxpbyQuant8)
+        QT_GEMM_CASE(kDense, kDense, kStore)
+        QT_GEMM_CASE(kDense, kDense, kAxpbyDense)
+        QT_GEMM_CASE(kDense, kDense, kNewton)
+        default:
+            set_error(kBadArgument, "gemm: combination A kind %d, B kind %d, epilogue %d is not built", ka, kb, ep);
+            return;
+    }
+#undef QT_GEMM_CASE
+    launch_ok("gemm");
+}

@@ -1,0 +1,201 @@
+"""Batched fp32 products on the MI355X matrix cores with the (de)quantization fused in.
+
+No counterpart module exists in the reference: there these steps are separate torch calls per
+matrix -- dequantize, then `@` (optimizers/shampoo2.py:255-268, shampoo1.py:164-178, 224-237)
+and the matmuls of optimizers/matrix_functions.py:127-140.  Every function here takes GPU
+tensors only and launches libqtensor_hip.so's qtensor_hip_gemm on torch's current stream.
+"""
+import ctypes as ct
+from typing import Optional, Sequence
+
+import torch
+from torch import Tensor
+
+import qtensor.functional as F
+
+DENSE, DENSE_T, QUANT4, QUANT8 = 0, 1, 2, 3
+EPI_STORE, EPI_AXPBY_DENSE, EPI_AXPBY_QUANT4, EPI_AXPBY_QUANT8, EPI_NEWTON = 0, 1, 2, 3, 4
+
+
+class BatchPtr(ct.Structure):
+    _fields_ = [("base", ct.c_void_p), ("list", ct.c_void_p), ("stride", ct.c_longlong)]
+
+
+class QuantRef(ct.Structure):
+    _fields_ = [("codes", BatchPtr), ("absmax", BatchPtr), ("diag", BatchPtr), ("order", ct.c_int),
+                ("bs_shift", ct.c_int)]
+
+
+class GemmArgs(ct.Structure):
+    _fields_ = [("M_", ct.c_int), ("N_", ct.c_int), ("K_", ct.c_int),
+                ("A", BatchPtr), ("lda", ct.c_int),
+                ("B", BatchPtr), ("ldb", ct.c_int),
+                ("Aq", QuantRef), ("Bq", QuantRef),
+                ("C", BatchPtr), ("ldc", ct.c_int),
+                ("alpha", ct.c_float), ("beta", ct.c_float),
+                ("E", BatchPtr), ("lde", ct.c_int),
+                ("Eq", QuantRef),
+                ("T", BatchPtr), ("ldt", ct.c_int),
+                ("newton_w", ct.c_float),
+                ("err", ct.c_void_p), ("skip", ct.c_void_p), ("code", ct.c_void_p)]
+
+
+class GemmDesc(ct.Structure):
+    _fields_ = [("M", ct.c_int), ("N", ct.c_int), ("K", ct.c_int), ("batch", ct.c_int),
+                ("kind_a", ct.c_int), ("kind_b", ct.c_int), ("epilogue", ct.c_int), ("args", GemmArgs)]
+
+
+if F.lib is not None:
+    F.lib.qtensor_hip_gemm.restype = None
+    F.lib.qtensor_hip_gemm.argtypes = [ct.POINTER(GemmDesc), ct.c_void_p]
+
+
+class Quantized:
+    """A batch of equally sized quantized square matrices held in stacked buffers.
+
+    codes [batch, order*order*bits/8] uint8, absmax [batch, order*order/blocksize] fp32,
+    diag [batch, order] fp32 or None, all contiguous on one GPU.  Entry b is exactly what
+    quantize_blockwise(_diagreal) writes for one matrix."""
+
+    def __init__(self, codes: Tensor, absmax: Tensor, diag: Optional[Tensor], order: int, blocksize: int,
+                 bits: int, code: Tensor):
+        if order % blocksize:
+            raise ValueError("fused kernels need blocksize to divide the order")
+        self.codes, self.absmax, self.diag = codes, absmax, diag
+        self.order, self.blocksize, self.bits, self.code = order, blocksize, bits, code
+        self.batch = codes.shape[0] if codes.dim() == 2 else 1
+
+    @classmethod
+    def from_holder(cls, h) -> "Quantized":
+        """View of one qtensor.utils holder (QTensor or QTensorDiagReal in low-bit mode)."""
+        return cls(h.var.view(1, -1), h.absmax.view(1, -1), None if getattr(h, "diag", None) is None else h.diag.view(1, -1),
+                   h.var_order, h.blocksize, h.bits, h.name2qmap[h.code])
+
+    def ref(self) -> QuantRef:
+        q = QuantRef()
+        q.codes = BatchPtr(self.codes.data_ptr(), None, self.codes.stride(0) if self.codes.dim() == 2 else 0)
+        q.absmax = BatchPtr(self.absmax.data_ptr(), None, self.absmax.stride(0) if self.absmax.dim() == 2 else 0)
+        if self.diag is not None:
+            q.diag = BatchPtr(self.diag.data_ptr(), None, self.diag.stride(0) if self.diag.dim() == 2 else 0)
+        q.order = self.order
+        q.bs_shift = self.blocksize.bit_length() - 1
+        return q
+
+    @property
+    def kind(self) -> int:
+        return QUANT4 if self.bits == 4 else QUANT8
+
+
+def _dense(t: Tensor):
+    """(BatchPtr, leading dimension, batch, rows, cols) of a [rows, cols] or [batch, rows, cols] fp32 tensor whose
+    last dimension is contiguous."""
+    if t.dtype != torch.float32 or not t.is_cuda:
+        raise ValueError("fused products take fp32 GPU tensors")
+    if t.dim() == 2:
+        t = t.unsqueeze(0)
+    if t.dim() != 3 or t.stride(2) != 1:
+        raise ValueError("expected [rows, cols] or [batch, rows, cols] with a contiguous last dimension")
+    return BatchPtr(t.data_ptr(), None, t.stride(0)), t.stride(1), t.shape[0], t.shape[1], t.shape[2]
+
+
+def _launch(desc: GemmDesc, device: torch.device) -> None:
+    if F.lib is None:
+        raise RuntimeError("libqtensor_hip.so is not available")
+    F._call(lambda d, s: F.lib.qtensor_hip_gemm(d, s), device, ct.byref(desc))
+
+
+def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, alpha=1.0, beta=0.0,
+         addend=None, newton=None, skip: Optional[Tensor] = None) -> Tensor:
+    """out[b] = epilogue(op(A[b]) @ op(B[b])).
+
+    A, B: fp32 tensors ([m,k] / [batch,m,k]; with trans_x the stored matrix is the transpose) or a
+    `Quantized` (square; then the other operand must be dense).
+    addend: None, a dense tensor E or a `Quantized` E: out = beta*E + alpha*product.
+    newton: None or (T_out, w, err): also writes T_out = (1-w) I + w*product and folds
+    max|product - I| into err[b] (fp32 [batch], zeroed by the caller).
+    skip: optional int32 [batch]; entries with a nonzero flag are not touched."""
+    d = GemmDesc()
+    a = d.args
+    dev = None
+    code = None
+    if isinstance(A, Quantized):
+        if trans_a:
+            raise ValueError("a quantized operand cannot be transposed")
+        d.kind_a, a.Aq, batch_a, m, k = A.kind, A.ref(), A.batch, A.order, A.order
+        dev, code = A.codes.device, A.code
+    else:
+        a.A, a.lda, batch_a, r, c = _dense(A)
+        m, k = (c, r) if trans_a else (r, c)
+        d.kind_a = DENSE_T if trans_a else DENSE
+        dev = A.device
+    if isinstance(B, Quantized):
+        if trans_b:
+            raise ValueError("a quantized operand cannot be transposed")
+        d.kind_b, a.Bq, batch_b, k2, n = B.kind, B.ref(), B.batch, B.order, B.order
+        code = B.code
+    else:
+        a.B, a.ldb, batch_b, r, c = _dense(B)
+        k2, n = (c, r) if trans_b else (r, c)
+        d.kind_b = DENSE_T if trans_b else DENSE
+    if k != k2:
+        raise ValueError(f"inner dimensions differ: {k} vs {k2}")
+    if batch_a != batch_b:
+        raise ValueError(f"batch sizes differ: {batch_a} vs {batch_b}")
+    batch = batch_a
+    if out is None:
+        out = torch.empty((batch, m, n), device=dev, dtype=torch.float32)
+        squeeze = (not isinstance(A, Quantized) and A.dim() == 2) or (not isinstance(B, Quantized) and B.dim() == 2)
+        if squeeze and batch == 1:
+            out = out[0]
+    a.C, a.ldc, batch_c, mc, nc = _dense(out)
+    if (batch_c, mc, nc) != (batch, m, n):
+        raise ValueError(f"out has shape {tuple(out.shape)}, expected batch {batch} x {m} x {n}")
+    d.M, d.N, d.K, d.batch = m, n, k, batch
+    d.epilogue = EPI_STORE
+    a.alpha, a.beta = alpha, beta
+    if addend is not None:
+        if isinstance(addend, Quantized):
+            if addend.batch != batch or addend.order != m or m != n:
+                raise ValueError("quantized addend must match the batch and be m x m")
+            a.Eq = addend.ref()
+            d.epilogue = EPI_AXPBY_QUANT4 if addend.bits == 4 else EPI_AXPBY_QUANT8
+            code = addend.code
+        else:
+            a.E, a.lde, be, me, ne = _dense(addend)
+            if (be, me, ne) != (batch, m, n):
+                raise ValueError("dense addend must have the shape of the result")
+            d.epilogue = EPI_AXPBY_DENSE
+    keep = [out]
+    if newton is not None:
+        if addend is not None:
+            raise ValueError("the Newton epilogue takes no addend")
+        t_out, w, err = newton
+        a.T, a.ldt, bt, mt, nt = _dense(t_out)
+        if (bt, mt, nt) != (batch, m, n) or err.numel() != batch or err.dtype != torch.float32:
+            raise ValueError("Newton outputs must match the result")
+        a.newton_w = w
+        a.err = err.data_ptr()
+        d.epilogue = EPI_NEWTON
+    if skip is not None:
+        if skip.dtype != torch.int32 or skip.numel() != batch:
+            raise ValueError("skip must be int32 [batch]")
+        a.skip = skip.data_ptr()
+    if code is not None:
+        a.code = code.data_ptr()
+    _launch(d, dev)
+    return out
+
+
+def precondition(G: Tensor, left, right, out: Optional[Tensor] = None) -> Tensor:
+    """deq(left) @ G @ deq(right) with both factors expanded inside the products.
+    left / right: `Quantized` or dense fp32 matrices."""
+    tmp = gemm(left, G)
+    return gemm(tmp, right, out=out)
+
+
+def gram(G: Tensor, axis: int, *, stat=None, beta=0.0, alpha=1.0, out: Optional[Tensor] = None) -> Tensor:
+    """axis 0: G @ G.T, axis 1: G.T @ G; with `stat` (dense or `Quantized`) returns
+    beta * stat + alpha * that product, i.e. the Shampoo statistics update in one launch."""
+    if axis == 0:
+        return gemm(G, G, trans_b=True, addend=stat, alpha=alpha, beta=beta, out=out)
+    return gemm(G, G, trans_a=True, addend=stat, alpha=alpha, beta=beta, out=out)

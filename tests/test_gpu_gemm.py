@@ -1,0 +1,171 @@
+"""GPU parity of the fused matrix-core products (qtensor.fused.gemm -> qtensor_hip_gemm).
+
+Reference for every case: dequantize with the CPU oracle, multiply in float64 on the CPU.
+Tolerance: relative Frobenius error <= 1e-5 (fp32 products accumulate in fp32 on the matrix
+cores; observed errors are around 1e-7)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import quant_np as Q
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def mods():
+    import qtensor.functional as F
+    import qtensor.fused as X
+    assert torch.cuda.is_available() and F.lib is not None
+    return F, X
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    want = want.double()
+    return float((got.detach().cpu().double() - want).norm() / want.norm().clamp_min(1e-300))
+
+
+def make_quantized(F, X, mats: torch.Tensor, code: np.ndarray, bits, bs, diag):
+    """Quantize a [batch, n, n] stack on the GPU into stacked buffers; also returns the oracle's
+    dequantized float64 copy of the same codes."""
+    batch, n, _ = mats.shape
+    code_d = torch.from_numpy(code).cuda()
+    codes = torch.empty(batch, n * n * bits // 8, dtype=torch.uint8, device="cuda")
+    absmax = torch.empty(batch, n * n // bs, dtype=torch.float32, device="cuda")
+    dg = torch.empty(batch, n, dtype=torch.float32, device="cuda") if diag else None
+    deq = []
+    for b in range(batch):
+        m = mats[b].contiguous().cuda()
+        if diag:
+            F.quantize_blockwise_diagreal(m, code_d, n, absmax=absmax[b], diag=dg[b], out=codes[b], blocksize=bs, bits=bits)
+        else:
+            F.quantize_blockwise(m, code_d, n, absmax=absmax[b], out=codes[b], blocksize=bs, bits=bits)
+        o = Q.quantize_c(mats[b].numpy(), code, n, bs, bits, diag)
+        assert np.array_equal(codes[b].cpu().numpy(), o[0])
+        deq.append(Q.dequantize_c(o[0], code, n, o[1], bs, bits, diag=o[2] if diag else None))
+    q = X.Quantized(codes, absmax, dg, n, bs, bits, code_d)
+    return q, torch.from_numpy(np.stack(deq)).double()
+
+
+@pytest.mark.parametrize("m,n,k,batch", [(128, 128, 128, 1), (64, 64, 16, 3), (100, 65, 33, 2), (257, 129, 70, 1),
+                                         (768, 3072, 768, 1), (1024, 1024, 1024, 2), (1, 1, 1, 1), (300, 5, 1000, 1)])
+def test_dense_products_all_layouts(mods, m, n, k, batch):
+    _, X = mods
+    g = torch.Generator().manual_seed(m * 7 + n)
+    A = torch.randn(batch, m, k, generator=g)
+    B = torch.randn(batch, k, n, generator=g)
+    want = A.double() @ B.double()
+    Ad, Bd = A.cuda(), B.cuda()
+    assert rel_err(X.gemm(Ad, Bd), want) <= TOL
+    assert rel_err(X.gemm(Ad.transpose(1, 2).contiguous(), Bd, trans_a=True), want) <= TOL
+    assert rel_err(X.gemm(Ad, Bd.transpose(1, 2).contiguous(), trans_b=True), want) <= TOL
+    # views with a larger leading dimension and an unaligned start
+    big = torch.zeros(batch, m + 3, k + 5, device="cuda")
+    big[:, 1:m + 1, 1:k + 1] = Ad
+    assert rel_err(X.gemm(big[:, 1:m + 1, 1:k + 1], Bd), want) <= TOL
+    if batch == 1:
+        out2 = X.gemm(Ad[0], Bd[0])
+        assert out2.shape == (m, n) and rel_err(out2, want[0]) <= TOL
+
+
+@pytest.mark.parametrize("bits,bs,name", [(4, 64, "linear-2"), (8, 256, "dynamic"), (8, 64, "linear-2"), (4, 128, "dynamic")])
+@pytest.mark.parametrize("diag", [False, True])
+def test_quantized_factor_times_dense(mods, code_maps, bits, bs, name, diag):
+    F, X = mods
+    g = torch.Generator().manual_seed(bits + bs)
+    for n, other, batch in ((256, 100, 2), (768, 320, 1), (1024, 64, 1)):
+        if n % bs:
+            continue
+        mats = torch.randn(batch, n, n, generator=g)
+        mats[:, 3, :64] = 0.0                                  # a zero-maximum segment
+        q, deq = make_quantized(F, X, mats, code_maps[(name, bits)], bits, bs, diag)
+        G_left = torch.randn(batch, n, other, generator=g)
+        G_right = torch.randn(batch, other, n, generator=g)
+        assert rel_err(X.gemm(q, G_left.cuda()), deq @ G_left.double()) <= TOL
+        assert rel_err(X.gemm(G_right.cuda(), q), G_right.double() @ deq) <= TOL
+
+
+def test_config3_preconditioned_gradient(mods, code_maps):
+    """G 768 x 3072 ~ N(0, 0.02^2); L (768) and R (3072) are inverse 4th roots of seeded PSD matrices with
+    eigenvalues log-uniform in [1e-6, 1], stored 4-bit / block 64 with exact diagonal."""
+    F, X = mods
+    code = code_maps[("linear-2", 4)]
+    g = torch.Generator().manual_seed(3)
+
+    def inv_root(n):
+        qm, _ = torch.linalg.qr(torch.randn(n, n, generator=g, dtype=torch.float64))
+        lam = 10.0 ** (-6 * torch.rand(n, generator=g, dtype=torch.float64))
+        return ((qm * lam ** -0.25) @ qm.T).float()
+
+    L, R = inv_root(768), inv_root(3072)
+    G = 0.02 * torch.randn(768, 3072, generator=g)
+    for diag in (True, False):
+        Lq, Ld = make_quantized(F, X, L[None], code, 4, 64, diag)
+        Rq, Rd = make_quantized(F, X, R[None], code, 4, 64, diag)
+        want = Ld[0] @ G.double() @ Rd[0]
+        got = X.precondition(G.cuda(), Lq, Rq)
+        assert got.shape == (768, 3072)
+        assert rel_err(got, want) <= TOL
+        # and equal, to the same tolerance, to dequantize-then-matmul on the device
+        Lg = F.dequantize_blockwise_diagreal(Lq.codes[0], Lq.code, 768, Lq.absmax[0], Lq.diag[0], blocksize=64, bits=4) if diag \
+            else F.dequantize_blockwise(Lq.codes[0], Lq.code, 768, Lq.absmax[0], blocksize=64, bits=4)
+        assert torch.equal(Lg.cpu().double(), Ld[0])
+        Rg = torch.from_numpy(Rd[0].numpy().astype(np.float32)).cuda()
+        assert rel_err(got, (Lg @ G.cuda() @ Rg).cpu()) <= TOL
+
+
+@pytest.mark.parametrize("m,n", [(256, 512), (768, 1024), (100, 260), (1024, 768)])
+def test_gram_and_statistics_update(mods, code_maps, m, n):
+    F, X = mods
+    g = torch.Generator().manual_seed(m + n)
+    G = 0.02 * torch.randn(2, m, n, generator=g)
+    Gd = G.cuda()
+    assert rel_err(X.gram(Gd, 0), G.double() @ G.double().transpose(1, 2)) <= TOL
+    assert rel_err(X.gram(Gd, 1), G.double().transpose(1, 2) @ G.double()) <= TOL
+    beta = 0.95
+    for axis, order in ((0, m), (1, n)):
+        S = (G.double() @ G.double().transpose(1, 2)) if axis == 0 else (G.double().transpose(1, 2) @ G.double())
+        old = torch.randn(2, order, order, generator=g) * 1e-3
+        old = old @ old.transpose(1, 2) + 1e-6 * torch.eye(order)
+        assert rel_err(X.gram(Gd, axis, stat=old.cuda(), beta=beta, alpha=1 - beta), beta * old.double() + (1 - beta) * S) <= TOL
+        if order % 64 == 0:
+            q, deq = make_quantized(F, X, old, code_maps[("linear-2", 4)], 4, 64, True)
+            assert rel_err(X.gram(Gd, axis, stat=q, beta=beta, alpha=1 - beta), beta * deq + (1 - beta) * S) <= TOL
+
+
+def test_newton_epilogue_and_skip_flags(mods):
+    _, X = mods
+    g = torch.Generator().manual_seed(9)
+    n, batch = 192, 3
+    A = torch.randn(batch, n, n, generator=g) / n ** 0.5
+    B = torch.randn(batch, n, n, generator=g) / n ** 0.5
+    want = A.double() @ B.double()
+    w = -0.25
+    out = torch.full((batch, n, n), 7.0, device="cuda")
+    T = torch.full((batch, n, n), 7.0, device="cuda")
+    err = torch.zeros(batch, device="cuda")
+    skip = torch.tensor([0, 1, 0], dtype=torch.int32, device="cuda")
+    X.gemm(A.cuda(), B.cuda(), out=out, newton=(T, w, err), skip=skip)
+    eye = torch.eye(n, dtype=torch.float64)
+    for b in (0, 2):
+        assert rel_err(out[b], want[b]) <= TOL
+        assert rel_err(T[b], (1 - w) * eye + w * want[b]) <= TOL
+        assert abs(float(err[b]) - float((want[b] - eye).abs().max())) <= 1e-5
+    assert bool((out[1] == 7.0).all()) and bool((T[1] == 7.0).all()) and float(err[1]) == 0.0
+
+
+def test_argument_errors(mods, code_maps):
+    F, X = mods
+    A = torch.randn(64, 32, device="cuda")
+    with pytest.raises(ValueError):
+        X.gemm(A, torch.randn(31, 8, device="cuda"))
+    with pytest.raises(ValueError):
+        X.gemm(A.double(), A.double().T)
+    with pytest.raises(ValueError):
+        X.gemm(A.cpu(), A.cpu().T.contiguous())
+    q, _ = make_quantized(F, X, torch.randn(1, 128, 128), code_maps[("linear-2", 4)], 4, 64, True)
+    with pytest.raises(RuntimeError):                           # two quantized factors: not built
+        X.gemm(q, q)
+    with pytest.raises(ValueError):
+        X.gemm(q, torch.randn(64, 8, device="cuda"))
