@@ -88,6 +88,17 @@ void cdequantize_blockwise_diagreal_8bit_bf16_stream(unsigned char *A, float *co
 void cdequantize_blockwise_diagreal_4bit_fp32_stream(unsigned char *A, float *code, int order, float *absmax, float *diag, float *out, int blocksize, qtensor_stream_t stream);
 void cdequantize_blockwise_diagreal_4bit_bf16_stream(unsigned char *A, float *code, int order, float *absmax, float *diag, qtensor_bf16 *out, int blocksize, qtensor_stream_t stream);
 
+/* ---- stacks of equally sized matrices in one launch (no counterpart in the reference, which
+ * loops over matrices in Python: optimizers/shampoo2.py:184-200, 249-269) --------------------
+ * A is batch x order x order, contiguous; absmax, diag and out are the per-matrix buffers of
+ * the single-matrix entry points laid end to end.  Needs blocksize to divide order, 16-byte
+ * aligned A/out and batch*order*order < 2^31.  diag == NULL selects the plain form. */
+void qtensor_hip_quantize_batched(const void *A, int a_is_bf16, const float *code, int bits, int order, int batch,
+                                  float *absmax, float *diag, unsigned char *out, int blocksize, qtensor_stream_t stream);
+void qtensor_hip_dequantize_batched(const unsigned char *q, const float *code, int bits, int order, int batch,
+                                    const float *absmax, const float *diag, void *out, int out_is_bf16, int blocksize,
+                                    qtensor_stream_t stream);
+
 /* ---- self check and calibration (no counterpart in the reference) ------------------------
  * The flat-path quantizer replaces IEEE division by the segment maximum a with r = rcp(a) refined
  * by one Newton step and q = fma(fma(-x*r, a, x), r, x*r).  This entry point compares both

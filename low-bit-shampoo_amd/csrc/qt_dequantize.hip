@@ -53,7 +53,7 @@ template <> struct Vec4Store<uint16_t> {
 template <typename T, int BITS, bool DIAG, bool STREAM>
 __global__ __launch_bounds__(kFlatThreads) void dequantize_flat_kernel(
     const uint8_t *__restrict__ q, const float *__restrict__ code, uint32_t n_super, uint32_t bs_shift,
-    FastDiv row_div, const float *__restrict__ absmax, const float *__restrict__ diag, T *__restrict__ out) {
+    FastDiv row_div, FastDiv order_div, const float *__restrict__ absmax, const float *__restrict__ diag, T *__restrict__ out) {
     constexpr int NCODE = 1 << BITS;
     constexpr int kWaves = kFlatThreads / 64;
     constexpr int CODE_VECS = BITS == 4 ? 1 : 2;            // uint4 loads per lane per step
@@ -100,10 +100,11 @@ __global__ __launch_bounds__(kFlatThreads) void dequantize_flat_kernel(
         wave_lds_sync();
 
         const uint32_t k4_0 = st * (uint32_t)(kSuper / 4) + lane;   // index of this lane's first 4-vector
-        uint32_t row = 0, col4 = 0;
+        uint32_t row = 0, col4 = 0, lrow = 0;                        // row of the stack, and inside its matrix
         if (DIAG) {
             row = fastdiv(k4_0, row_div);
             col4 = k4_0 - row * row_div.divisor;
+            lrow = row - fastdiv(row, order_div) * order_div.divisor;
         }
 #pragma unroll
         for (uint32_t j = 0; j < 8; ++j) {
@@ -124,13 +125,17 @@ __global__ __launch_bounds__(kFlatThreads) void dequantize_flat_kernel(
                 y = make_float4(s_code[id0] * scale, s_code[id1] * scale, s_code[id2] * scale, s_code[id3] * scale);
             }
             if (DIAG) {
-                if ((row >> 2) == col4) {
+                if ((lrow >> 2) == col4) {
                     const float d = diag[row];
-                    const uint32_t e = row & 3u;
+                    const uint32_t e = lrow & 3u;
                     if (e == 0) y.x = d; else if (e == 1) y.y = d; else if (e == 2) y.z = d; else y.w = d;
                 }
                 col4 += 64u;
-                while (col4 >= row_div.divisor) { col4 -= row_div.divisor; ++row; }
+                while (col4 >= row_div.divisor) {
+                    col4 -= row_div.divisor;
+                    ++row;
+                    if (++lrow == order_div.divisor) lrow = 0;
+                }
             }
             Vec4Store<T>::template store<STREAM>(out, (k4_0 + j * 64u) << 2, y);
         }
@@ -171,7 +176,7 @@ int capped_grid(uint32_t blocks_needed, int blocks_per_cu) {
 
 template <typename T, int BITS, bool DIAG>
 void dequantize_dispatch(const uint8_t *q, const float *code, int order_i, const float *absmax, const float *diag,
-                         T *out, int blocksize, hipStream_t stream) {
+                         T *out, int blocksize, hipStream_t stream, int batch = 1) {
     clear_error();
     int bs_shift = 0;
     switch (blocksize) {
@@ -185,8 +190,9 @@ void dequantize_dispatch(const uint8_t *q, const float *code, int order_i, const
             set_error(kBadBlocksize, "dequantize_blockwise: blocksize %d is not one of 64,128,256,512,1024,2048", blocksize);
             return;
     }
-    if (order_i < 1 || (int64_t)order_i * order_i >= (int64_t(1) << 31)) {
-        set_error(kBadOrder, "dequantize_blockwise: order %d out of range (need 1 <= order and order*order < 2^31)", order_i);
+    if (order_i < 1 || batch < 1 || (int64_t)order_i * order_i * batch >= (int64_t(1) << 31)) {
+        set_error(kBadOrder, "dequantize_blockwise: order %d (batch %d) out of range (need order >= 1 and batch*order*order < 2^31)",
+                  order_i, batch);
         return;
     }
     if (!q || !code || !absmax || !out || (DIAG && !diag)) {
@@ -194,8 +200,12 @@ void dequantize_dispatch(const uint8_t *q, const float *code, int order_i, const
         return;
     }
     const uint32_t order = (uint32_t)order_i, bs = (uint32_t)blocksize;
-    const uint32_t total = order * order;
+    const uint32_t total = order * order * (uint32_t)batch;
     const bool flat = order % bs == 0 && is_aligned(out, 4 * sizeof(T)) && is_aligned(q, 16) && is_aligned(absmax, 4);
+    if (batch > 1 && !flat) {
+        set_error(kBadArgument, "dequantize_blockwise: a stack of matrices needs blocksize to divide the order and aligned buffers");
+        return;
+    }
     if (flat) {
         constexpr uint32_t kWaves = kFlatThreads / 64;
         const uint32_t n_super = total / kSuper;
@@ -204,10 +214,10 @@ void dequantize_dispatch(const uint8_t *q, const float *code, int order_i, const
         // Outputs far beyond the 256 MB last-level cache are written with the streaming hint.
         if (total >= (1u << 25)) {
             hipLaunchKernelGGL((dequantize_flat_kernel<T, BITS, DIAG, true>), grid, dim3(kFlatThreads), 0, stream,
-                               q, code, n_super, (uint32_t)bs_shift, make_fastdiv(order / 4), absmax, diag, out);
+                               q, code, n_super, (uint32_t)bs_shift, make_fastdiv(order / 4), make_fastdiv(order), absmax, diag, out);
         } else {
             hipLaunchKernelGGL((dequantize_flat_kernel<T, BITS, DIAG, false>), grid, dim3(kFlatThreads), 0, stream,
-                               q, code, n_super, (uint32_t)bs_shift, make_fastdiv(order / 4), absmax, diag, out);
+                               q, code, n_super, (uint32_t)bs_shift, make_fastdiv(order / 4), make_fastdiv(order), absmax, diag, out);
         }
     } else {
         const uint32_t nb = (order + bs - 1) / bs;
@@ -244,3 +254,17 @@ QT_DEFINE_DEQUANT(8bit_fp32, float, 8)
 QT_DEFINE_DEQUANT(8bit_bf16, uint16_t, 8)
 QT_DEFINE_DEQUANT(4bit_fp32, float, 4)
 QT_DEFINE_DEQUANT(4bit_bf16, uint16_t, 4)
+
+extern "C" void qtensor_hip_dequantize_batched(const unsigned char *q, const float *code, int bits, int order, int batch,
+                                               const float *absmax, const float *diag, void *out, int out_is_bf16,
+                                               int blocksize, void *stream) {
+    using namespace qt;
+    hipStream_t st = (hipStream_t)stream;
+    if (bits != 4 && bits != 8) { clear_error(); set_error(kBadArgument, "dequantize_batched: bits must be 4 or 8"); return; }
+#define QT_DB(T, BITS)                                                                                           \
+    (diag ? dequantize_dispatch<T, BITS, true>(q, code, order, absmax, diag, (T *)out, blocksize, st, batch)       \
+          : dequantize_dispatch<T, BITS, false>(q, code, order, absmax, nullptr, (T *)out, blocksize, st, batch))
+    if (out_is_bf16) { if (bits == 4) QT_DB(uint16_t, 4); else QT_DB(uint16_t, 8); }
+    else { if (bits == 4) QT_DB(float, 4); else QT_DB(float, 8); }
+#undef QT_DB
+}

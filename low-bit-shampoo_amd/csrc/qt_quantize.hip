@@ -103,6 +103,7 @@ struct FlatQuantizer {
     const uint2 *lut;
     WaveStage<BITS> &stage;
     FastDiv row_div;                                        // by order/4
+    FastDiv order_div;                                      // by order (rows of a stack -> row inside its matrix)
     bool fast_ok, ascending;
     uint32_t lane;
 
@@ -119,18 +120,23 @@ struct FlatQuantizer {
     __device__ __forceinline__ void process(Step &s, uint32_t step) const {
         if (DIAG) {
             const uint32_t k4 = step * (uint32_t)(kStep / 4) + lane;
-            uint32_t row = fastdiv(k4, row_div);
+            uint32_t row = fastdiv(k4, row_div);            // row of the stack of matrices
             uint32_t col4 = k4 - row * row_div.divisor;
+            uint32_t lrow = row - fastdiv(row, order_div) * order_div.divisor;   // row inside its matrix
 #pragma unroll
             for (int j = 0; j < J; ++j) {
-                if ((row >> 2) == col4) {                   // this vector holds element (row, row)
-                    const uint32_t e = row & 3u;
+                if ((lrow >> 2) == col4) {                  // this vector holds a diagonal element
+                    const uint32_t e = lrow & 3u;
                     float4 &v = s.v[j];
                     diag[row] = e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w;
                     if (e == 0) v.x = 0.0f; else if (e == 1) v.y = 0.0f; else if (e == 2) v.z = 0.0f; else v.w = 0.0f;
                 }
                 col4 += 64u;
-                while (col4 >= row_div.divisor) { col4 -= row_div.divisor; ++row; }
+                while (col4 >= row_div.divisor) {
+                    col4 -= row_div.divisor;
+                    ++row;
+                    if (++lrow == order_div.divisor) lrow = 0;
+                }
             }
         }
 
@@ -198,7 +204,7 @@ struct FlatQuantizer {
 
 template <typename T, int BITS, int BS, bool DIAG, bool USE_LUT, bool STREAM>
 __global__ __launch_bounds__(kFlatThreads) void quantize_flat_kernel(
-    const T *__restrict__ A, const float *__restrict__ code, uint32_t n_steps, FastDiv row_div,
+    const T *__restrict__ A, const float *__restrict__ code, uint32_t n_steps, FastDiv row_div, FastDiv order_div,
     float *__restrict__ absmax, float *__restrict__ diag, uint8_t *__restrict__ out) {
     using Q = FlatQuantizer<T, BITS, BS, DIAG, USE_LUT, STREAM>;
     constexpr int NCODE = Q::NCODE;
@@ -212,7 +218,7 @@ __global__ __launch_bounds__(kFlatThreads) void quantize_flat_kernel(
     const int flags = tab.flags;
 
     const uint32_t w = threadIdx.x >> 6;
-    const Q q{A, absmax, diag, out, tab, lut, stages[w], row_div, (flags & kFlagLut) != 0,
+    const Q q{A, absmax, diag, out, tab, lut, stages[w], row_div, order_div, (flags & kFlagLut) != 0,
               (flags & kFlagAscending) != 0, threadIdx.x & 63u};
     const uint32_t n_waves = gridDim.x * kWaves;
     uint32_t step = blockIdx.x * kWaves + w;
@@ -294,11 +300,11 @@ int grid_for(uint32_t work_items_per_block_unit, int blocks_per_cu) {
 }
 
 template <typename T, int BITS, int BS, bool DIAG>
-void launch_flat(const T *A, const float *code, uint32_t order, float *absmax, float *diag, uint8_t *out, hipStream_t stream) {
+void launch_flat(const T *A, const float *code, uint32_t order, uint32_t batch, float *absmax, float *diag, uint8_t *out, hipStream_t stream) {
     constexpr uint32_t kWaves = kFlatThreads / 64;
-    const uint32_t total = order * order;
+    const uint32_t total = order * order * batch;
     const uint32_t n_steps = total / kStep;
-    const FastDiv rd = make_fastdiv(order / 4);
+    const FastDiv rd = make_fastdiv(order / 4), od = make_fastdiv(order);
     const uint32_t blocks_needed = (n_steps + kWaves - 1) / kWaves;
     const int grid = grid_for(blocks_needed, kFlatBlocksPerCU);
     // The bucket table costs a few microseconds of set-up per workgroup; it pays from about
@@ -306,13 +312,13 @@ void launch_flat(const T *A, const float *code, uint32_t order, float *absmax, f
     // streaming hint.
     if (total >= (1u << 25)) {
         hipLaunchKernelGGL((quantize_flat_kernel<T, BITS, BS, DIAG, true, true>), dim3(grid), dim3(kFlatThreads), 0, stream,
-                           A, code, n_steps, rd, absmax, diag, out);
+                           A, code, n_steps, rd, od, absmax, diag, out);
     } else if (total >= (1u << 20)) {
         hipLaunchKernelGGL((quantize_flat_kernel<T, BITS, BS, DIAG, true, false>), dim3(grid), dim3(kFlatThreads), 0, stream,
-                           A, code, n_steps, rd, absmax, diag, out);
+                           A, code, n_steps, rd, od, absmax, diag, out);
     } else {
         hipLaunchKernelGGL((quantize_flat_kernel<T, BITS, BS, DIAG, false, false>), dim3(grid), dim3(kFlatThreads), 0, stream,
-                           A, code, n_steps, rd, absmax, diag, out);
+                           A, code, n_steps, rd, od, absmax, diag, out);
     }
 }
 
@@ -330,14 +336,16 @@ void launch_general(const T *A, const float *code, uint32_t order, uint32_t bs, 
 }
 
 template <typename T, int BITS, bool DIAG>
-void quantize_dispatch(const T *A, const float *code, int order_i, float *absmax, float *diag, uint8_t *out, int blocksize, hipStream_t stream) {
+void quantize_dispatch(const T *A, const float *code, int order_i, float *absmax, float *diag, uint8_t *out, int blocksize, hipStream_t stream,
+                       int batch = 1) {
     clear_error();
     if (!(blocksize == 64 || blocksize == 128 || blocksize == 256 || blocksize == 512 || blocksize == 1024 || blocksize == 2048)) {
         set_error(kBadBlocksize, "quantize_blockwise: blocksize %d is not one of 64,128,256,512,1024,2048", blocksize);
         return;
     }
-    if (order_i < 1 || (int64_t)order_i * order_i >= (int64_t(1) << 31)) {
-        set_error(kBadOrder, "quantize_blockwise: order %d out of range (need 1 <= order and order*order < 2^31)", order_i);
+    if (order_i < 1 || batch < 1 || (int64_t)order_i * order_i * batch >= (int64_t(1) << 31)) {
+        set_error(kBadOrder, "quantize_blockwise: order %d (batch %d) out of range (need order >= 1 and batch*order*order < 2^31)",
+                  order_i, batch);
         return;
     }
     if (!A || !code || !absmax || !out || (DIAG && !diag)) {
@@ -346,14 +354,18 @@ void quantize_dispatch(const T *A, const float *code, int order_i, float *absmax
     }
     const uint32_t order = (uint32_t)order_i, bs = (uint32_t)blocksize;
     const bool flat = order % bs == 0 && is_aligned(A, 4 * sizeof(T)) && is_aligned(out, 16) && is_aligned(absmax, 4);
+    if (batch > 1 && !flat) {
+        set_error(kBadArgument, "quantize_blockwise: a stack of matrices needs blocksize to divide the order and aligned buffers");
+        return;
+    }
     if (flat) {
         switch (blocksize) {
-            case 64: launch_flat<T, BITS, 64, DIAG>(A, code, order, absmax, diag, out, stream); break;
-            case 128: launch_flat<T, BITS, 128, DIAG>(A, code, order, absmax, diag, out, stream); break;
-            case 256: launch_flat<T, BITS, 256, DIAG>(A, code, order, absmax, diag, out, stream); break;
-            case 512: launch_flat<T, BITS, 512, DIAG>(A, code, order, absmax, diag, out, stream); break;
-            case 1024: launch_flat<T, BITS, 1024, DIAG>(A, code, order, absmax, diag, out, stream); break;
-            default: launch_flat<T, BITS, 2048, DIAG>(A, code, order, absmax, diag, out, stream); break;
+            case 64: launch_flat<T, BITS, 64, DIAG>(A, code, order, (uint32_t)batch, absmax, diag, out, stream); break;
+            case 128: launch_flat<T, BITS, 128, DIAG>(A, code, order, (uint32_t)batch, absmax, diag, out, stream); break;
+            case 256: launch_flat<T, BITS, 256, DIAG>(A, code, order, (uint32_t)batch, absmax, diag, out, stream); break;
+            case 512: launch_flat<T, BITS, 512, DIAG>(A, code, order, (uint32_t)batch, absmax, diag, out, stream); break;
+            case 1024: launch_flat<T, BITS, 1024, DIAG>(A, code, order, (uint32_t)batch, absmax, diag, out, stream); break;
+            default: launch_flat<T, BITS, 2048, DIAG>(A, code, order, (uint32_t)batch, absmax, diag, out, stream); break;
         }
     } else {
         launch_general<T, BITS, DIAG>(A, code, order, bs, absmax, diag, out, stream);
@@ -387,3 +399,18 @@ QT_DEFINE_QUANT(8bit_fp32, float, 8)
 QT_DEFINE_QUANT(8bit_bf16, uint16_t, 8)
 QT_DEFINE_QUANT(4bit_fp32, float, 4)
 QT_DEFINE_QUANT(4bit_bf16, uint16_t, 4)
+
+extern "C" void qtensor_hip_quantize_batched(const void *A, int a_is_bf16, const float *code, int bits, int order, int batch,
+                                             float *absmax, float *diag, unsigned char *out, int blocksize, void *stream) {
+    using namespace qt;
+    hipStream_t st = (hipStream_t)stream;
+    float *c = const_cast<float *>(code);
+    (void)c;
+    if (bits != 4 && bits != 8) { clear_error(); set_error(kBadArgument, "quantize_batched: bits must be 4 or 8"); return; }
+#define QT_QB(T, BITS)                                                                                        \
+    (diag ? quantize_dispatch<T, BITS, true>((const T *)A, code, order, absmax, diag, out, blocksize, st, batch)    \
+          : quantize_dispatch<T, BITS, false>((const T *)A, code, order, absmax, nullptr, out, blocksize, st, batch))
+    if (a_is_bf16) { if (bits == 4) QT_QB(uint16_t, 4); else QT_QB(uint16_t, 8); }
+    else { if (bits == 4) QT_QB(float, 4); else QT_QB(float, 8); }
+#undef QT_QB
+}

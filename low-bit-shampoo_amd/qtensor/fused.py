@@ -86,9 +86,26 @@ class Quantized:
         return QUANT4 if self.bits == 4 else QUANT8
 
 
-def _dense(t: Tensor):
+class PtrList:
+    """A batch of dense fp32 matrices given by a device array of addresses (int64 [batch]), all of
+    shape rows x cols with leading dimension ld (default cols).  Lets a caller choose per batch
+    entry, on the device, which buffer an operand comes from or a result goes to."""
+
+    def __init__(self, ptrs: Tensor, shape, ld: Optional[int] = None):
+        if ptrs.dtype != torch.int64 or not ptrs.is_cuda or ptrs.dim() != 1 or ptrs.numel() != shape[0]:
+            raise ValueError("PtrList needs an int64 GPU vector with one address per batch entry")
+        self.ptrs, self.shape, self.ld = ptrs.contiguous(), tuple(shape), (shape[2] if ld is None else ld)
+        self.device = ptrs.device
+
+    def dim(self):
+        return 3
+
+
+def _dense(t):
     """(BatchPtr, leading dimension, batch, rows, cols) of a [rows, cols] or [batch, rows, cols] fp32 tensor whose
-    last dimension is contiguous."""
+    last dimension is contiguous, or of a PtrList."""
+    if isinstance(t, PtrList):
+        return BatchPtr(None, t.ptrs.data_ptr(), 0), t.ld, t.shape[0], t.shape[1], t.shape[2]
     if t.dtype != torch.float32 or not t.is_cuda:
         raise ValueError("fused products take fp32 GPU tensors")
     if t.dim() == 2:
@@ -199,3 +216,52 @@ def gram(G: Tensor, axis: int, *, stat=None, beta=0.0, alpha=1.0, out: Optional[
     if axis == 0:
         return gemm(G, G, trans_b=True, addend=stat, alpha=alpha, beta=beta, out=out)
     return gemm(G, G, trans_a=True, addend=stat, alpha=alpha, beta=beta, out=out)
+
+
+# --------------------------------------------------------------------------- stacks of matrices
+if F.lib is not None:
+    F.lib.qtensor_hip_quantize_batched.restype = None
+    F.lib.qtensor_hip_quantize_batched.argtypes = [ct.c_void_p, ct.c_int, ct.c_void_p, ct.c_int, ct.c_int, ct.c_int,
+                                                   ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_void_p]
+    F.lib.qtensor_hip_dequantize_batched.restype = None
+    F.lib.qtensor_hip_dequantize_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_int, ct.c_void_p,
+                                                     ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
+
+
+def empty_quantized(batch: int, order: int, blocksize: int, bits: int, code: Tensor, diagreal: bool) -> Quantized:
+    """Uninitialised stacked buffers for `batch` matrices of the given order."""
+    dev = code.device
+    codes = torch.empty(batch, order * order * bits // 8, dtype=torch.uint8, device=dev)
+    absmax = torch.empty(batch, order * order // blocksize, dtype=torch.float32, device=dev)
+    diag = torch.empty(batch, order, dtype=torch.float32, device=dev) if diagreal else None
+    return Quantized(codes, absmax, diag, order, blocksize, bits, code)
+
+
+def quantize_stack(mats: Tensor, q: Quantized) -> Quantized:
+    """Quantize the contiguous stack mats [batch, order, order] (fp32 or bf16) into q's buffers in one
+    launch; entry b equals quantize_blockwise(_diagreal)(mats[b])."""
+    if F.lib is None:
+        raise RuntimeError("libqtensor_hip.so is not available")
+    if not mats.is_cuda or not mats.is_contiguous() or mats.shape != (q.batch, q.order, q.order):
+        raise ValueError(f"expected a contiguous GPU stack of shape {(q.batch, q.order, q.order)}")
+    slot = F._dtype_slot(mats.dtype, "mats")
+    for t in (q.codes, q.absmax) + ((q.diag,) if q.diag is not None else ()):
+        if not t.is_contiguous():
+            raise ValueError("stacked quantized buffers must be contiguous")
+    F._call(F.lib.qtensor_hip_quantize_batched, mats.device, mats.data_ptr(), slot, q.code.data_ptr(), q.bits, q.order,
+            q.batch, q.absmax.data_ptr(), None if q.diag is None else q.diag.data_ptr(), q.codes.data_ptr(), q.blocksize)
+    return q
+
+
+def dequantize_stack(q: Quantized, out: Optional[Tensor] = None, outdtype=torch.float32) -> Tensor:
+    """[batch, order, order] stack of dequantized matrices in one launch."""
+    if F.lib is None:
+        raise RuntimeError("libqtensor_hip.so is not available")
+    if out is None:
+        out = torch.empty(q.batch, q.order, q.order, dtype=outdtype, device=q.codes.device)
+    if not out.is_contiguous() or out.shape != (q.batch, q.order, q.order):
+        raise ValueError(f"out must be a contiguous stack of shape {(q.batch, q.order, q.order)}")
+    slot = F._dtype_slot(out.dtype, "out")
+    F._call(F.lib.qtensor_hip_dequantize_batched, out.device, q.codes.data_ptr(), q.code.data_ptr(), q.bits, q.order,
+            q.batch, q.absmax.data_ptr(), None if q.diag is None else q.diag.data_ptr(), out.data_ptr(), slot, q.blocksize)
+    return out

@@ -169,3 +169,31 @@ def test_argument_errors(mods, code_maps):
         X.gemm(q, q)
     with pytest.raises(ValueError):
         X.gemm(q, torch.randn(64, 8, device="cuda"))
+
+
+@pytest.mark.parametrize("bits,bs,name,n,batch", [(4, 64, "linear-2", 768, 5), (4, 64, "linear-2", 64, 33),
+                                                   (8, 256, "dynamic", 512, 3), (4, 128, "dynamic", 128, 7)])
+def test_stack_quantize_dequantize_equal_per_matrix_calls(mods, code_maps, bits, bs, name, n, batch):
+    F, X = mods
+    g = torch.Generator().manual_seed(n + batch)
+    mats = torch.randn(batch, n, n, generator=g)
+    mats[1, 2, :] = 0.0
+    code = code_maps[(name, bits)]
+    code_d = torch.from_numpy(code).cuda()
+    for diag in (False, True):
+        for dtype in (torch.float32, torch.bfloat16):
+            src = mats.to(dtype)
+            q = X.quantize_stack(src.cuda(), X.empty_quantized(batch, n, bs, bits, code_d, diag))
+            back = X.dequantize_stack(q)
+            back16 = X.dequantize_stack(q, outdtype=torch.bfloat16)
+            torch.cuda.synchronize()
+            for b in range(batch):
+                o = Q.quantize_c(src[b].float().numpy(), code, n, bs, bits, diag)
+                assert np.array_equal(q.codes[b].cpu().numpy(), o[0])
+                assert np.array_equal(q.absmax[b].cpu().numpy(), o[1])
+                if diag:
+                    assert np.array_equal(q.diag[b].cpu().numpy(), o[2])
+                want = Q.dequantize_c(o[0], code, n, o[1], bs, bits, diag=o[2] if diag else None)
+                assert np.array_equal(back[b].cpu().numpy(), want)
+                want16 = Q.dequantize_c(o[0], code, n, o[1], bs, bits, diag=o[2] if diag else None, to_bf16=True)
+                assert np.array_equal(back16[b].float().cpu().numpy(), want16)
