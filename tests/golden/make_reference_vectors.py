@@ -9,7 +9,10 @@ Only functions whose exact outputs nothing else pins are executed here:
   * the seeded coupled-Newton inverse root and power iteration (they draw from the
     global torch RNG),
   * the eigenbasis bookkeeping of the 32-bit QTensorSVDFast path (QR signs, sort order),
-  * compute_power (Bjorck steps + inverse root in the kept subspace).
+  * compute_power (Bjorck steps + inverse root in the kept subspace),
+  * the preconditioner / optimizer step logic of optimizers/shampoo1.py and shampoo2.py on tiny
+    CPU parameters (block partitioning, statistics update, inverse roots, grafting, SGD and
+    AdamW updates).
 The blockwise quantizer itself is not run: IEEE-754 plus the written rules fix it.
 The reference's prebuilt native libraries are never loaded (its loader raises on a
 build of torch without a CUDA version string before it touches any file).
@@ -19,6 +22,68 @@ from pathlib import Path
 
 import numpy as np
 import torch
+
+
+def optimizer_runs():
+    """A few steps of the reference's preconditioners and optimizers on tiny CPU parameters (the
+    reference keeps everything in 32 bit on the CPU).  The global generator is re-seeded before
+    every step because the power iteration draws its start vector from it."""
+    import os
+    import tempfile
+
+    from optimizers import shampoo1 as R1
+    from optimizers import shampoo2 as R2
+
+    res = {}
+    cwd = os.getcwd()
+    with tempfile.TemporaryDirectory() as tmp:
+        os.chdir(tmp)                                   # shampoo2 writes logs/*.csv on first use
+        try:
+            g = torch.Generator().manual_seed(42)
+            shapes = [(6, 10), (5,), (4, 1, 3), (9, 9)]
+            grads = [[torch.randn(s, generator=g) for s in shapes] for _ in range(4)]
+            init = [torch.randn(s, generator=g) for s in shapes]
+            for k, t in enumerate(init):
+                res[f"opt_init_{k}"] = t.numpy().copy()
+            for st, gs in enumerate(grads):
+                for k, t in enumerate(gs):
+                    res[f"opt_grad_{st}_{k}"] = t.numpy().copy()
+
+            # bare preconditioners
+            for tag, mod, kw in (("s1", R1, {}), ("s2m0", R2, dict(inv_root_mode=0)), ("s2m1", R2, dict(inv_root_mode=1))):
+                var = init[0].clone()
+                pre = mod.Preconditioner(var, {}, stat_decay=0.9, matrix_eps=1e-6, prec_maxorder=4, prec_bits=32, **kw)
+                res[f"pre_{tag}_shapes"] = np.array(pre._partitioner.shapes_for_preconditioners())
+                for st in range(3):
+                    torch.manual_seed(1000 + st)
+                    pre.add_statistics(grads[st][0])
+                    pre.compute_preconditioners()
+                    res[f"pre_{tag}_out_{st}"] = pre.preconditioned_grad(grads[st][0]).numpy().copy()
+                for i, h in enumerate(pre.preconditioners):
+                    res[f"pre_{tag}_prec_{i}"] = h.dequantize().numpy().copy()
+                if tag == "s1":
+                    for i, h in enumerate(pre.statistics):
+                        res[f"pre_{tag}_stat_{i}"] = h.dequantize().numpy().copy()
+
+            # whole optimizers
+            runs = (("adamw1", R1.ShampooAdamW, dict(lr=1e-2, weight_decay=0.05)),
+                    ("sgd1", R1.ShampooSGD, dict(lr=1e-2, momentum=0.9, weight_decay=1e-3, nesterov=True)),
+                    ("adamw2", R2.ShampooAdamW, dict(lr=1e-2, weight_decay=0.05, inv_root_mode=0)),
+                    ("sgd2", R2.ShampooSGD, dict(lr=1e-2, momentum=0.9, inv_root_mode=1)))
+            for tag, cls, kw in runs:
+                params = [torch.nn.Parameter(t.clone()) for t in init]
+                opt = cls(params, start_prec_step=2, stat_compute_steps=1, prec_compute_steps=2, stat_decay=0.9,
+                          prec_maxorder=4, prec_bits=32, **kw)
+                for st in range(4):
+                    for p_, g_ in zip(params, grads[st]):
+                        p_.grad = g_.clone()
+                    torch.manual_seed(2000 + st)
+                    opt.step()
+                for k, p_ in enumerate(params):
+                    res[f"opt_{tag}_final_{k}"] = p_.detach().numpy().copy()
+        finally:
+            os.chdir(cwd)
+    return res
 
 
 def main() -> None:
@@ -87,6 +152,8 @@ def main() -> None:
     out["cp_keep"] = keep.numpy().copy()
     out["cp_out"] = RF.compute_power(vt, s, 4, iter_count=4, ridge_epsilon=1e-6,
                                      indices=keep, max_eigen=torch.tensor(3.0)).numpy().copy()
+
+    out.update(optimizer_runs())
 
     dest = Path(__file__).with_name("reference_vectors.npz")
     np.savez_compressed(dest, **out)
