@@ -1,0 +1,209 @@
+"""Batched execution of the "naive" low-bit Shampoo preconditioner over all parameters at once.
+
+The reference walks parameters, blocks and sides in Python and issues a handful of small
+kernels for each of them (optimizers/shampoo1.py:148-241, called per parameter from
+:371-427).  A ViT-B/32 has 124 blocks and 248 statistics of only four distinct orders, so the
+same arithmetic is done here with one launch per group of equally shaped blocks:
+
+  statistics   L <- b L + (1-b) G G^T : one fused product per (block shape, side) that reads the
+               quantized L inside its epilogue, then one stack quantize
+  inverse root one stack dequantize, one batched sync-free Newton run, one stack quantize per order
+  P_L G P_R    two fused products per block shape, the quantized factors expanded on the fly
+
+The quantized state of all blocks of one order lives in one stacked allocation
+(codes [B, n*n/2], maxima [B, n*n/bs], diagonals [B, n]); entry b is bit-for-bit what
+quantize_blockwise_diagreal writes for that matrix.  Parameters with a block the fused kernels
+cannot take (an order that the blocksize does not divide, or too small to quantize) keep a
+per-parameter `Preconditioner`.
+"""
+from collections import defaultdict
+
+import torch
+
+from optimizers.matrix_functions import ComputePowerBatched
+from optimizers.shampoo_common import BlockPartitioner
+from qtensor import fused as X
+
+
+class _Group:
+    """All blocks of one (rows, cols, leading dimension) shape."""
+
+    def __init__(self, bm, bn, ld):
+        self.bm, self.bn, self.ld = bm, bn, ld
+        self.param_index, self.offset = [], []       # which parameter, element offset of the block
+        self.slot = [None, None]                     # (order, first row in that order's stack) per side
+        self.grad_key, self.grad_ptrs, self.out_ptrs = None, None, None
+
+    def __len__(self):
+        return len(self.param_index)
+
+
+class ShampooBank:
+    def __init__(self, params, name2qmap, code, stat_decay=0.95, matrix_eps=1e-6, prec_maxorder=1200,
+                 prec_bits=4, min_lowbit_size=4096, quan_blocksize=64):
+        self.stat_decay, self.matrix_eps = stat_decay, matrix_eps
+        self.bits, self.blocksize = prec_bits, quan_blocksize
+        self.params = list(params)
+        self.device = self.params[0].device
+        self.code = name2qmap[code].to(self.device)
+        name2qmap[code] = self.code
+        self.shapes = []                              # matrix view (m, n) of every parameter
+        groups = {}
+        for pi, p in enumerate(self.params):
+            m, n = self.matrix_shape(p)
+            self.shapes.append((m, n))
+            part = BlockPartitioner(torch.empty(m, n, device="meta"), prec_maxorder)
+            rows = self._pieces(m, prec_maxorder)
+            cols = self._pieces(n, prec_maxorder)
+            assert len(part.shapes_for_preconditioners()) == 2 * len(rows) * len(cols)
+            r0 = 0
+            for bm in rows:
+                c0 = 0
+                for bn in cols:
+                    g = groups.setdefault((bm, bn, n), _Group(bm, bn, n))
+                    g.param_index.append(pi)
+                    g.offset.append(r0 * n + c0)
+                    c0 += bn
+                r0 += bm
+        self.groups = list(groups.values())
+        per_order = defaultdict(int)
+        for g in self.groups:
+            for side, order in enumerate((g.bm, g.bn)):
+                g.slot[side] = (order, per_order[order])
+                per_order[order] += len(g)
+        self.stats, self.precs, self.scratch = {}, {}, {}
+        for order, count in per_order.items():
+            eye = torch.eye(order, device=self.device).expand(count, order, order)
+            self.stats[order] = X.quantize_stack((matrix_eps * eye).contiguous(),
+                                                 X.empty_quantized(count, order, quan_blocksize, prec_bits, self.code, True))
+            self.precs[order] = X.quantize_stack(eye.contiguous(),
+                                                 X.empty_quantized(count, order, quan_blocksize, prec_bits, self.code, True))
+            biggest = max(len(g) for g in self.groups for o in (g.bm, g.bn) if o == order)
+            self.scratch[order] = torch.empty(biggest, order, order, device=self.device)
+        self.outputs = [torch.empty(m, n, device=self.device) for m, n in self.shapes]
+        for g in self.groups:
+            g.out_ptrs = torch.tensor([self.outputs[pi].data_ptr() + 4 * off for pi, off in zip(g.param_index, g.offset)],
+                                      dtype=torch.int64, device=self.device)
+        self._active = False
+
+    # ---- eligibility -----------------------------------------------------------------------------
+    @staticmethod
+    def matrix_shape(p):
+        dims = [d for d in p.shape if d != 1]
+        if len(dims) <= 1:
+            return None
+        first = dims[0]
+        return first, p.numel() // first
+
+    @staticmethod
+    def _pieces(extent, block):
+        if block > 0 and extent > block:
+            cuts = (extent - 1) // block
+            return [block] * cuts + [extent - cuts * block]
+        return [extent]
+
+    @classmethod
+    def accepts(cls, p, prec_maxorder, prec_bits, min_lowbit_size, quan_blocksize):
+        """A parameter can live in the bank when it is an fp32 GPU matrix all of whose block orders are
+        quantized in the layout the fused kernels read (blocksize divides the order)."""
+        if not p.is_cuda or p.dtype != torch.float32 or prec_bits not in (4, 8):
+            return False
+        shape = cls.matrix_shape(p)
+        if shape is None:
+            return False
+        orders = set(cls._pieces(shape[0], prec_maxorder) + cls._pieces(shape[1], prec_maxorder))
+        return all(o % quan_blocksize == 0 and o * o >= min_lowbit_size for o in orders)
+
+    # ---- per-step plumbing -----------------------------------------------------------------------
+    def _segment(self, table, g, side):
+        order, first = g.slot[side]
+        q = table[order]
+        n = len(g)
+        return X.Quantized(q.codes[first:first + n], q.absmax[first:first + n], q.diag[first:first + n], order,
+                           q.blocksize, q.bits, q.code)
+
+    def _grad_list(self, g, grads):
+        key = tuple(grads[pi].data_ptr() for pi in g.param_index)
+        if key != g.grad_key:
+            g.grad_ptrs = torch.tensor([base + 4 * off for base, off in zip(key, g.offset)], dtype=torch.int64,
+                                       device=self.device)
+            g.grad_key = key
+        return X.PtrList(g.grad_ptrs, (len(g), g.bm, g.bn), ld=g.ld)
+
+    def _check(self, grads):
+        if len(grads) != len(self.params):
+            raise ValueError("one gradient per parameter, in the order given at construction")
+        for grad, (m, n) in zip(grads, self.shapes):
+            if grad.numel() != m * n or not grad.is_contiguous() or grad.dtype != torch.float32 or not grad.is_cuda:
+                raise ValueError("gradients must be contiguous fp32 GPU tensors of the parameters' shapes")
+
+    # ---- the three operations of the reference's Preconditioner, for all parameters at once ------
+    @torch.no_grad()
+    def add_statistics(self, grads):
+        self._check(grads)
+        w1 = self.stat_decay
+        w2 = 1.0 if w1 == 1.0 else 1.0 - w1
+        for g in self.groups:
+            G = self._grad_list(g, grads)
+            for side in (0, 1):
+                seg = self._segment(self.stats, g, side)
+                out = self.scratch[seg.order][:len(g)]
+                X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, out=out)
+                X.quantize_stack(out, seg)
+
+    @torch.no_grad()
+    def compute_preconditioners(self, v0=None):
+        """v0: optional dict order -> [count, order] start vectors of the power iteration."""
+        for order, stat in self.stats.items():
+            dense = X.dequantize_stack(stat)
+            roots = ComputePowerBatched(dense, 4, ridge_epsilon=self.matrix_eps, v0=None if v0 is None else v0[order])
+            X.quantize_stack(roots.contiguous(), self.precs[order])
+        self._active = True
+
+    @torch.no_grad()
+    def preconditioned_grads(self, grads):
+        """List of P_L G P_R per parameter (buffers owned by the bank, overwritten by the next call)."""
+        self._check(grads)
+        for g in self.groups:
+            G = self._grad_list(g, grads)
+            tmp = X.gemm(self._segment(self.precs, g, 0), G)
+            X.gemm(tmp, self._segment(self.precs, g, 1), out=X.PtrList(g.out_ptrs, (len(g), g.bm, g.bn), ld=g.ld))
+        return [out.view(p.shape) for out, p in zip(self.outputs, self.params)]
+
+    def is_active(self):
+        return self._active
+
+    # ---- inspection (tests, checkpoints) ---------------------------------------------------------
+    def block_table(self):
+        """[(parameter index, block index within the parameter (row-major), side, order, row in that
+        order's stack)] -- where every statistic / preconditioner of the per-parameter layout lives."""
+        per_param = defaultdict(list)
+        for g in self.groups:
+            for i, (pi, off) in enumerate(zip(g.param_index, g.offset)):
+                per_param[pi].append((off, g, i))
+        rows = []
+        for pi in sorted(per_param):
+            n = self.shapes[pi][1]
+            items = sorted(per_param[pi], key=lambda t: (t[0] // n, t[0] % n))
+            for j, (_, g, i) in enumerate(items):
+                for side in (0, 1):
+                    order, first = g.slot[side]
+                    rows.append((pi, j, side, order, first + i))
+        return rows
+
+    def state_dict(self):
+        out = {"active": self._active}
+        for name, table in (("stats", self.stats), ("precs", self.precs)):
+            for order, q in table.items():
+                out[f"{name}.{order}.codes"] = q.codes
+                out[f"{name}.{order}.absmax"] = q.absmax
+                out[f"{name}.{order}.diag"] = q.diag
+        return out
+
+    def load_state_dict(self, sd):
+        self._active = bool(sd["active"])
+        for name, table in (("stats", self.stats), ("precs", self.precs)):
+            for order, q in table.items():
+                q.codes.copy_(sd[f"{name}.{order}.codes"])
+                q.absmax.copy_(sd[f"{name}.{order}.absmax"])
+                q.diag.copy_(sd[f"{name}.{order}.diag"])

@@ -38,15 +38,126 @@ class Preconditioner(PreconditionerBase):
         # Like the reference (shampoo1.py:198), a statistic held in fp32 is passed without a copy,
         # so the ridge term the Newton routine adds in place stays in the stored statistic.
         stat = holder.dequantize()
-        return newton_inverse_root(stat, exp, eps).to(stat.dtype)
+        return newton_inverse_root(stat, exp, eps, getattr(self, '_v0', None)).to(stat.dtype)
 
 
 class ShampooSGD(ShampooSGDBase):
+    """fused=True (not in the reference) runs all eligible GPU parameters through one batched
+    ShampooBank instead of one Preconditioner object per parameter; the arithmetic is the same."""
     preconditioner_class = Preconditioner
+
+    def __init__(self, params, *args, fused=False, **kwargs):
+        super().__init__(params, *args, **kwargs)
+        self._fused = fused
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        if not self._fused:
+            return super().step(closure)
+        for group in self.param_groups:
+            fused_step(self, group, _sgd_update)
 
 
 class ShampooAdamW(ShampooAdamWBase):
+    """fused=True (not in the reference) runs all eligible GPU parameters through one batched
+    ShampooBank instead of one Preconditioner object per parameter; the arithmetic is the same."""
     preconditioner_class = Preconditioner
+
+    def __init__(self, params, *args, fused=False, **kwargs):
+        super().__init__(params, *args, **kwargs)
+        self._fused = fused
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        if not self._fused:
+            return super().step(closure)
+        for group in self.param_groups:
+            fused_step(self, group, _adamw_update)
+
+
+def fused_step(opt, group, update):
+    """One optimizer step of a parameter group with the preconditioner work batched."""
+    import math  # noqa: F401
+    from optimizers.engine import ShampooBank
+
+    params = [p for p in group['params'] if p.grad is not None]
+    if not params:
+        return
+    cache = opt.__dict__.setdefault('_fused_cache', {})
+    entry = cache.get(id(group))
+    if entry is None:
+        keys = ('prec_maxorder', 'prec_bits', 'min_lowbit_size', 'quan_blocksize')
+        banked = [p for p in params if ShampooBank.accepts(p, *(group[k] for k in keys))]
+        bank = ShampooBank(banked, opt.name2qmap, CODE, stat_decay=group['stat_decay'], matrix_eps=group['matrix_eps'],
+                           **{k: group[k] for k in keys}) if banked else None
+        entry = cache[id(group)] = dict(bank=bank, banked=banked, ids={id(p) for p in banked}, step=0)
+        for p in params:
+            state = opt.state[p]
+            state['step'] = 0
+            if id(p) not in entry['ids']:
+                state['preconditioner'] = opt._make_preconditioner(p, group)
+    entry['step'] += 1
+    step, bank, banked = entry['step'], entry['bank'], entry['banked']
+    others = [p for p in params if id(p) not in entry['ids']]
+    for p in params:
+        opt.state[p]['step'] = step
+    if update is _adamw_update:
+        torch._foreach_mul_(params, 1 - group['lr'] * group['weight_decay'])
+    bgrads = [p.grad.contiguous() for p in banked]
+    directions = {}
+    if bank is not None:
+        if step % group['stat_compute_steps'] == 0:
+            bank.add_statistics(bgrads)
+        if step % group['prec_compute_steps'] == 0:
+            bank.compute_preconditioners()
+        if step >= group['start_prec_step'] and bank.is_active():
+            outs = bank.preconditioned_grads(bgrads)
+            gnorm = torch._foreach_norm(bgrads)
+            onorm = torch._foreach_norm(outs)
+            torch._foreach_add_(onorm, 1e-12)
+            torch._foreach_div_(gnorm, onorm)
+            torch._foreach_mul_(outs, gnorm)                      # keep each gradient's norm
+            directions = {id(p): o for p, o in zip(banked, outs)}
+    for p in others:
+        directions[id(p)] = opt._shampoo_direction(p, p.grad, group, opt.state[p])
+    update(opt, group, params, [directions.get(id(p), p.grad) for p in params], step)
+
+
+def _adamw_update(opt, group, params, dirs, step):
+    import math
+    for p in params:
+        state = opt.state[p]
+        if 'exp_avg' not in state:
+            state['exp_avg'] = torch.zeros_like(p, memory_format=torch.preserve_format)
+            state['exp_avg_sq'] = torch.zeros_like(p, memory_format=torch.preserve_format)
+    m = [opt.state[p]['exp_avg'] for p in params]
+    v = [opt.state[p]['exp_avg_sq'] for p in params]
+    beta1, beta2 = group['betas']
+    torch._foreach_mul_(m, beta1)
+    torch._foreach_add_(m, dirs, alpha=1 - beta1)
+    torch._foreach_mul_(v, beta2)
+    torch._foreach_addcmul_(v, dirs, dirs, value=1 - beta2)
+    denom = torch._foreach_sqrt(v)
+    torch._foreach_div_(denom, math.sqrt(1 - beta2 ** step))
+    torch._foreach_add_(denom, group['eps'])
+    torch._foreach_addcdiv_(params, m, denom, value=-group['lr'] / (1 - beta1 ** step))
+
+
+def _sgd_update(opt, group, params, dirs, step):
+    for p in params:
+        state = opt.state[p]
+        if 'momentum' not in state:
+            state['momentum'] = torch.zeros_like(p, memory_format=torch.preserve_format)
+    if group['weight_decay'] != 0.0:
+        torch._foreach_add_(dirs, params, alpha=group['weight_decay'])
+    bufs = [opt.state[p]['momentum'] for p in params]
+    torch._foreach_mul_(bufs, group['momentum'])
+    torch._foreach_add_(bufs, dirs)
+    if group['nesterov']:
+        dirs = torch._foreach_add(dirs, bufs, alpha=group['momentum'])
+    else:
+        dirs = bufs
+    torch._foreach_add_(params, dirs, alpha=-group['lr'])
 
 
 ShampooSGD.__doc__ = _DOC.format(base="SGD", more="")

@@ -48,7 +48,7 @@ class Preconditioner(PreconditionerBase):
         if self.inv_root_mode == 0:
             return holder.computepower(exp, ridge_epsilon=eps)
         stat, _ = holder.dequantize()
-        return newton_inverse_root(stat, exp, eps).to(stat.dtype)
+        return newton_inverse_root(stat, exp, eps, getattr(self, '_v0', None)).to(stat.dtype)
 
 
 class ShampooSGD(ShampooSGDBase):

@@ -141,10 +141,14 @@ class PreconditionerBase:
             for axis in range(rank):
                 self._accumulate(self.statistics[j * rank + axis], block, axis, w1, w2)
 
-    def compute_preconditioners(self):
-        """Refresh every preconditioner with the inverse 4th root of its statistic."""
-        for stat, prec in zip(self.statistics, self.preconditioners):
+    def compute_preconditioners(self, v0=None):
+        """Refresh every preconditioner with the inverse 4th root of its statistic.
+        v0 (not in the reference): optional start vectors of the power iteration, one per
+        statistic; by default they are drawn from the global generator as the reference does."""
+        for i, (stat, prec) in enumerate(zip(self.statistics, self.preconditioners)):
+            self._v0 = None if v0 is None else v0[i]
             prec.quantize(self._inverse_root(stat, 4, self.matrix_eps))
+        self._v0 = None
         self._active = True
 
     def preconditioned_grad(self, grad):
@@ -176,12 +180,13 @@ def dense_gram(block, axis):
     return block.T @ block if axis == 1 else block @ block.T
 
 
-def newton_inverse_root(mat, exp, eps):
+def newton_inverse_root(mat, exp, eps, v0=None):
     """(mat + ridge)^(-1/exp) by the coupled Newton iteration; matrix cores on a GPU."""
     mat = mat.float()
     if mat.is_cuda and F.lib is not None and mat.dim() == 2 and mat.shape[0] > 1:
-        return ComputePowerBatched(mat.unsqueeze(0).contiguous(), exp, ridge_epsilon=eps)[0]
-    return ComputePower(mat, exp, ridge_epsilon=eps)
+        start = None if v0 is None else v0.reshape(1, -1)
+        return ComputePowerBatched(mat.unsqueeze(0).contiguous(), exp, ridge_epsilon=eps, v0=start)[0]
+    return ComputePower(mat, exp, ridge_epsilon=eps, v0=v0)
 
 
 def build_code_maps(prec_bits):

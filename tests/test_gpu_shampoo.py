@@ -1,0 +1,154 @@
+"""GPU parity of the low-bit preconditioner step: the per-parameter Preconditioner (reference
+layout), the batched ShampooBank and the fused optimizer, against the CPU restatement with the
+quantizer oracle (oracle/shampoo_ref.py) on identical gradients and start vectors.
+
+Tolerances.  One fused statistics update differs from the CPU flow only by fp32 summation order
+inside the products (~1e-7 relative), so after quantization almost every code agrees; a code can
+flip where a quotient sits within that distance of a decision threshold.  Bounds used: at most
+0.1 % of codes differ after three updates; dequantized statistics within 1e-3, preconditioned
+gradients within 2e-3 relative Frobenius norm.  Bank against per-parameter path (same kernels,
+same start vectors): bit-identical statistics, inverse roots equal to rounding."""
+import numpy as np
+import pytest
+import torch
+
+from oracle.shampoo_ref import RefPreconditioner
+
+pytestmark = pytest.mark.gpu
+SHAPES = [(128, 192), (256, 64), (64,), (192, 1, 128)]
+KW = dict(stat_decay=0.95, matrix_eps=1e-6, prec_maxorder=128, prec_bits=4, min_lowbit_size=4096, quan_blocksize=64)
+
+
+def rel(a, b):
+    a, b = torch.as_tensor(a).double().cpu(), torch.as_tensor(b).double().cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-300))
+
+
+@pytest.fixture(scope="module")
+def setup(code_maps):
+    import qtensor.functional as F
+    from optimizers import shampoo1 as S1
+    from optimizers.engine import ShampooBank
+    assert torch.cuda.is_available() and F.lib is not None
+    g = torch.Generator().manual_seed(11)
+    grads = [[0.02 * torch.randn(s, generator=g) for s in SHAPES] for _ in range(3)]
+    return S1, ShampooBank, grads, code_maps[("linear-2", 4)]
+
+
+def start_vectors(step, orders):
+    g = torch.Generator().manual_seed(500 + step)
+    return [torch.rand(o, generator=g) * 2 - 1 for o in orders]
+
+
+def test_per_parameter_low_bit_path_follows_the_oracle(setup):
+    S1, _, grads, code = setup
+    for k, shape in enumerate(SHAPES):
+        ref = RefPreconditioner(shape, code, **KW)
+        qmap = {"linear-2": torch.from_numpy(code)}
+        pre = S1.Preconditioner(torch.zeros(shape, device="cuda"), qmap, **KW)
+        assert len(pre.statistics) == len(ref.stats)
+        orders = [s.order for s in ref.stats]
+        for st in range(3):
+            grad = grads[st][k]
+            ref.add_statistics(grad)
+            pre.add_statistics(grad.cuda())
+            v0 = start_vectors(st, orders)
+            ref.compute_preconditioners(v0)
+            pre.compute_preconditioners([v.cuda() for v in v0])
+            out = pre.preconditioned_grad(grad.cuda())
+            want = ref.preconditioned_grad(grad)
+            assert out.shape == grad.shape
+            assert rel(out, want) <= 2e-3, (shape, st)
+        for h, slot in zip(pre.statistics, ref.stats):
+            assert h.bits == 4 and slot.low
+            codes, absmax, diag = slot.codes()
+            got = h.var.cpu().numpy()
+            differing = np.count_nonzero((got >> 4) != (codes >> 4)) + np.count_nonzero((got & 15) != (codes & 15))
+            assert differing <= 1e-3 * 2 * got.size
+            assert rel(h.absmax, absmax) <= 1e-5 and rel(h.diag, diag) <= 1e-5
+            assert rel(h.dequantize(), slot.get()) <= 1e-3
+        for h, slot in zip(pre.preconditioners, ref.precs):
+            assert rel(h.dequantize(), slot.get()) <= 2e-3
+
+
+def test_bank_equals_per_parameter_path(setup):
+    S1, ShampooBank, grads, code = setup
+    mats = [s for s in SHAPES if len([d for d in s if d != 1]) > 1]
+    params = [torch.zeros(s, device="cuda") for s in mats]
+    kw = {k: v for k, v in KW.items() if k in ("prec_maxorder", "prec_bits", "min_lowbit_size", "quan_blocksize")}
+    assert all(ShampooBank.accepts(p, **kw) for p in params)
+    assert not ShampooBank.accepts(torch.zeros(64, device="cuda"), **kw)
+    assert not ShampooBank.accepts(torch.zeros(128, 100, device="cuda"), **kw)       # 100 is not a multiple of 64
+    assert not ShampooBank.accepts(torch.zeros(128, 128), **kw)                      # CPU
+    qmap = {"linear-2": torch.from_numpy(code)}
+    bank = ShampooBank(params, qmap, "linear-2", **KW)
+    pres = [S1.Preconditioner(p, qmap, **KW) for p in params]
+    table = bank.block_table()
+    assert len(table) == sum(len(p.statistics) for p in pres)
+    idx = [SHAPES.index(s) for s in mats]
+    for st in range(3):
+        gl = [grads[st][i].cuda() for i in idx]
+        bank.add_statistics(gl)
+        v0_bank = {o: torch.empty(q.batch, o) for o, q in bank.stats.items()}
+        v0_pre = []
+        for pi, pre in enumerate(pres):
+            pre.add_statistics(gl[pi])
+            orders = [h.var_order for h in pre.statistics]
+            vs = start_vectors(st * 10 + pi, orders)
+            v0_pre.append(vs)
+            for (tpi, j, side, order, row) in table:
+                if tpi == pi:
+                    v0_bank[order][row] = vs[2 * j + side]
+        bank.compute_preconditioners({o: v.cuda() for o, v in v0_bank.items()})
+        outs = bank.preconditioned_grads(gl)
+        for pi, pre in enumerate(pres):
+            pre.compute_preconditioners([v.cuda() for v in v0_pre[pi]])
+            want = pre.preconditioned_grad(gl[pi])
+            assert outs[pi].shape == want.shape
+            assert rel(outs[pi], want) <= 1e-4
+    for (pi, j, side, order, row) in table:
+        h = pres[pi].statistics[2 * j + side]              # statistics: same kernels, bit-identical
+        assert torch.equal(bank.stats[order].codes[row], h.var)
+        assert torch.equal(bank.stats[order].absmax[row], h.absmax)
+        assert torch.equal(bank.stats[order].diag[row], h.diag)
+        # inverse roots: torch's batched reductions (norms, matrix-vector products) round differently
+        # for a stack of one and a stack of many, so agreement is to rounding, not to the bit
+        h = pres[pi].preconditioners[2 * j + side]
+        got, want = bank.precs[order].codes[row], h.var
+        differing = int(((got >> 4) != (want >> 4)).sum() + ((got & 15) != (want & 15)).sum())
+        assert differing <= 1e-3 * 2 * got.numel()
+        assert rel(bank.precs[order].absmax[row], h.absmax) <= 1e-5
+        assert rel(bank.precs[order].diag[row], h.diag) <= 1e-5
+    sd = bank.state_dict()
+    bank2 = ShampooBank(params, qmap, "linear-2", **KW)
+    bank2.load_state_dict(sd)
+    first = outs[0].clone()
+    assert bank2.is_active() and torch.equal(bank2.preconditioned_grads(gl)[0], first)
+
+
+@pytest.mark.parametrize("which", ["adamw", "sgd"])
+def test_fused_optimizer_matches_per_parameter_optimizer(setup, which, monkeypatch):
+    S1, _, grads, _ = setup
+    import optimizers.matrix_functions as MF
+    real_rand = torch.rand
+    # identical, deterministic power-iteration start vectors on both paths
+    monkeypatch.setattr(MF.torch, "rand", lambda *size, **kw: torch.full(size, 0.75, **kw))
+    shapes = SHAPES + [(128, 100)]                     # the last one cannot enter the bank
+    g = torch.Generator().manual_seed(5)
+    init = [real_rand(s, generator=g) for s in shapes]
+    gs = [[0.02 * torch.randn(s, generator=g) for s in shapes] for _ in range(4)]
+    finals = []
+    for fused in (False, True):
+        params = [torch.nn.Parameter(t.clone().cuda()) for t in init]
+        common = dict(start_prec_step=2, stat_compute_steps=1, prec_compute_steps=2, fused=fused, **KW)
+        opt = (S1.ShampooAdamW(params, lr=1e-2, weight_decay=0.05, **common) if which == "adamw"
+               else S1.ShampooSGD(params, lr=1e-2, momentum=0.9, weight_decay=1e-3, nesterov=True, **common))
+        for st in range(4):
+            for p, gr in zip(params, gs[st]):
+                p.grad = gr.clone().cuda()
+            opt.step()
+        finals.append([p.detach().cpu() for p in params])
+    # four steps of size lr = 1e-2 on O(1) parameters; the two paths agree to a small fraction of one
+    # update (Adam's normalisation magnifies the rounding-level differences of the inverse roots)
+    for a, b in zip(*finals):
+        assert rel(a, b) <= 2e-4
