@@ -2,10 +2,12 @@
 (268,435,456 elements, 1 GiB; 99% N(0,1) + 1% outliers of sigma 10; linear-2 table, block 64)
 on one MI355X, reported as achieved HBM GB/s over the algorithmic bytes.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-step]
 
 One "step" = one quantize launch + one dequantize launch over the whole tensor, inputs
-resident in HBM.  Prints one JSON line.
+resident in HBM.  The same JSON line also carries, under "precond_step", the second half of the
+metric: ms per 4-bit Shampoo preconditioner step over the ViT-B/32 weight shapes, with the CPU
+restatement timed on a bounded sample beside it.  Prints one JSON line.
 """
 import argparse
 import json
@@ -60,12 +62,106 @@ def cpu_baseline(torch, x_slice, code):
     }
 
 
+def vit_b32_shapes():
+    """All 2-D weights of a ViT-Base/32 (12 layers) plus patch embedding and a 100-way head."""
+    shapes = []
+    for _ in range(12):
+        shapes += [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
+    return shapes + [(3072, 768), (768, 100)]
+
+
+STEP_KW = dict(stat_decay=0.95, matrix_eps=1e-6, prec_maxorder=1024, prec_bits=4, min_lowbit_size=4096,
+               quan_blocksize=64)
+
+
+def precond_step_gpu(torch):
+    """ms per full 4-bit Shampoo (statistics stored quantized, Newton inverse roots) + AdamW step over the
+    ViT-B/32 shapes: statistics every step, inverse 4th roots every 10th step, preconditioned and
+    norm-grafted update every step.  Ten untimed steps bring the preconditioners into use."""
+    from optimizers import shampoo1 as S1
+
+    g = torch.Generator(device="cuda").manual_seed(1)
+    params = [torch.nn.Parameter(0.02 * torch.randn(s, device="cuda", generator=g)) for s in vit_b32_shapes()]
+    grads = [0.02 * torch.randn(p.shape, device="cuda", generator=g) for p in params]
+    opt = S1.ShampooAdamW(params, lr=1e-3, weight_decay=0.05, start_prec_step=1, stat_compute_steps=1,
+                          prec_compute_steps=10, fused=True, **STEP_KW)
+    for p, gr in zip(params, grads):
+        p.grad = gr
+
+    def timed_step():
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        opt.step()
+        e1.record()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3, e0.elapsed_time(e1)
+
+    for _ in range(10):
+        timed_step()
+    regular, newton = [], []
+    for i in range(11, 31):
+        wall, dev = timed_step()
+        (newton if i % 10 == 0 else regular).append((wall, dev))
+    mean = lambda xs, k: sum(x[k] for x in xs) / len(xs)          # noqa: E731
+    reg, new = mean(regular, 0), mean(newton, 0)
+    blocks = sum(((m - 1) // 1024 + 1) * ((n - 1) // 1024 + 1) for m, n in vit_b32_shapes())
+    gram_flop = sum(2 * m * m * n + 2 * m * n * n for m, n in vit_b32_shapes())   # unblocked upper bound is not used:
+    gram_flop = 0
+    for m, n in vit_b32_shapes():
+        rows = [1024] * ((m - 1) // 1024) + [m - 1024 * ((m - 1) // 1024)]
+        cols = [1024] * ((n - 1) // 1024) + [n - 1024 * ((n - 1) // 1024)]
+        gram_flop += sum(2 * a * a * b + 2 * a * b * b for a in rows for b in cols)
+    return {
+        "workload": "ViT-B/32 2-D weights (50 parameters, %d blocks of at most 1024, %d quantized statistics and as many "
+                    "preconditioners), fp32 N(0,0.02^2) gradients, 4-bit linear-2 blocksize 64, beta 0.95, statistics "
+                    "every step, coupled-Newton inverse 4th roots every 10th step, AdamW update; "
+                    "optimizers.shampoo1.ShampooAdamW(fused=True)" % (blocks, 2 * blocks, ),
+        "ms_per_step_regular": round(reg, 3),
+        "ms_per_step_with_inverse_roots": round(new, 3),
+        "ms_per_step_amortized_over_10": round((9 * reg + new) / 10, 3),
+        "device_ms_regular": round(mean(regular, 1), 3),
+        "device_ms_with_inverse_roots": round(mean(newton, 1), 3),
+        "product_gflop_per_regular_step": round(2 * gram_flop / 1e9, 1),
+        "product_tflops_regular": round(2 * gram_flop / (mean(regular, 1) * 1e-3) / 1e12, 1),
+    }
+
+
+def precond_step_cpu(torch, code_host):
+    """The same regular step (statistics update + preconditioned gradient) for ONE transformer layer
+    (qkv, proj, fc1, fc2: 10 of the 124 blocks) through the CPU restatement whose quantizer is the
+    reference's per-segment torch loop; the inverse roots are timed separately on the same layer."""
+    from oracle.shampoo_ref import RefPreconditioner
+
+    g = torch.Generator().manual_seed(1)
+    shapes = [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
+    grads = [0.02 * torch.randn(s, generator=g) for s in shapes]
+    pres = [RefPreconditioner(s, code_host.numpy(), loop=True, **STEP_KW) for s in shapes]
+    t0 = time.perf_counter()
+    for pre, gr in zip(pres, grads):
+        pre.add_statistics(gr)
+        out = pre.preconditioned_grad(gr)
+        out.mul_(gr.norm() / (out.norm() + 1e-12))
+    regular = time.perf_counter() - t0
+    return {
+        "kind": "port",
+        "cores": torch.get_num_threads(),
+        "sample": "one transformer layer (4 of 50 parameters, 10 of 124 blocks, 20 of 248 statistics): statistics "
+                  "update + preconditioned gradient + norm graft; quantizer = per-segment torch loop (1 core), "
+                  "products = torch.matmul on %d threads" % torch.get_num_threads(),
+        "seconds_for_sample": round(regular, 3),
+        "ms_per_full_step_extrapolated": round(regular * 1e3 * 124 / 10, 1),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-step", action="store_true", help="skip the Shampoo preconditioner-step measurement")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
@@ -163,9 +259,18 @@ def main():
             "avg_launch_ms": round(d_ms, 4),
         },
     }
+    x_slice = None if args.no_cpu_baseline else x.view(-1)[: 4096 * 4096].cpu()
+    del x, out, absmax, back
+    torch.cuda.empty_cache()
+    if not args.no_step:
+        result["precond_step"] = precond_step_gpu(torch)
     if not args.no_cpu_baseline:
-        x_slice = x.view(-1)[: 4096 * 4096].cpu()
         result["cpu_baseline"] = cpu_baseline(torch, x_slice, code_host)
+        if not args.no_step:
+            cpu = precond_step_cpu(torch, code_host)
+            result["precond_step"]["cpu_baseline"] = cpu
+            result["precond_step"]["speedup_vs_cpu_regular_step"] = round(
+                cpu["ms_per_full_step_extrapolated"] / result["precond_step"]["ms_per_step_regular"], 1)
     print(json.dumps(result))
 
 
