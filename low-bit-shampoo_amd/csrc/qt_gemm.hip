@@ -14,9 +14,10 @@
 //              Newton: C = acc, T = (1 - w) I + w * acc, err = max |acc - I|.
 //
 // Tiling: workgroup = 4 waves in a 2 x 2 grid, block tile BM x BN x 16, each wave owns
-// (BM/2) x (BN/2) as 32 x 32 MFMA blocks.  Both operand tiles sit in LDS as [row][k] with an odd
-// row stride so the per-lane fragment reads (row = lane % 32, k = lane / 32) hit 32 different
-// banks.  Global loads for tile t+1 are issued before the MFMAs of tile t.
+// (BM/2) x (BN/2) as 32 x 32 MFMA blocks.  Both operand tiles sit in LDS k-major ([k][row], row
+// stride rows + 4) so the per-lane fragment reads (row = lane % 32, k = lane / 32) are
+// consecutive words and row-contiguous sources are written with 16-byte stores.  Global loads
+// run two tiles ahead of the MFMAs; the LDS commit sits in the middle of the MFMA stream.
 #include "qt_common.h"
 
 #include <type_traits>
@@ -61,8 +62,24 @@ namespace {
 
 constexpr int BK = 16;
 constexpr uint32_t kDies = 8;          // accelerator dies (XCDs) of an MI355X
-constexpr int LDS_STRIDE = BK + 1;
+constexpr int LDS_PAD = 4;   // row stride = rows + 4 floats: k-major tiles, 16-byte aligned rows
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+// Pointers that arrive inside a by-value struct or from a pointer table are "generic" to the
+// compiler, which then emits flat_* instructions (slower, and they also count on the LDS wait
+// counter).  Everything here lives in global memory: say so.
+#define QT_GLOBAL __attribute__((address_space(1)))
+__device__ __forceinline__ float gload(const float *p) { return *(const QT_GLOBAL float *)p; }
+__device__ __forceinline__ float4 gload4(const float *p) {
+    const qt_f32x4 v = *(const QT_GLOBAL qt_f32x4 *)p;
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint32_t gload_u32(const void *p) { return *(const QT_GLOBAL uint32_t *)p; }
+__device__ __forceinline__ uint2 gload_u32x2(const void *p) {
+    const qt_u32x2 v = *(const QT_GLOBAL qt_u32x2 *)p;
+    return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint32_t gload_u8(const uint8_t *p) { return *(const QT_GLOBAL uint8_t *)p; }
+__device__ __forceinline__ void gstore(float *p, float v) { *(QT_GLOBAL float *)p = v; }
 
 template <typename T>
 __device__ __forceinline__ const T *batch_ptr(const BatchPtr &p, int b) {
@@ -76,16 +93,16 @@ inline bool has_host_ptr(const BatchPtr &p) { return p.base != nullptr || p.list
 template <int BITS>
 __device__ __forceinline__ float dequant_element(const uint8_t *codes, const float *absmax, const float *diag,
                                                  const float *s_code, int order, int bs_shift, int r, int c) {
-    if (diag != nullptr && r == c) return diag[r];
+    if (diag != nullptr && r == c) return gload(diag + r);
     const long long k = (long long)r * order + c;
     uint32_t id;
-    if (BITS == 8) id = codes[k];
-    else { const uint32_t byte = codes[k >> 1]; id = (k & 1) ? (byte & 15u) : (byte >> 4); }
-    const float a = absmax[k >> bs_shift];
+    if (BITS == 8) id = gload_u8(codes + k);
+    else { const uint32_t byte = gload_u8(codes + (k >> 1)); id = (k & 1) ? (byte & 15u) : (byte >> 4); }
+    const float a = gload(absmax + (k >> bs_shift));
     return a == 0.0f ? 0.0f : s_code[id] * a;
 }
 
-// ---- tile loaders: global -> registers -> LDS ([row][k], row stride LDS_STRIDE) -------------
+// ---- tile loaders: global -> registers -> LDS ([k][row], row stride rows + LDS_PAD) -------------
 // Every loader covers ROWS x BK elements with 256 threads and keeps them in registers between
 // `fetch` (global loads, issued early) and `commit` (LDS stores, after the barrier).
 
@@ -103,24 +120,25 @@ struct LoadKContig {
             float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
             if (gr < rows) {
                 const float *p = base + (long long)gr * ld + gk;
-                if (vec_ok && gk + 3 < K) x = *reinterpret_cast<const float4 *>(p);
+                if (vec_ok && gk + 3 < K) x = gload4(p);
                 else {
-                    if (gk < K) x.x = p[0];
-                    if (gk + 1 < K) x.y = p[1];
-                    if (gk + 2 < K) x.z = p[2];
-                    if (gk + 3 < K) x.w = p[3];
+                    if (gk < K) x.x = gload(p);
+                    if (gk + 1 < K) x.y = gload(p + 1);
+                    if (gk + 2 < K) x.z = gload(p + 2);
+                    if (gk + 3 < K) x.w = gload(p + 3);
                 }
             }
             v[i] = x;
         }
     }
     __device__ __forceinline__ void commit(float *lds) const {
+        constexpr int LD = ROWS + LDS_PAD;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const int f = threadIdx.x + i * 256;
             const int r = f >> 2, kq = (f & 3) << 2;
-            float *d = lds + r * LDS_STRIDE + kq;
-            d[0] = v[i].x; d[1] = v[i].y; d[2] = v[i].z; d[3] = v[i].w;
+            float *d = lds + kq * LD + r;
+            d[0] = v[i].x; d[LD] = v[i].y; d[2 * LD] = v[i].z; d[3 * LD] = v[i].w;
         }
     }
 };
@@ -139,12 +157,12 @@ struct LoadRowContig {
             float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
             if (gk < K) {
                 const float *p = base + (long long)gk * ld + gr;
-                if (vec_ok && gr + 3 < rows) x = *reinterpret_cast<const float4 *>(p);
+                if (vec_ok && gr + 3 < rows) x = gload4(p);
                 else {
-                    if (gr < rows) x.x = p[0];
-                    if (gr + 1 < rows) x.y = p[1];
-                    if (gr + 2 < rows) x.z = p[2];
-                    if (gr + 3 < rows) x.w = p[3];
+                    if (gr < rows) x.x = gload(p);
+                    if (gr + 1 < rows) x.y = gload(p + 1);
+                    if (gr + 2 < rows) x.z = gload(p + 2);
+                    if (gr + 3 < rows) x.w = gload(p + 3);
                 }
             }
             v[i] = x;
@@ -155,8 +173,7 @@ struct LoadRowContig {
         for (int i = 0; i < VEC; ++i) {
             const int f = threadIdx.x + i * 256;
             const int kk = f / (ROWS / 4), rq = (f % (ROWS / 4)) << 2;
-            float *d = lds + rq * LDS_STRIDE + kk;
-            d[0] = v[i].x; d[LDS_STRIDE] = v[i].y; d[2 * LDS_STRIDE] = v[i].z; d[3 * LDS_STRIDE] = v[i].w;
+            *reinterpret_cast<float4 *>(lds + kk * (ROWS + LDS_PAD) + rq) = v[i];
         }
     }
 };
@@ -188,10 +205,10 @@ struct LoadQuant {
             const int mc = ALONG_K ? k0 + tc : row0 + tc;     // first matrix column of the group
             if (mr < q.order && mc < q.order) {               // order is a multiple of 64: whole group inside
                 const long long k = (long long)mr * q.order + mc;
-                const float a = absmax[k >> q.bs_shift];
+                const float a = gload(absmax + (k >> q.bs_shift));
                 uint32_t id[8];
                 if (BITS == 4) {
-                    const uint32_t w = *reinterpret_cast<const uint32_t *>(codes + (k >> 1));
+                    const uint32_t w = gload_u32(codes + (k >> 1));
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const uint32_t byte = (w >> (8 * e)) & 255u;
@@ -199,13 +216,13 @@ struct LoadQuant {
                         id[2 * e + 1] = byte & 15u;
                     }
                 } else {
-                    const uint2 w = *reinterpret_cast<const uint2 *>(codes + k);
+                    const uint2 w = gload_u32x2(codes + k);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) { id[e] = (w.x >> (8 * e)) & 255u; id[4 + e] = (w.y >> (8 * e)) & 255u; }
                 }
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[g][e] = a == 0.0f ? 0.0f : s_code[id[e]] * a;
-                if (diag != nullptr && mr >= mc && mr < mc + 8) v[g][mr - mc] = diag[mr];
+                if (diag != nullptr && mr >= mc && mr < mc + 8) v[g][mr - mc] = gload(diag + mr);
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[g][e] = 0.0f;
@@ -218,14 +235,15 @@ struct LoadQuant {
             if (!active(g)) continue;
             int tr, tc;
             locate(g, tr, tc);
+            constexpr int LD = ROWS + LDS_PAD;
             if (ALONG_K) {
-                float *d = lds + tr * LDS_STRIDE + tc;
+                float *d = lds + tc * LD + tr;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) d[e] = v[g][e];
+                for (int e = 0; e < 8; ++e) d[e * LD] = v[g][e];
             } else {
-                float *d = lds + tc * LDS_STRIDE + tr;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) d[e * LDS_STRIDE] = v[g][e];
+                float4 *d = reinterpret_cast<float4 *>(lds + tr * LD + tc);
+                d[0] = make_float4(v[g][0], v[g][1], v[g][2], v[g][3]);
+                d[1] = make_float4(v[g][4], v[g][5], v[g][6], v[g][7]);
             }
         }
     }
@@ -248,8 +266,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     const int b = id / tiles_m;
     if (args.skip != nullptr && args.skip[b] != 0) return;
 
-    __shared__ float s_a[2][BM * LDS_STRIDE];
-    __shared__ float s_b[2][BN * LDS_STRIDE];
+    constexpr int LDA = BM + LDS_PAD, LDB = BN + LDS_PAD;
+    __shared__ __attribute__((aligned(16))) float s_a[2][BK * LDA];
+    __shared__ __attribute__((aligned(16))) float s_b[2][BK * LDB];
     __shared__ float s_code[256];
     constexpr bool kNeedCode = KA >= kQuant4 || KB >= kQuant4 || EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8;
     if (kNeedCode) {
@@ -301,22 +320,22 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     const int frag_row = lane & 31, frag_k = lane >> 5;
     for (int t = 0; t < n_tiles; ++t) {
         const int cur = t & 1;
-        const float *pa = s_a[cur] + (wm + frag_row) * LDS_STRIDE + frag_k;
-        const float *pb = s_b[cur] + (wn + frag_row) * LDS_STRIDE + frag_k;
+        const float *pa = s_a[cur] + frag_k * LDA + wm + frag_row;
+        const float *pb = s_b[cur] + frag_k * LDB + wn + frag_row;
         // fragments for step ks+1 are read from LDS before the MFMAs of step ks are issued
         float fa[2][MI], fb[2][NI];
 #pragma unroll
-        for (int i = 0; i < MI; ++i) fa[0][i] = pa[i * 32 * LDS_STRIDE];
+        for (int i = 0; i < MI; ++i) fa[0][i] = pa[i * 32];
 #pragma unroll
-        for (int j = 0; j < NI; ++j) fb[0][j] = pb[j * 32 * LDS_STRIDE];
+        for (int j = 0; j < NI; ++j) fb[0][j] = pb[j * 32];
 #pragma unroll
         for (int ks = 0; ks < BK / 2; ++ks) {
             const int now = ks & 1, nxt = now ^ 1;
             if (ks + 1 < BK / 2) {
 #pragma unroll
-                for (int i = 0; i < MI; ++i) fa[nxt][i] = pa[i * 32 * LDS_STRIDE + 2 * (ks + 1)];
+                for (int i = 0; i < MI; ++i) fa[nxt][i] = pa[i * 32 + 2 * (ks + 1) * LDA];
 #pragma unroll
-                for (int j = 0; j < NI; ++j) fb[nxt][j] = pb[j * 32 * LDS_STRIDE + 2 * (ks + 1)];
+                for (int j = 0; j < NI; ++j) fb[nxt][j] = pb[j * 32 + 2 * (ks + 1) * LDB];
             }
             if (ks == BK / 4 && t + 1 < n_tiles) {
                 la.commit(s_a[cur ^ 1]);
@@ -347,7 +366,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
                 float y = acc[i][j][r];
                 if (EPI == kAxpbyDense) {
                     const float *E = batch_ptr<float>(args.E, b);
-                    y = args.beta * E[(long long)row * args.lde + col] + args.alpha * y;
+                    y = args.beta * gload(E + (long long)row * args.lde + col) + args.alpha * y;
                 } else if (EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8) {
                     const float e = dequant_element<EPI == kAxpbyQuant4 ? 4 : 8>(
                         batch_ptr<uint8_t>(args.Eq.codes, b), batch_ptr<float>(args.Eq.absmax, b),
@@ -359,9 +378,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
                     const float eye = row == col ? 1.0f : 0.0f;
                     local_err = fmaxf(local_err, fabsf(y - eye));
                     float *T = const_cast<float *>(batch_ptr<float>(args.T, b));
-                    T[(long long)row * args.ldt + col] = (1.0f - args.newton_w) * eye + args.newton_w * y;
+                    gstore(T + (long long)row * args.ldt + col, (1.0f - args.newton_w) * eye + args.newton_w * y);
                 }
-                C[(long long)row * args.ldc + col] = y;
+                gstore(C + (long long)row * args.ldc + col, y);
             }
         }
     if (EPI == kNewton) {
