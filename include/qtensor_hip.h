@@ -161,6 +161,9 @@ typedef struct {
         float *err;             /* NEWTON: err[b] = max(err[b], max |A B - I|); caller zeroes   */
         const int *skip;        /* optional device array: skip[b] != 0 leaves entry b untouched */
         const float *code;      /* code table of the quantized operands / addend               */
+        int symmetric;          /* != 0: A B is known to be symmetric (M == N, dense operands): only the tiles
+                                 * on and above the diagonal are multiplied out and every off-diagonal
+                                 * tile is also stored mirrored; an addend is read at the mirrored place   */
     } args;
 } qtensor_gemm_desc;
 

@@ -56,6 +56,8 @@ struct GemmArgs {
     float *err;                   // kNewton: err[b] = max |acc - I| (must be zeroed by the caller)
     const int *skip;              // optional: skip[b] != 0 -> this batch entry is left untouched
     const float *code;            // code table for quantized operands / addend
+    int symmetric;                // != 0: the product is symmetric (M == N); only tiles on or above the
+                                  // diagonal are computed and every off-diagonal tile is also written mirrored
 };
 
 namespace {
@@ -79,7 +81,13 @@ __device__ __forceinline__ uint2 gload_u32x2(const void *p) {
     return make_uint2(v.x, v.y);
 }
 __device__ __forceinline__ uint32_t gload_u8(const uint8_t *p) { return *(const QT_GLOBAL uint8_t *)p; }
+__device__ __forceinline__ uint32_t gload_u16(const void *p) { return *(const QT_GLOBAL uint16_t *)p; }
 __device__ __forceinline__ void gstore(float *p, float v) { *(QT_GLOBAL float *)p = v; }
+__device__ __forceinline__ void gstore4(float *p, const float v[4]) {
+    qt_f32x4 x;
+    x.x = v[0]; x.y = v[1]; x.z = v[2]; x.w = v[3];
+    *(QT_GLOBAL qt_f32x4 *)p = x;
+}
 
 template <typename T>
 __device__ __forceinline__ const T *batch_ptr(const BatchPtr &p, int b) {
@@ -100,6 +108,25 @@ __device__ __forceinline__ float dequant_element(const uint8_t *codes, const flo
     else { const uint32_t byte = gload_u8(codes + (k >> 1)); id = (k & 1) ? (byte & 15u) : (byte >> 4); }
     const float a = gload(absmax + (k >> bs_shift));
     return a == 0.0f ? 0.0f : s_code[id] * a;
+}
+
+// Four consecutive off-diagonal elements (r, c0 .. c0+3), c0 a multiple of 4, of the same matrix.
+template <int BITS>
+__device__ __forceinline__ void dequant_four(const uint8_t *codes, const float *absmax, const float *s_code, int order,
+                                             int bs_shift, int r, int c0, float out[4]) {
+    const long long k = (long long)r * order + c0;
+    uint32_t id[4];
+    if (BITS == 8) {
+        const uint32_t w = gload_u32(codes + k);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) id[e] = (w >> (8 * e)) & 255u;
+    } else {
+        const uint32_t w = gload_u16(codes + (k >> 1));
+        id[0] = (w >> 4) & 15u; id[1] = w & 15u; id[2] = (w >> 12) & 15u; id[3] = (w >> 8) & 15u;
+    }
+    const float a = gload(absmax + (k >> bs_shift));
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out[e] = a == 0.0f ? 0.0f : s_code[id[e]] * a;
 }
 
 // ---- tile loaders: global -> registers -> LDS ([k][row], row stride rows + LDS_PAD) -------------
@@ -260,10 +287,20 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     const uint32_t die = blockIdx.x % kDies, slot = blockIdx.x / kDies;
     const uint32_t per = total / kDies, extra = total % kDies;
     uint32_t id = die * per + min(die, extra) + slot;
-    const int tile_n = id % tiles_n;
-    id /= tiles_n;
-    const int tile_m = id % tiles_m;
-    const int b = id / tiles_m;
+    int tile_m, tile_n, b;
+    if (args.symmetric) {                  // row-major walk over the tiles on and above the diagonal
+        const uint32_t upper = (uint32_t)tiles_n * (tiles_n + 1) / 2;
+        b = id / upper;
+        uint32_t rest = id % upper, width = tiles_n;
+        tile_m = 0;
+        while (rest >= width) { rest -= width; --width; ++tile_m; }
+        tile_n = tile_m + rest;
+    } else {
+        tile_n = id % tiles_n;
+        id /= tiles_n;
+        tile_m = id % tiles_m;
+        b = id / tiles_m;
+    }
     if (args.skip != nullptr && args.skip[b] != 0) return;
 
     constexpr int LDA = BM + LDS_PAD, LDB = BN + LDS_PAD;
@@ -353,6 +390,19 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
 
     // ---- epilogue: accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
     float *C = const_cast<float *>(batch_ptr<float>(args.C, b));
+    float *T = EPI == kNewton ? const_cast<float *>(batch_ptr<float>(args.T, b)) : nullptr;
+    const float *E = EPI == kAxpbyDense ? batch_ptr<float>(args.E, b) : nullptr;
+    constexpr bool kQuantAddend = EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8;
+    constexpr int EBITS = EPI == kAxpbyQuant8 ? 8 : 4;
+    const uint8_t *e_codes = kQuantAddend ? batch_ptr<uint8_t>(args.Eq.codes, b) : nullptr;
+    const float *e_absmax = kQuantAddend ? batch_ptr<float>(args.Eq.absmax, b) : nullptr;
+    const float *e_diag = kQuantAddend && has_ptr(args.Eq.diag) ? batch_ptr<float>(args.Eq.diag, b) : nullptr;
+    // an off-diagonal tile of a symmetric product also provides its mirror image; the addend is
+    // read at the mirrored position, so an addend that is not exactly symmetric is honoured
+    const bool mirror = args.symmetric != 0 && tile_n != tile_m;
+    const bool mirror_vec = (args.M & 3) == 0 && (args.ldc & 3) == 0 && is_aligned16(C) &&
+                            (EPI != kNewton || ((args.ldt & 3) == 0 && is_aligned16(T))) &&
+                            (EPI != kAxpbyDense || ((args.lde & 3) == 0 && is_aligned16(E)));
     float local_err = 0.0f;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
@@ -360,27 +410,62 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
         for (int j = 0; j < NI; ++j) {
             const int col = n0 + wn + j * 32 + (lane & 31);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (row >= args.M || col >= args.N) continue;
-                float y = acc[i][j][r];
-                if (EPI == kAxpbyDense) {
-                    const float *E = batch_ptr<float>(args.E, b);
-                    y = args.beta * gload(E + (long long)row * args.lde + col) + args.alpha * y;
-                } else if (EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8) {
-                    const float e = dequant_element<EPI == kAxpbyQuant4 ? 4 : 8>(
-                        batch_ptr<uint8_t>(args.Eq.codes, b), batch_ptr<float>(args.Eq.absmax, b),
-                        has_ptr(args.Eq.diag) ? batch_ptr<float>(args.Eq.diag, b) : nullptr, s_code, args.Eq.order,
-                        args.Eq.bs_shift, row, col);
-                    // same two roundings as tensor.mul_(beta).add_(S, alpha=1-beta)
-                    y = __builtin_fmaf(args.alpha, y, args.beta * e);
-                } else if (EPI == kNewton) {
-                    const float eye = row == col ? 1.0f : 0.0f;
-                    local_err = fmaxf(local_err, fabsf(y - eye));
-                    float *T = const_cast<float *>(batch_ptr<float>(args.T, b));
-                    gstore(T + (long long)row * args.ldt + col, (1.0f - args.newton_w) * eye + args.newton_w * y);
+            for (int rq = 0; rq < 4; ++rq) {
+                const int row4 = m0 + wm + i * 32 + 8 * rq + 4 * (lane >> 5);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int row = row4 + q;
+                    if (row >= args.M || col >= args.N) continue;
+                    float y = acc[i][j][4 * rq + q];
+                    if (EPI == kAxpbyDense) {
+                        y = args.beta * gload(E + (long long)row * args.lde + col) + args.alpha * y;
+                    } else if (kQuantAddend) {
+                        const float e = dequant_element<EBITS>(e_codes, e_absmax, e_diag, s_code, args.Eq.order,
+                                                               args.Eq.bs_shift, row, col);
+                        // same two roundings as tensor.mul_(beta).add_(S, alpha=1-beta)
+                        y = __builtin_fmaf(args.alpha, y, args.beta * e);
+                    } else if (EPI == kNewton) {
+                        const float eye = row == col ? 1.0f : 0.0f;
+                        local_err = fmaxf(local_err, fabsf(y - eye));
+                        gstore(T + (long long)row * args.ldt + col, (1.0f - args.newton_w) * eye + args.newton_w * y);
+                    }
+                    gstore(C + (long long)row * args.ldc + col, y);
                 }
-                gstore(C + (long long)row * args.ldc + col, y);
+                if (!mirror || col >= args.N || row4 >= args.M) continue;
+                // mirrored: elements (col, row4 .. row4+3), never on the diagonal
+                float y[4], e[4] = {0.f, 0.f, 0.f, 0.f};
+                const bool whole = mirror_vec;                  // M % 4 == 0: row4 + 3 < M
+                if (EPI == kAxpbyDense) {
+                    if (whole) { const float4 x = gload4(E + (long long)col * args.lde + row4); e[0] = x.x; e[1] = x.y; e[2] = x.z; e[3] = x.w; }
+                    else
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) if (row4 + q < args.M) e[q] = gload(E + (long long)col * args.lde + row4 + q);
+                } else if (kQuantAddend) {
+                    // flat quantized layout: the order is a multiple of 64, so the four codes share a segment
+                    dequant_four<EBITS>(e_codes, e_absmax, s_code, args.Eq.order, args.Eq.bs_shift, col, row4, e);
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float a = acc[i][j][4 * rq + q];
+                    if (EPI == kAxpbyDense) y[q] = args.beta * e[q] + args.alpha * a;
+                    else if (kQuantAddend) y[q] = __builtin_fmaf(args.alpha, a, args.beta * e[q]);
+                    else y[q] = a;
+                }
+                float *cm = C + (long long)col * args.ldc + row4;
+                if (whole) gstore4(cm, y);
+                else
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) if (row4 + q < args.M) gstore(cm + q, y[q]);
+                if (EPI == kNewton) {
+                    float t[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) t[q] = args.newton_w * y[q];
+                    float *tm = T + (long long)col * args.ldt + row4;
+                    if (whole) gstore4(tm, t);
+                    else
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) if (row4 + q < args.M) gstore(tm + q, t[q]);
+                }
             }
         }
     if (EPI == kNewton) {
@@ -392,7 +477,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
 
 template <int BM, int BN, int KA, int KB, int EPI>
 void launch_gemm(const GemmArgs &a, int batch, hipStream_t stream) {
-    const long long blocks = (long long)((a.N + BN - 1) / BN) * ((a.M + BM - 1) / BM) * batch;
+    const long long tn = (a.N + BN - 1) / BN, tm = (a.M + BM - 1) / BM;
+    if (a.symmetric && BM != BN) { set_error(kBadArgument, "gemm: symmetric products need square tiles"); return; }
+    const long long blocks = (a.symmetric ? tn * (tn + 1) / 2 : tn * tm) * batch;
     if (blocks > 0x7fffffffLL) { set_error(kBadArgument, "gemm: too many tiles (%lld)", blocks); return; }
     hipLaunchKernelGGL((gemm_kernel<BM, BN, KA, KB, EPI>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
 }
@@ -459,12 +546,18 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
         if (a.Eq.order != d->M || d->M != d->N) { set_error(kBadArgument, "gemm: quantized addend must be M x N square of its order"); return; }
     }
     if (ep == kNewton && (!has_host_ptr(a.T) || a.ldt < d->N || !a.err)) { set_error(kBadArgument, "gemm: Newton epilogue needs T and err"); return; }
+    a.symmetric = a.symmetric != 0;
+    if (a.symmetric && (d->M != d->N || ka >= kQuant4 || kb >= kQuant4)) {
+        set_error(kBadArgument, "gemm: symmetric products need M == N and dense operands");
+        return;
+    }
     const bool need_code = ka >= kQuant4 || kb >= kQuant4 || ep == kAxpbyQuant4 || ep == kAxpbyQuant8;
     if (need_code && !a.code) { set_error(kNullPointer, "gemm: code table missing"); return; }
 
     // 128 x 128 tiles when that still gives every compute unit work, else 64 x 64 (quantized
     // operands always use a 128-wide tile on their side).
-    const long long big_tiles = (long long)((d->M + 127) / 128) * ((d->N + 127) / 128) * d->batch;
+    const long long t128 = (d->N + 127) / 128;
+    const long long big_tiles = (a.symmetric ? t128 * (t128 + 1) / 2 : (long long)((d->M + 127) / 128) * t128) * d->batch;
     const bool big = big_tiles >= compute_units();
     const int combo = ka * 100 + kb * 10 + ep;
 #define QT_GEMM_CASE(KA, KB, EP)                                                                             \

@@ -148,7 +148,8 @@ class ShampooBank:
             for side in (0, 1):
                 seg = self._segment(self.stats, g, side)
                 out = self.scratch[seg.order][:len(g)]
-                X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, out=out)
+                X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, out=out,
+                       symmetric=True)
                 X.quantize_stack(out, seg)
 
     @torch.no_grad()

@@ -113,9 +113,14 @@ def PowerIterBatched(mats, error_tolerance=1e-6, num_iters=10, v0=None):
 
 @torch.no_grad()
 def ComputePowerBatched(mats, p=4, iter_count=10, error_tolerance=1e-6, ridge_epsilon=1e-6, v0=None,
-                        out: Optional[torch.Tensor] = None):
+                        out: Optional[torch.Tensor] = None, symmetric: bool = False):
     """ComputePower for a GPU stack mats [B, n, n] (fp32, overwritten with mats + ridge like the
-    reference does for its argument).  Returns [B, n, n]."""
+    reference does for its argument).  Returns [B, n, n].
+
+    symmetric: the caller guarantees mats[b] == mats[b].T bit for bit.  All iterates are then
+    symmetric in exact arithmetic and only their upper halves are multiplied out (half the work).
+    A dequantized low-bit statistic is NOT symmetric (every row segment has its own scale), and
+    the reference iterates on it as it is: leave the flag off for those."""
     from qtensor import fused as X
 
     if not mats.is_cuda or mats.dtype != torch.float32 or mats.dim() != 3:
@@ -156,16 +161,17 @@ def ComputePowerBatched(mats, p=4, iter_count=10, error_tolerance=1e-6, ridge_ep
         oth = lambda tab: torch.where(side, tab[0], tab[1])                   # noqa: E731
         Rc, Ro, Mc, Mo, Tc, To = cur(R_ptr), oth(R_ptr), cur(M_ptr), oth(M_ptr), cur(T_ptr), oth(T_ptr)
         shape = (B, n, n)
-        X.gemm(X.PtrList(Rc, shape), X.PtrList(Tc, shape), out=X.PtrList(Ro, shape), skip=skip)     # candidate root
+        X.gemm(X.PtrList(Rc, shape), X.PtrList(Tc, shape), out=X.PtrList(Ro, shape), skip=skip,
+               symmetric=symmetric)                                          # candidate root
         power = X.PtrList(Tc, shape)                                         # T^p by repeated squaring
         done_p = 1
         while done_p < p:
             dst = Tp if power is T2 else T2
-            X.gemm(power, power, out=dst, skip=skip)
+            X.gemm(power, power, out=dst, skip=skip, symmetric=symmetric)
             power, done_p = dst, done_p * 2
         new_err = torch.zeros(B, device=dev)
         X.gemm(power, X.PtrList(Mc, shape), out=X.PtrList(Mo, shape), newton=(X.PtrList(To, shape), w, new_err),
-               skip=skip)
+               skip=skip, symmetric=symmetric)
         accept = (~done) & ~(new_err > err * 1.2)
         side = side ^ accept
         err = torch.where(accept, new_err, err)

@@ -37,7 +37,7 @@ class GemmArgs(ct.Structure):
                 ("Eq", QuantRef),
                 ("T", BatchPtr), ("ldt", ct.c_int),
                 ("newton_w", ct.c_float),
-                ("err", ct.c_void_p), ("skip", ct.c_void_p), ("code", ct.c_void_p)]
+                ("err", ct.c_void_p), ("skip", ct.c_void_p), ("code", ct.c_void_p), ("symmetric", ct.c_int)]
 
 
 class GemmDesc(ct.Structure):
@@ -122,7 +122,7 @@ def _launch(desc: GemmDesc, device: torch.device) -> None:
 
 
 def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, alpha=1.0, beta=0.0,
-         addend=None, newton=None, skip: Optional[Tensor] = None) -> Tensor:
+         addend=None, newton=None, skip: Optional[Tensor] = None, symmetric: bool = False) -> Tensor:
     """out[b] = epilogue(op(A[b]) @ op(B[b])).
 
     A, B: fp32 tensors ([m,k] / [batch,m,k]; with trans_x the stored matrix is the transpose) or a
@@ -130,7 +130,10 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
     addend: None, a dense tensor E or a `Quantized` E: out = beta*E + alpha*product.
     newton: None or (T_out, w, err): also writes T_out = (1-w) I + w*product and folds
     max|product - I| into err[b] (fp32 [batch], zeroed by the caller).
-    skip: optional int32 [batch]; entries with a nonzero flag are not touched."""
+    skip: optional int32 [batch]; entries with a nonzero flag are not touched.
+    symmetric: the caller knows the product to be symmetric (a Gram matrix, a product of commuting
+    symmetric matrices): only the tiles on and above the diagonal are multiplied out and mirrored,
+    which halves the work; the result is then symmetric bit for bit outside the diagonal tiles."""
     d = GemmDesc()
     a = d.args
     dev = None
@@ -199,6 +202,10 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
         a.skip = skip.data_ptr()
     if code is not None:
         a.code = code.data_ptr()
+    if symmetric:
+        if m != n or isinstance(A, Quantized) or isinstance(B, Quantized):
+            raise ValueError("symmetric products are square with dense operands")
+        a.symmetric = 1
     _launch(d, dev)
     return out
 
@@ -214,8 +221,8 @@ def gram(G: Tensor, axis: int, *, stat=None, beta=0.0, alpha=1.0, out: Optional[
     """axis 0: G @ G.T, axis 1: G.T @ G; with `stat` (dense or `Quantized`) returns
     beta * stat + alpha * that product, i.e. the Shampoo statistics update in one launch."""
     if axis == 0:
-        return gemm(G, G, trans_b=True, addend=stat, alpha=alpha, beta=beta, out=out)
-    return gemm(G, G, trans_a=True, addend=stat, alpha=alpha, beta=beta, out=out)
+        return gemm(G, G, trans_b=True, addend=stat, alpha=alpha, beta=beta, out=out, symmetric=True)
+    return gemm(G, G, trans_a=True, addend=stat, alpha=alpha, beta=beta, out=out, symmetric=True)
 
 
 # --------------------------------------------------------------------------- stacks of matrices

@@ -115,7 +115,7 @@ def test_config3_preconditioned_gradient(mods, code_maps):
         assert rel_err(got, (Lg @ G.cuda() @ Rg).cpu()) <= TOL
 
 
-@pytest.mark.parametrize("m,n", [(256, 512), (768, 1024), (100, 260), (1024, 768)])
+@pytest.mark.parametrize("m,n", [(256, 512), (768, 1024), (100, 260), (1024, 768), (101, 330), (2, 131)])
 def test_gram_and_statistics_update(mods, code_maps, m, n):
     F, X = mods
     g = torch.Generator().manual_seed(m + n)
@@ -153,6 +153,48 @@ def test_newton_epilogue_and_skip_flags(mods):
         assert rel_err(T[b], (1 - w) * eye + w * want[b]) <= TOL
         assert abs(float(err[b]) - float((want[b] - eye).abs().max())) <= 1e-5
     assert bool((out[1] == 7.0).all()) and bool((T[1] == 7.0).all()) and float(err[1]) == 0.0
+
+
+@pytest.mark.parametrize("n,batch", [(192, 3), (1024, 2), (150, 2), (77, 1)])
+def test_symmetric_products_compute_the_upper_half_and_mirror_it(mods, n, batch):
+    """Products of commuting symmetric matrices (the Newton iterates of a symmetric statistic)."""
+    _, X = mods
+    g = torch.Generator().manual_seed(n)
+    S = torch.randn(batch, n, n, generator=g) / n ** 0.5
+    S = (S + S.transpose(1, 2)) / 2
+    P = (S @ S + 0.5 * S).contiguous()                           # a polynomial in S: commutes with S
+    P = ((P + P.transpose(1, 2)) / 2).contiguous()
+    want = S.double() @ P.double()
+    w = -0.25
+    out = torch.full((batch, n, n), 7.0, device="cuda")
+    T = torch.full((batch, n, n), 7.0, device="cuda")
+    err = torch.zeros(batch, device="cuda")
+    skip = torch.zeros(batch, dtype=torch.int32, device="cuda")
+    skip[-1] = 1 if batch > 1 else 0
+    X.gemm(S.cuda(), P.cuda(), out=out, newton=(T, w, err), skip=skip, symmetric=True)
+    eye = torch.eye(n, dtype=torch.float64)
+    for b in range(batch):
+        if int(skip[b]):
+            assert bool((out[b] == 7.0).all()) and bool((T[b] == 7.0).all()) and float(err[b]) == 0.0
+            continue
+        # the float64 product is symmetric only up to the non-commutation left by rounding P
+        assert rel_err(out[b], (want[b] + want[b].T) / 2) <= TOL
+        assert rel_err(T[b], (1 - w) * eye + w * (want[b] + want[b].T) / 2) <= TOL
+        assert abs(float(err[b]) - float((want[b] - eye).abs().max())) <= 1e-5
+        big = 128 if (-(-n // 128)) * (-(-n // 128) + 1) // 2 * batch >= 256 else 64
+        tile = torch.arange(n) // big
+        off = tile[:, None] != tile[None, :]                    # outside the diagonal tiles: exact mirror
+        o = out[b].cpu()
+        assert torch.equal(o[off], o.T[off])
+    plain = X.gemm(S.cuda(), P.cuda())
+    sym = X.gemm(S.cuda(), P.cuda(), symmetric=True)
+    tile = torch.arange(n) // 64
+    upper_tiles = tile[:, None] <= tile[None, :]
+    # on and above the diagonal tiles both modes run the same arithmetic
+    if n <= 192:
+        assert torch.equal(plain.cpu()[:, upper_tiles], sym.cpu()[:, upper_tiles])
+    with pytest.raises(ValueError):
+        X.gemm(torch.zeros(64, 32, device="cuda"), torch.zeros(32, 48, device="cuda"), symmetric=True)
 
 
 def test_argument_errors(mods, code_maps):
