@@ -171,6 +171,33 @@ typedef struct {
  * (DENSE_T, DENSE, STORE|AXPBY_*), (DENSE, DENSE, STORE|AXPBY_DENSE|NEWTON); anything else is an error. */
 void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
 
+/* ---- the elementwise end of an optimizer step for all parameters at once -------------------------
+ * Replaces the per-parameter torch calls of the reference's step():
+ *   grafting   direction.mul_(grad.norm() / (direction.norm() + 1e-12))   optimizers/shampoo1.py:421, shampoo2.py:453
+ *   AdamW      p.mul_(1 - lr*wd); exp_avg / exp_avg_sq update; p.addcdiv_  optimizers/shampoo1.py:405-427, shampoo2.py:446-468
+ *   SGD        weight decay, momentum buffer, (Nesterov) update             optimizers/shampoo1.py:310-331, shampoo2.py:346-367
+ * table: device array with one row per tensor; chunk_tensor: device array, row index of the tensor
+ * that owns chunk c; a tensor of n elements owns ceil(n / qtensor_hip_tail_chunk()) consecutive
+ * chunks starting at first_chunk.  partial: device scratch of 2 * n_chunks floats (only used when
+ * graft != 0).  Rows with flags bit 0 set get dir rescaled to the norm of grad (dir itself is not
+ * written); the others use dir as it is.  All tensors fp32. */
+typedef struct {
+    float *param;
+    const float *dir;           /* preconditioned gradient, or the gradient itself            */
+    const float *grad;          /* read only for grafted rows                                 */
+    float *m;                   /* AdamW: exp_avg; SGD: momentum buffer                       */
+    float *v;                   /* AdamW: exp_avg_sq; SGD: unused                             */
+    long long n;
+    long long first_chunk;
+    long long flags;            /* bit 0: graft                                               */
+} qtensor_tail_tensor;
+int qtensor_hip_tail_chunk(void);
+void qtensor_hip_adamw_tail(const qtensor_tail_tensor *table, const int *chunk_tensor, int n_chunks, float *partial, int graft,
+                            double lr, double beta1, double beta2, double eps, double weight_decay, long long step,
+                            qtensor_stream_t stream);
+void qtensor_hip_sgd_tail(const qtensor_tail_tensor *table, const int *chunk_tensor, int n_chunks, float *partial, int graft,
+                          double lr, double momentum, double weight_decay, int nesterov, qtensor_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,7 +77,6 @@ class ShampooAdamW(ShampooAdamWBase):
 
 def fused_step(opt, group, update):
     """One optimizer step of a parameter group with the preconditioner work batched."""
-    import math  # noqa: F401
     from optimizers.engine import ShampooBank
 
     params = [p for p in group['params'] if p.grad is not None]
@@ -98,32 +97,47 @@ def fused_step(opt, group, update):
                 state['preconditioner'] = opt._make_preconditioner(p, group)
     entry['step'] += 1
     step, bank, banked = entry['step'], entry['bank'], entry['banked']
-    others = [p for p in params if id(p) not in entry['ids']]
     for p in params:
         opt.state[p]['step'] = step
-    if update is _adamw_update:
-        torch._foreach_mul_(params, 1 - group['lr'] * group['weight_decay'])
-    bgrads = [p.grad.contiguous() for p in banked]
-    directions = {}
+    grads = {id(p): p.grad.contiguous() for p in params}
+    directions, grafted = {}, set()
     if bank is not None:
+        bgrads = [grads[id(p)] for p in banked]
         if step % group['stat_compute_steps'] == 0:
             bank.add_statistics(bgrads)
         if step % group['prec_compute_steps'] == 0:
             bank.compute_preconditioners()
         if step >= group['start_prec_step'] and bank.is_active():
-            outs = bank.preconditioned_grads(bgrads)
-            gnorm = torch._foreach_norm(bgrads)
-            onorm = torch._foreach_norm(outs)
-            torch._foreach_add_(onorm, 1e-12)
-            torch._foreach_div_(gnorm, onorm)
-            torch._foreach_mul_(outs, gnorm)                      # keep each gradient's norm
-            directions = {id(p): o for p, o in zip(banked, outs)}
-    for p in others:
-        directions[id(p)] = opt._shampoo_direction(p, p.grad, group, opt.state[p])
-    update(opt, group, params, [directions.get(id(p), p.grad) for p in params], step)
+            # the rescaling to each gradient's norm happens inside the fused update
+            directions = {id(p): o for p, o in zip(banked, bank.preconditioned_grads(bgrads))}
+            grafted = set(directions)
+    for p in params:
+        if id(p) not in entry['ids']:
+            directions[id(p)] = opt._shampoo_direction(p, grads[id(p)], group, opt.state[p])
+    update(opt, group, params, [directions.get(id(p), grads[id(p)]) for p in params], [grads[id(p)] for p in params],
+           [id(p) in grafted for p in params], step, entry)
 
 
-def _adamw_update(opt, group, params, dirs, step):
+def _fused_tail_ok(params, dirs):
+    return all(p.is_cuda and p.dtype == torch.float32 and p.is_contiguous() and d.dtype == torch.float32 and d.is_contiguous()
+               for p, d in zip(params, dirs))
+
+
+def _tail_plan(entry):
+    from optimizers.tail import TailPlan
+    if entry.get('tail') is None:
+        entry['tail'] = TailPlan()
+    return entry['tail']
+
+
+def _graft(dirs, grads, graft):
+    # keep each gradient's norm (reference: shampoo1.py:421)
+    for d, g, f in zip(dirs, grads, graft):
+        if f:
+            d.mul_(g.norm() / (d.norm() + 1e-12))
+
+
+def _adamw_update(opt, group, params, dirs, grads, graft, step, entry):
     import math
     for p in params:
         state = opt.state[p]
@@ -133,6 +147,12 @@ def _adamw_update(opt, group, params, dirs, step):
     m = [opt.state[p]['exp_avg'] for p in params]
     v = [opt.state[p]['exp_avg_sq'] for p in params]
     beta1, beta2 = group['betas']
+    if _fused_tail_ok(params, dirs):
+        plan = _tail_plan(entry)
+        plan.adamw(params, dirs, grads, m, v, graft, group['lr'], (beta1, beta2), group['eps'], group['weight_decay'], step)
+        return
+    _graft(dirs, grads, graft)
+    torch._foreach_mul_(params, 1 - group['lr'] * group['weight_decay'])
     torch._foreach_mul_(m, beta1)
     torch._foreach_add_(m, dirs, alpha=1 - beta1)
     torch._foreach_mul_(v, beta2)
@@ -143,14 +163,19 @@ def _adamw_update(opt, group, params, dirs, step):
     torch._foreach_addcdiv_(params, m, denom, value=-group['lr'] / (1 - beta1 ** step))
 
 
-def _sgd_update(opt, group, params, dirs, step):
+def _sgd_update(opt, group, params, dirs, grads, graft, step, entry):
     for p in params:
         state = opt.state[p]
         if 'momentum' not in state:
             state['momentum'] = torch.zeros_like(p, memory_format=torch.preserve_format)
+    bufs = [opt.state[p]['momentum'] for p in params]
+    if _fused_tail_ok(params, dirs):
+        plan = _tail_plan(entry)
+        plan.sgd(params, dirs, grads, bufs, graft, group['lr'], group['momentum'], group['weight_decay'], group['nesterov'])
+        return
+    _graft(dirs, grads, graft)
     if group['weight_decay'] != 0.0:
         torch._foreach_add_(dirs, params, alpha=group['weight_decay'])
-    bufs = [opt.state[p]['momentum'] for p in params]
     torch._foreach_mul_(bufs, group['momentum'])
     torch._foreach_add_(bufs, dirs)
     if group['nesterov']:

@@ -1,0 +1,68 @@
+"""The elementwise end of an optimizer step (grafting + AdamW / SGD update) for all parameters of
+a group in two launches of libqtensor_hip.so instead of a dozen torch kernels per parameter.
+
+Arithmetic of the reference's step(): optimizers/shampoo1.py:310-331 (SGD), :405-427 (AdamW)
+and the same lines of shampoo2.py.
+"""
+import ctypes as ct
+
+import torch
+
+import qtensor.functional as F
+
+if F.lib is not None:
+    F.lib.qtensor_hip_tail_chunk.restype = ct.c_int
+    F.lib.qtensor_hip_tail_chunk.argtypes = []
+    F.lib.qtensor_hip_adamw_tail.restype = None
+    F.lib.qtensor_hip_adamw_tail.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_void_p, ct.c_int, ct.c_double, ct.c_double,
+                                             ct.c_double, ct.c_double, ct.c_double, ct.c_longlong, ct.c_void_p]
+    F.lib.qtensor_hip_sgd_tail.restype = None
+    F.lib.qtensor_hip_sgd_tail.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_void_p, ct.c_int, ct.c_double, ct.c_double,
+                                           ct.c_double, ct.c_int, ct.c_void_p]
+
+
+class TailPlan:
+    """Device-side table of (param, direction, grad, moment buffers) rows and the chunk map the
+    kernels walk.  Rebuilt only when a buffer has moved."""
+
+    def __init__(self):
+        if F.lib is None:
+            raise RuntimeError("libqtensor_hip.so is not available")
+        self.chunk = F.lib.qtensor_hip_tail_chunk()
+        self.key = None
+        self.keep = None
+
+    def _prepare(self, params, dirs, grads, m, v, graft):
+        key = tuple((p.data_ptr(), d.data_ptr(), g.data_ptr(), a.data_ptr(), 0 if b is None else b.data_ptr(), bool(f))
+                    for p, d, g, a, b, f in zip(params, dirs, grads, m, v, graft))
+        if key == self.key:
+            return
+        rows, owner, first = [], [], 0
+        for i, (p, d, g, a, b, f) in enumerate(zip(params, dirs, grads, m, v, graft)):
+            tensors = [p, d, a] + ([g] if f else []) + ([] if b is None else [b])
+            for t in tensors:
+                if not t.is_cuda or t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != p.numel():
+                    raise ValueError("the fused update takes contiguous fp32 GPU tensors of equal size per parameter")
+            chunks = -(-p.numel() // self.chunk)
+            rows.append([p.data_ptr(), d.data_ptr(), g.data_ptr() if f else 0, a.data_ptr(), 0 if b is None else b.data_ptr(),
+                         p.numel(), first, 1 if f else 0])
+            owner += [i] * chunks
+            first += chunks
+        dev = params[0].device
+        self.table = torch.tensor(rows, dtype=torch.int64).to(dev)
+        self.owner = torch.tensor(owner, dtype=torch.int32).to(dev)
+        self.partial = torch.empty(2 * max(first, 1), dtype=torch.float32, device=dev)
+        self.n_chunks = first
+        self.any_graft = any(graft)
+        self.key = key
+        self.keep = (list(params), list(dirs), list(grads), list(m), list(v))     # the table holds raw addresses
+
+    def adamw(self, params, dirs, grads, exp_avg, exp_avg_sq, graft, lr, betas, eps, weight_decay, step):
+        self._prepare(params, dirs, grads, exp_avg, exp_avg_sq, graft)
+        F._call(F.lib.qtensor_hip_adamw_tail, params[0].device, self.table.data_ptr(), self.owner.data_ptr(), self.n_chunks,
+                self.partial.data_ptr(), int(self.any_graft), lr, betas[0], betas[1], eps, weight_decay, step)
+
+    def sgd(self, params, dirs, grads, momentum_bufs, graft, lr, momentum, weight_decay, nesterov):
+        self._prepare(params, dirs, grads, momentum_bufs, [None] * len(params), graft)
+        F._call(F.lib.qtensor_hip_sgd_tail, params[0].device, self.table.data_ptr(), self.owner.data_ptr(), self.n_chunks,
+                self.partial.data_ptr(), int(self.any_graft), lr, momentum, weight_decay, int(bool(nesterov)))

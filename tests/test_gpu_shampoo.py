@@ -152,3 +152,61 @@ def test_fused_optimizer_matches_per_parameter_optimizer(setup, which, monkeypat
     # update (Adam's normalisation magnifies the rounding-level differences of the inverse roots)
     for a, b in zip(*finals):
         assert rel(a, b) <= 2e-4
+
+
+@pytest.mark.parametrize("which", ["adamw", "sgd", "sgd-nesterov"])
+def test_fused_update_kernels_match_the_torch_update_rules(which):
+    """Grafting + AdamW / SGD update of all tensors in two launches against the reference's torch
+    calls (shampoo1.py:310-331, 405-427) on ragged, unaligned and multi-chunk tensors."""
+    import math
+    from optimizers.tail import TailPlan
+    g = torch.Generator().manual_seed(11)
+    sizes = [5, 16384, 16385, 100003, 3 * 16384 + 2, 1]
+    graft = [True, True, False, True, True, True]
+    pool = torch.randn(sum(sizes) + 64, generator=g).cuda()
+
+    def carve(unaligned):
+        out, at = [], 1 if unaligned else 0
+        for n in sizes:
+            out.append(pool[at:at + n].clone() if not unaligned else torch.randn(n + 1, generator=g).cuda()[1:])
+            at += n
+        return out
+
+    for unaligned in (False, True):
+        params, dirs, grads = carve(unaligned), carve(unaligned), carve(unaligned)
+        m = [0.1 * torch.randn(n, generator=g).cuda() for n in sizes]
+        v = [0.01 * torch.rand(n, generator=g).cuda() for n in sizes]
+        want_p, want_m, want_v = [t.clone() for t in params], [t.clone() for t in m], [t.clone() for t in v]
+        lr, wd, step = 1e-2, 0.05, 3
+        plan = TailPlan()
+        for p, d, gr, a, b, f in zip(want_p, dirs, grads, want_m, want_v, graft):
+            d = d.clone()
+            if f:
+                d.mul_(gr.norm() / (d.norm() + 1e-12))
+            if which == "adamw":
+                beta1, beta2, eps = 0.9, 0.999, 1e-8
+                p.mul_(1 - lr * wd)
+                a.mul_(beta1).add_(d, alpha=1 - beta1)
+                b.mul_(beta2).addcmul_(d, d, value=1 - beta2)
+                denom = (b.sqrt() / math.sqrt(1 - beta2 ** step)).add_(eps)
+                p.addcdiv_(a, denom, value=-lr / (1 - beta1 ** step))
+            else:
+                d.add_(p, alpha=wd)
+                buf = a.mul_(0.9).add_(d)
+                p.add_(d.add(buf, alpha=0.9) if which == "sgd-nesterov" else buf, alpha=-lr)
+        before = [d.clone() for d in dirs]
+        if which == "adamw":
+            plan.adamw(params, dirs, grads, m, v, graft, lr, (0.9, 0.999), 1e-8, wd, step)
+        else:
+            plan.sgd(params, dirs, grads, m, graft, lr, 0.9, wd, which == "sgd-nesterov")
+        for got, want in zip(params + m + (v if which == "adamw" else []), want_p + want_m + (want_v if which == "adamw" else [])):
+            assert rel(got, want) <= 2e-6
+        assert all(torch.equal(a, b) for a, b in zip(dirs, before))      # directions are read only
+        # the plan is reused while no buffer moves, and rebuilt when one does
+        table = plan.table
+        (plan.adamw(params, dirs, grads, m, v, graft, lr, (0.9, 0.999), 1e-8, wd, step + 1) if which == "adamw"
+         else plan.sgd(params, dirs, grads, m, graft, lr, 0.9, wd, False))
+        assert plan.table is table
+    with pytest.raises(ValueError):
+        TailPlan().sgd([torch.zeros(4, device="cuda")], [torch.zeros(4)], [torch.zeros(4, device="cuda")],
+                       [torch.zeros(4, device="cuda")], [False], 0.1, 0.9, 0.0, False)
