@@ -158,7 +158,7 @@ struct LoadKContig {
             v[i] = x;
         }
     }
-    __device__ __forceinline__ void commit(float *lds) const {
+    __device__ __forceinline__ void commit(float *lds, const float *) const {
         constexpr int LD = ROWS + LDS_PAD;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
@@ -195,7 +195,7 @@ struct LoadRowContig {
             v[i] = x;
         }
     }
-    __device__ __forceinline__ void commit(float *lds) const {
+    __device__ __forceinline__ void commit(float *lds, const float *) const {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const int f = threadIdx.x + i * 256;
@@ -212,14 +212,21 @@ template <int ROWS, int BITS, bool ALONG_K>
 struct LoadQuant {
     static constexpr int TOTAL = ROWS * BK / 8;              // 8-element groups in the tile
     static constexpr int GROUPS = (TOTAL + 255) / 256;       // per thread
-    float v[GROUPS][8];
+    // `fetch` only issues the global loads (packed codes, the segment maximum, the exact diagonal
+    // entry if the group crosses the diagonal); the table lookups wait until `commit`, one tile
+    // later, when the loads have long landed.
+    uint2 raw[GROUPS];
+    float amax[GROUPS];
+    float dval[GROUPS];
+    int dpos[GROUPS];                                        // element of the group on the diagonal, -1: none, -2: outside
     __device__ __forceinline__ bool active(int g) const { return (int)threadIdx.x + g * 256 < TOTAL; }
     __device__ __forceinline__ void locate(int g, int &mr, int &mc) const {
         const int f = threadIdx.x + g * 256;
-        if (ALONG_K) { mr = f >> 1; mc = (f & 1) << 3; }                    // tile row = matrix row, 2 groups per row
+        if (ALONG_K) { mr = f % ROWS; mc = (f / ROWS) << 3; }               // tile row = matrix row, 2 groups per row
         else { mr = f / (ROWS / 8); mc = (f % (ROWS / 8)) << 3; }           // tile k = matrix row
     }
     __device__ __forceinline__ void fetch(const QuantRef &q, int b, const float *s_code, int row0, int k0) {
+        (void)s_code;
         const uint8_t *codes = batch_ptr<uint8_t>(q.codes, b);
         const float *absmax = batch_ptr<float>(q.absmax, b);
         const float *diag = has_ptr(q.diag) ? batch_ptr<float>(q.diag, b) : nullptr;
@@ -230,47 +237,60 @@ struct LoadQuant {
             locate(g, tr, tc);
             const int mr = ALONG_K ? row0 + tr : k0 + tr;     // matrix row
             const int mc = ALONG_K ? k0 + tc : row0 + tc;     // first matrix column of the group
+            dpos[g] = -2;
             if (mr < q.order && mc < q.order) {               // order is a multiple of 64: whole group inside
                 const long long k = (long long)mr * q.order + mc;
-                const float a = gload(absmax + (k >> q.bs_shift));
-                uint32_t id[8];
-                if (BITS == 4) {
-                    const uint32_t w = gload_u32(codes + (k >> 1));
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t byte = (w >> (8 * e)) & 255u;
-                        id[2 * e] = byte >> 4;
-                        id[2 * e + 1] = byte & 15u;
-                    }
-                } else {
-                    const uint2 w = gload_u32x2(codes + k);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) { id[e] = (w.x >> (8 * e)) & 255u; id[4 + e] = (w.y >> (8 * e)) & 255u; }
-                }
-#pragma unroll
-                for (int e = 0; e < 8; ++e) v[g][e] = a == 0.0f ? 0.0f : s_code[id[e]] * a;
-                if (diag != nullptr && mr >= mc && mr < mc + 8) v[g][mr - mc] = gload(diag + mr);
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) v[g][e] = 0.0f;
+                amax[g] = gload(absmax + (k >> q.bs_shift));
+                if (BITS == 4) raw[g].x = gload_u32(codes + (k >> 1));
+                else raw[g] = gload_u32x2(codes + k);
+                dpos[g] = -1;
+                if (diag != nullptr && mr >= mc && mr < mc + 8) { dpos[g] = mr - mc; dval[g] = gload(diag + mr); }
             }
         }
     }
-    __device__ __forceinline__ void commit(float *lds) const {
+    __device__ __forceinline__ void expand(int g, const float *s_code, float v[8]) const {
+        if (dpos[g] == -2) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+            return;
+        }
+        uint32_t id[8];
+        if (BITS == 4) {
+            const uint32_t w = raw[g].x;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t byte = (w >> (8 * e)) & 255u;
+                id[2 * e] = byte >> 4;
+                id[2 * e + 1] = byte & 15u;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { id[e] = (raw[g].x >> (8 * e)) & 255u; id[4 + e] = (raw[g].y >> (8 * e)) & 255u; }
+        }
+        const float a = amax[g];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float x = a == 0.0f ? 0.0f : s_code[id[e]] * a;
+            v[e] = e == dpos[g] ? dval[g] : x;
+        }
+    }
+    __device__ __forceinline__ void commit(float *lds, const float *s_code) const {
 #pragma unroll
         for (int g = 0; g < GROUPS; ++g) {
             if (!active(g)) continue;
             int tr, tc;
             locate(g, tr, tc);
+            float v[8];
+            expand(g, s_code, v);
             constexpr int LD = ROWS + LDS_PAD;
             if (ALONG_K) {
-                float *d = lds + tc * LD + tr;
+                float *d = lds + tc * LD + tr;                // consecutive lanes: consecutive words
 #pragma unroll
-                for (int e = 0; e < 8; ++e) d[e * LD] = v[g][e];
+                for (int e = 0; e < 8; ++e) d[e * LD] = v[e];
             } else {
                 float4 *d = reinterpret_cast<float4 *>(lds + tr * LD + tc);
-                d[0] = make_float4(v[g][0], v[g][1], v[g][2], v[g][3]);
-                d[1] = make_float4(v[g][4], v[g][5], v[g][6], v[g][7]);
+                d[0] = make_float4(v[0], v[1], v[2], v[3]);
+                d[1] = make_float4(v[4], v[5], v[6], v[7]);
             }
         }
     }
@@ -350,8 +370,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     // the MFMA stream and the loads of tile t+2 are issued right after.  One barrier per tile.
     const int n_tiles = (args.K + BK - 1) / BK;
     fetch(0);
-    la.commit(s_a[0]);
-    lb.commit(s_b[0]);
+    la.commit(s_a[0], s_code);
+    lb.commit(s_b[0], s_code);
     if (n_tiles > 1) fetch(BK);
     __syncthreads();
     const int frag_row = lane & 31, frag_k = lane >> 5;
@@ -375,8 +395,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
                 for (int j = 0; j < NI; ++j) fb[nxt][j] = pb[j * 32 + 2 * (ks + 1) * LDB];
             }
             if (ks == BK / 4 && t + 1 < n_tiles) {
-                la.commit(s_a[cur ^ 1]);
-                lb.commit(s_b[cur ^ 1]);
+                la.commit(s_a[cur ^ 1], s_code);
+                lb.commit(s_b[cur ^ 1], s_code);
                 if (t + 2 < n_tiles) fetch((t + 2) * BK);
             }
 #pragma unroll

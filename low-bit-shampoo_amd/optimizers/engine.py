@@ -40,7 +40,7 @@ class _Group:
 
 class ShampooBank:
     def __init__(self, params, name2qmap, code, stat_decay=0.95, matrix_eps=1e-6, prec_maxorder=1200,
-                 prec_bits=4, min_lowbit_size=4096, quan_blocksize=64):
+                 prec_bits=4, min_lowbit_size=4096, quan_blocksize=64, streams=3):
         self.stat_decay, self.matrix_eps = stat_decay, matrix_eps
         self.bits, self.blocksize = prec_bits, quan_blocksize
         self.params = list(params)
@@ -71,20 +71,46 @@ class ShampooBank:
             for side, order in enumerate((g.bm, g.bn)):
                 g.slot[side] = (order, per_order[order])
                 per_order[order] += len(g)
-        self.stats, self.precs, self.scratch = {}, {}, {}
+        self.stats, self.precs = {}, {}
         for order, count in per_order.items():
             eye = torch.eye(order, device=self.device).expand(count, order, order)
             self.stats[order] = X.quantize_stack((matrix_eps * eye).contiguous(),
                                                  X.empty_quantized(count, order, quan_blocksize, prec_bits, self.code, True))
             self.precs[order] = X.quantize_stack(eye.contiguous(),
                                                  X.empty_quantized(count, order, quan_blocksize, prec_bits, self.code, True))
-            biggest = max(len(g) for g in self.groups for o in (g.bm, g.bn) if o == order)
-            self.scratch[order] = torch.empty(biggest, order, order, device=self.device)
+        for g in self.groups:       # fp32 landing areas of the updated statistics and of P_L G, per group
+            g.scratch = [torch.empty(len(g), o, o, device=self.device) for o in (g.bm, g.bn)]
+            g.half = torch.empty(len(g), g.bm, g.bn, device=self.device)
         self.outputs = [torch.empty(m, n, device=self.device) for m, n in self.shapes]
         for g in self.groups:
             g.out_ptrs = torch.tensor([self.outputs[pi].data_ptr() + 4 * off for pi, off in zip(g.param_index, g.offset)],
                                       dtype=torch.int64, device=self.device)
         self._active = False
+        # Independent groups run on a few side streams so that the tail of one launch overlaps the
+        # head of the next; biggest first.
+        self.groups.sort(key=lambda g: -len(g) * g.bm * g.bn * (g.bm + g.bn))
+        self.streams = [torch.cuda.Stream(device=self.device) for _ in range(min(streams, len(self.groups)))]
+
+    def _fan_out(self, jobs):
+        """Run the callables round-robin on the side streams, after everything already queued on the
+        current stream; the current stream then waits for all of them."""
+        if not self.streams:
+            for job in jobs:
+                job()
+            return
+        main = torch.cuda.current_stream(self.device)
+        start = torch.cuda.Event()
+        start.record(main)
+        for i, job in enumerate(jobs):
+            side = self.streams[i % len(self.streams)]
+            if i < len(self.streams):
+                side.wait_event(start)
+            with torch.cuda.stream(side):
+                job()
+        for side in self.streams[:len(jobs)]:
+            done = torch.cuda.Event()
+            done.record(side)
+            main.wait_event(done)
 
     # ---- eligibility -----------------------------------------------------------------------------
     @staticmethod
@@ -143,32 +169,51 @@ class ShampooBank:
         self._check(grads)
         w1 = self.stat_decay
         w2 = 1.0 if w1 == 1.0 else 1.0 - w1
-        for g in self.groups:
-            G = self._grad_list(g, grads)
-            for side in (0, 1):
+
+        def job(g, side):
+            def run():
+                G = self._grad_list(g, grads)
                 seg = self._segment(self.stats, g, side)
-                out = self.scratch[seg.order][:len(g)]
+                out = g.scratch[side]
                 X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, out=out,
                        symmetric=True)
                 X.quantize_stack(out, seg)
+            return run
+
+        for g in self.groups:           # address tables are written on the current stream, before the fan-out
+            self._grad_list(g, grads)
+        self._fan_out([job(g, side) for g in self.groups for side in (0, 1)])
 
     @torch.no_grad()
     def compute_preconditioners(self, v0=None):
         """v0: optional dict order -> [count, order] start vectors of the power iteration."""
-        for order, stat in self.stats.items():
-            dense = X.dequantize_stack(stat)
-            roots = ComputePowerBatched(dense, 4, ridge_epsilon=self.matrix_eps, v0=None if v0 is None else v0[order])
-            X.quantize_stack(roots.contiguous(), self.precs[order])
+        def job(order):
+            def run():
+                dense = X.dequantize_stack(self.stats[order])
+                roots = ComputePowerBatched(dense, 4, ridge_epsilon=self.matrix_eps, v0=starts[order])
+                X.quantize_stack(roots.contiguous(), self.precs[order])
+            return run
+
+        # start vectors come from the global generator in a fixed order, whatever the streams do
+        starts = {order: (torch.rand(stat.batch, order, device=self.device) * 2 - 1) if v0 is None else v0[order]
+                  for order, stat in self.stats.items()}
+        self._fan_out([job(order) for order in sorted(self.stats, key=lambda o: -o ** 3 * self.stats[o].batch)])
         self._active = True
 
     @torch.no_grad()
     def preconditioned_grads(self, grads):
         """List of P_L G P_R per parameter (buffers owned by the bank, overwritten by the next call)."""
         self._check(grads)
+
+        def job(g):
+            def run():
+                X.gemm(self._segment(self.precs, g, 0), self._grad_list(g, grads), out=g.half)
+                X.gemm(g.half, self._segment(self.precs, g, 1), out=X.PtrList(g.out_ptrs, (len(g), g.bm, g.bn), ld=g.ld))
+            return run
+
         for g in self.groups:
-            G = self._grad_list(g, grads)
-            tmp = X.gemm(self._segment(self.precs, g, 0), G)
-            X.gemm(tmp, self._segment(self.precs, g, 1), out=X.PtrList(g.out_ptrs, (len(g), g.bm, g.bn), ld=g.ld))
+            self._grad_list(g, grads)
+        self._fan_out([job(g) for g in self.groups])
         return [out.view(p.shape) for out, p in zip(self.outputs, self.params)]
 
     def is_active(self):
