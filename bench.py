@@ -7,7 +7,9 @@ on one MI355X, reported as achieved HBM GB/s over the algorithmic bytes.
 One "step" = one quantize launch + one dequantize launch over the whole tensor, inputs
 resident in HBM.  The same JSON line also carries, under "precond_step", the second half of the
 metric: ms per 4-bit Shampoo preconditioner step over the ViT-B/32 weight shapes, with the CPU
-restatement timed on a bounded sample beside it.  Prints one JSON line.
+restatement timed on a bounded sample beside it; under "fused_gemm" the fused dequantize -> MFMA
+products deq(L) G deq(R) against the fp32 matrix peak; under "other_formats" the 8-bit and
+blocksize-256 variants of the headline tensor.  Prints one JSON line.
 """
 import argparse
 import json
@@ -107,8 +109,7 @@ def precond_step_gpu(torch):
     mean = lambda xs, k: sum(x[k] for x in xs) / len(xs)          # noqa: E731
     reg, new = mean(regular, 0), mean(newton, 0)
     blocks = sum(((m - 1) // 1024 + 1) * ((n - 1) // 1024 + 1) for m, n in vit_b32_shapes())
-    gram_flop = sum(2 * m * m * n + 2 * m * n * n for m, n in vit_b32_shapes())   # unblocked upper bound is not used:
-    gram_flop = 0
+    gram_flop = 0                                        # G G^T and G^T G of every block of at most 1024 x 1024
     for m, n in vit_b32_shapes():
         rows = [1024] * ((m - 1) // 1024) + [m - 1024 * ((m - 1) // 1024)]
         cols = [1024] * ((n - 1) // 1024) + [n - 1024 * ((n - 1) // 1024)]
@@ -126,6 +127,84 @@ def precond_step_gpu(torch):
         "product_gflop_per_regular_step": round(2 * gram_flop / 1e9, 1),
         "product_tflops_regular": round(2 * gram_flop / (mean(regular, 1) * 1e-3) / 1e12, 1),
     }
+
+
+FP32_MATRIX_PEAK_TFLOPS = 157.3
+
+
+def fused_gemm_gpu(torch, code):
+    """deq(Lq) @ G @ deq(Rq) for G 768 x 3072, Lq 768^2 and Rq 3072^2 stored 4-bit / blocksize 64 with exact
+    diagonals: the two fused products, timed with events on the launch stream."""
+    import qtensor.fused as X
+    g = torch.Generator(device="cuda").manual_seed(3)
+    m, n = 768, 3072
+    G = 0.02 * torch.randn(m, n, device="cuda", generator=g)
+
+    def inverse_root_like(order):
+        q, _ = torch.linalg.qr(torch.randn(order, order, device="cuda", generator=g))
+        lam = torch.exp(torch.rand(order, device="cuda", generator=g) * (-6.0 * 2.302585093))   # log-uniform in [1e-6, 1]
+        return ((q * lam.pow(-0.25)) @ q.T).contiguous()
+
+    Lq = X.quantize_stack(inverse_root_like(m).unsqueeze(0), X.empty_quantized(1, m, BLOCK, BITS, code, True))
+    Rq = X.quantize_stack(inverse_root_like(n).unsqueeze(0), X.empty_quantized(1, n, BLOCK, BITS, code, True))
+    half, out = torch.empty(m, n, device="cuda"), torch.empty(m, n, device="cuda")
+
+    def run():
+        X.gemm(Lq, G, out=half)
+        X.gemm(half, Rq, out=out)
+
+    for _ in range(3):
+        run()
+    reps = 20
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+    ev[0].record()
+    for i in range(reps):
+        run()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    ms = sum(ev[i].elapsed_time(ev[i + 1]) for i in range(reps)) / reps
+    flop = 2.0 * m * m * n + 2.0 * m * n * n
+    tf = flop / (ms * 1e-3) / 1e12
+    return {
+        "workload": "deq(Lq 768x768) @ G(768x3072) @ deq(Rq 3072x3072), 4-bit linear-2 blocksize 64 factors with exact "
+                    "diagonal, fp32 MFMA (v_mfma_f32_32x32x2_f32), two fused launches",
+        "ms": round(ms, 4),
+        "gflop": round(flop / 1e9, 2),
+        "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tf / FP32_MATRIX_PEAK_TFLOPS, 4), "traffic": None},
+    }
+
+
+def other_formats_gpu(torch, F, x):
+    """The same tensor through the other table / blocksize combinations (informational)."""
+    n = x.numel()
+    out = {}
+    for bits, bs in ((4, 256), (8, 64), (8, 256)):
+        code = (F.create_linear_map(True, bits, 2) if bits == 4 else F.create_dynamic_map(True, bits, 1)).cuda()
+        q = torch.empty(n * bits // 8, dtype=torch.uint8, device="cuda")
+        am = torch.empty(n // bs, dtype=torch.float32, device="cuda")
+        back = torch.empty_like(x)
+
+        def step():
+            F.quantize_blockwise(x, code, ORDER, absmax=am, out=q, blocksize=bs, bits=bits)
+            F.dequantize_blockwise(q, code, ORDER, am, out=back, blocksize=bs, bits=bits)
+
+        for _ in range(2):
+            step()
+        reps = 10
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        nbytes = 2 * (4 + bits / 8 + 4 / bs) * n
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        out[f"{bits}bit_bs{bs}"] = {"table": "linear-2" if bits == 4 else "dynamic", "ms_per_step": round(ms, 4),
+                                    "GB/s": round(gbs, 1), "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2)}
+        del q, am, back
+    return out
 
 
 def precond_step_cpu(torch, code_host):
@@ -161,7 +240,12 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-step", action="store_true", help="skip the Shampoo preconditioner-step measurement")
+    ap.add_argument("--section", choices=["all", "quant", "gemm", "step"], default="all",
+                    help="run only one part (for profiling one kernel family); the JSON line then lacks the others")
+    ap.add_argument("--bank-streams", type=int, default=None,
+                    help="side streams of the batched preconditioner engine (0 serialises its launches, which "
+                         "keeps per-kernel durations in a profile free of overlap)")
+    ap.add_argument("--no-step", action="store_true", help="skip the fused-product, other-format and Shampoo-step measurements")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1).")
@@ -176,6 +260,15 @@ def main():
 
     code_host = F.create_linear_map(True, BITS, 2)
     code = code_host.cuda()
+    if args.bank_streams is not None:
+        from optimizers.engine import ShampooBank
+        ShampooBank.DEFAULT_STREAMS = args.bank_streams
+    if args.section in ("gemm", "step"):
+        part = fused_gemm_gpu(torch, code) if args.section == "gemm" else precond_step_gpu(torch)
+        print(json.dumps({"section": args.section, "n_gpus": 1, ("fused_gemm" if args.section == "gemm" else "precond_step"): part}))
+        return
+    if args.section == "quant":
+        args.no_step = args.no_cpu_baseline = True
     x = stress_tensor(torch, ORDER)
     n = ORDER * ORDER
     out = torch.empty(n * BITS // 8, dtype=torch.uint8, device="cuda")
@@ -260,9 +353,13 @@ def main():
         },
     }
     x_slice = None if args.no_cpu_baseline else x.view(-1)[: 4096 * 4096].cpu()
-    del x, out, absmax, back
+    del out, absmax, back
+    if not args.no_step:
+        result["other_formats"] = other_formats_gpu(torch, F, x)
+    del x
     torch.cuda.empty_cache()
     if not args.no_step:
+        result["fused_gemm"] = fused_gemm_gpu(torch, code)
         result["precond_step"] = precond_step_gpu(torch)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch, x_slice, code_host)

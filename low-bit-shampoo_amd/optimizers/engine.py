@@ -39,8 +39,10 @@ class _Group:
 
 
 class ShampooBank:
+    DEFAULT_STREAMS = 3          # side streams for independent groups (0: everything on the current stream)
+
     def __init__(self, params, name2qmap, code, stat_decay=0.95, matrix_eps=1e-6, prec_maxorder=1200,
-                 prec_bits=4, min_lowbit_size=4096, quan_blocksize=64, streams=3):
+                 prec_bits=4, min_lowbit_size=4096, quan_blocksize=64, streams=None):
         self.stat_decay, self.matrix_eps = stat_decay, matrix_eps
         self.bits, self.blocksize = prec_bits, quan_blocksize
         self.params = list(params)
@@ -89,6 +91,7 @@ class ShampooBank:
         # Independent groups run on a few side streams so that the tail of one launch overlaps the
         # head of the next; biggest first.
         self.groups.sort(key=lambda g: -len(g) * g.bm * g.bn * (g.bm + g.bn))
+        streams = self.DEFAULT_STREAMS if streams is None else streams
         self.streams = [torch.cuda.Stream(device=self.device) for _ in range(min(streams, len(self.groups)))]
 
     def _fan_out(self, jobs):
