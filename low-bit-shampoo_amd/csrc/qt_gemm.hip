@@ -20,6 +20,9 @@
 // run two tiles ahead of the MFMAs; the LDS commit sits in the middle of the MFMA stream.
 #include "qt_common.h"
 
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
 #include <type_traits>
 
 namespace qt {
@@ -574,17 +577,37 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
     const bool need_code = ka >= kQuant4 || kb >= kQuant4 || ep == kAxpbyQuant4 || ep == kAxpbyQuant8;
     if (need_code && !a.code) { set_error(kNullPointer, "gemm: code table missing"); return; }
 
-    // 128 x 128 tiles when that still gives every compute unit work, else 64 x 64 (quantized
-    // operands always use a 128-wide tile on their side).
-    const long long t128 = (d->N + 127) / 128;
-    const long long big_tiles = (a.symmetric ? t128 * (t128 + 1) / 2 : (long long)((d->M + 127) / 128) * t128) * d->batch;
-    const bool big = big_tiles >= compute_units();
+    // Tile shape: the one with the smallest estimated makespan.  Workgroups that share a compute unit
+    // share its matrix pipes, so the time is (most tiles on one unit) x (tile area) / (efficiency of
+    // that shape: smaller tiles read more LDS words per multiply).  Quantized operands keep a
+    // 128-wide tile on their side unless QT_GEMM_TILE=MxN (a tuning knob) says otherwise.
+    struct Shape { int bm, bn; double eff; };
+    static const Shape shapes[4] = {{128, 128, 1.0}, {128, 64, 0.92}, {64, 128, 0.92}, {64, 64, 0.82}};
+    int pick = 0;
+    static const char *forced = getenv("QT_GEMM_TILE");
+    if (forced != nullptr) {
+        int fm = 0, fn = 0;
+        if (sscanf(forced, "%dx%d", &fm, &fn) == 2)
+            for (int i = 0; i < 4; ++i) if (shapes[i].bm == fm && shapes[i].bn == fn) pick = i;
+    } else {
+        const double units = compute_units();
+        double best = 0.0;
+        for (int i = 0; i < 4; ++i) {
+            const Shape &sh = shapes[i];
+            if (a.symmetric && sh.bm != sh.bn) continue;
+            const long long tm = (d->M + sh.bm - 1) / sh.bm, tn = (d->N + sh.bn - 1) / sh.bn;
+            const double tiles = (double)(a.symmetric ? tn * (tn + 1) / 2 : tm * tn) * d->batch;
+            const double cost = ceil(tiles / units) * sh.bm * sh.bn / sh.eff;
+            if (i == 0 || cost < best) { best = cost; pick = i; }
+        }
+    }
+    if (a.symmetric && shapes[pick].bm != shapes[pick].bn) pick = 0;
     const int combo = ka * 100 + kb * 10 + ep;
 #define QT_GEMM_CASE(KA, KB, EP)                                                                             \
     case (KA) * 100 + (KB) * 10 + (EP):                                                                      \
-        if (big) launch_gemm<128, 128, KA, KB, EP>(a, d->batch, stream);                                     \
-        else if ((KA) >= kQuant4) launch_gemm<128, 64, KA, KB, EP>(a, d->batch, stream);                     \
-        else if ((KB) >= kQuant4) launch_gemm<64, 128, KA, KB, EP>(a, d->batch, stream);                     \
+        if (pick == 0) launch_gemm<128, 128, KA, KB, EP>(a, d->batch, stream);                               \
+        else if (pick == 1) launch_gemm<128, 64, KA, KB, EP>(a, d->batch, stream);                           \
+        else if (pick == 2) launch_gemm<64, 128, KA, KB, EP>(a, d->batch, stream);                           \
         else launch_gemm<64, 64, KA, KB, EP>(a, d->batch, stream);                                           \
         break;
     switch (combo) {
