@@ -41,41 +41,76 @@ class Preconditioner(PreconditionerBase):
         return newton_inverse_root(stat, exp, eps, getattr(self, '_v0', None)).to(stat.dtype)
 
 
-class ShampooSGD(ShampooSGDBase):
+class _FusedStep:
     """fused=True (not in the reference) runs all eligible GPU parameters through one batched
-    ShampooBank instead of one Preconditioner object per parameter; the arithmetic is the same."""
-    preconditioner_class = Preconditioner
+    ShampooBank instead of one Preconditioner object per parameter; the arithmetic is the same.
 
-    def __init__(self, params, *args, fused=False, **kwargs):
-        super().__init__(params, *args, **kwargs)
+    Checkpoints: state_dict() then carries, next to torch's usual entries, 'shampoo_bank': one
+    dict of plain tensors per parameter group -- per block order n the stacked 4/8-bit statistics
+    and preconditioners ('stats.n.codes' uint8 [count, n*n*bits/8] with the first element of a pair
+    in the high nibble, 'stats.n.absmax' fp32 [count, n*n/blocksize], 'stats.n.diag' fp32 [count, n],
+    the same under 'precs.'), 'block_table' int64 [statistics, 5] = (parameter index in the group,
+    block index within the parameter, side, order, row in that order's stack), and the step count.
+    Nothing in it is a pickled Python object, so torch.load(..., weights_only=True) reads it."""
+
+    _update = None
+
+    def _init_fused(self, fused):
         self._fused = fused
+        self._pending_bank_state = None
 
     @torch.no_grad()
     def step(self, closure=None):
         if not self._fused:
             return super().step(closure)
-        for group in self.param_groups:
-            fused_step(self, group, _sgd_update)
+        for index, group in enumerate(self.param_groups):
+            fused_step(self, group, type(self)._update, index)
+
+    def state_dict(self):
+        sd = super().state_dict()
+        if self._fused:
+            banks = []
+            for group in self.param_groups:
+                entry = self.__dict__.get('_fused_cache', {}).get(id(group))
+                if entry is None:
+                    banks.append(None)
+                    continue
+                one = {'step': torch.tensor(entry['step'])}
+                if entry['bank'] is not None:
+                    one.update(entry['bank'].state_dict())
+                    one['block_table'] = torch.tensor(entry['bank'].block_table(), dtype=torch.int64)
+                banks.append(one)
+            sd['shampoo_bank'] = banks
+        return sd
+
+    def load_state_dict(self, state_dict):
+        state_dict = dict(state_dict)
+        banks = state_dict.pop('shampoo_bank', None)
+        super().load_state_dict(state_dict)
+        if banks is not None:
+            self.__dict__.pop('_fused_cache', None)          # rebuilt, then filled, by the next step
+            self._pending_bank_state = list(banks)              # consumed group by group; the caller's list stays as it is
 
 
-class ShampooAdamW(ShampooAdamWBase):
-    """fused=True (not in the reference) runs all eligible GPU parameters through one batched
-    ShampooBank instead of one Preconditioner object per parameter; the arithmetic is the same."""
+class ShampooSGD(_FusedStep, ShampooSGDBase):
+    __doc__ = _FusedStep.__doc__
     preconditioner_class = Preconditioner
 
     def __init__(self, params, *args, fused=False, **kwargs):
         super().__init__(params, *args, **kwargs)
-        self._fused = fused
-
-    @torch.no_grad()
-    def step(self, closure=None):
-        if not self._fused:
-            return super().step(closure)
-        for group in self.param_groups:
-            fused_step(self, group, _adamw_update)
+        self._init_fused(fused)
 
 
-def fused_step(opt, group, update):
+class ShampooAdamW(_FusedStep, ShampooAdamWBase):
+    __doc__ = _FusedStep.__doc__
+    preconditioner_class = Preconditioner
+
+    def __init__(self, params, *args, fused=False, **kwargs):
+        super().__init__(params, *args, **kwargs)
+        self._init_fused(fused)
+
+
+def fused_step(opt, group, update, group_index=0):
     """One optimizer step of a parameter group with the preconditioner work batched."""
     from optimizers.engine import ShampooBank
 
@@ -92,9 +127,19 @@ def fused_step(opt, group, update):
         entry = cache[id(group)] = dict(bank=bank, banked=banked, ids={id(p) for p in banked}, step=0)
         for p in params:
             state = opt.state[p]
-            state['step'] = 0
-            if id(p) not in entry['ids']:
+            state.setdefault('step', 0)
+            if id(p) not in entry['ids'] and 'preconditioner' not in state:
                 state['preconditioner'] = opt._make_preconditioner(p, group)
+        pending = getattr(opt, '_pending_bank_state', None)
+        if pending is not None and group_index < len(pending) and pending[group_index] is not None:
+            saved = pending[group_index]
+            entry['step'] = int(saved['step'])
+            if bank is not None:
+                table = torch.tensor(bank.block_table(), dtype=torch.int64)
+                if 'block_table' not in saved or not torch.equal(saved['block_table'].cpu(), table):
+                    raise ValueError("checkpoint was written for other parameter shapes or block sizes")
+                bank.load_state_dict(saved)
+            pending[group_index] = None
     entry['step'] += 1
     step, bank, banked = entry['step'], entry['bank'], entry['banked']
     for p in params:
@@ -185,5 +230,7 @@ def _sgd_update(opt, group, params, dirs, grads, graft, step, entry):
     torch._foreach_add_(params, dirs, alpha=-group['lr'])
 
 
-ShampooSGD.__doc__ = _DOC.format(base="SGD", more="")
-ShampooAdamW.__doc__ = _DOC.format(base="AdamW", more="")
+ShampooSGD._update = staticmethod(_sgd_update)
+ShampooAdamW._update = staticmethod(_adamw_update)
+ShampooSGD.__doc__ = _DOC.format(base="SGD", more="") + _FusedStep.__doc__
+ShampooAdamW.__doc__ = _DOC.format(base="AdamW", more="") + _FusedStep.__doc__

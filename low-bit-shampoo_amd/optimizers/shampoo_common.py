@@ -215,7 +215,7 @@ class _ShampooOptimizer(optim.Optimizer):
         for group in self.param_groups:
             for p in group['params']:
                 state = self.state[p]
-                if len(state) != 0:
+                if len(state) != 0 and 'preconditioner' in state:     # absent for parameters held by a ShampooBank
                     state['preconditioner'].set_device(p.device)
 
     def _make_preconditioner(self, p, group):

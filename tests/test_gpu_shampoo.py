@@ -210,3 +210,59 @@ def test_fused_update_kernels_match_the_torch_update_rules(which):
     with pytest.raises(ValueError):
         TailPlan().sgd([torch.zeros(4, device="cuda")], [torch.zeros(4)], [torch.zeros(4, device="cuda")],
                        [torch.zeros(4, device="cuda")], [False], 0.1, 0.9, 0.0, False)
+
+
+@pytest.mark.parametrize("which", ["adamw", "sgd"])
+def test_fused_optimizer_checkpoint_round_trip(setup, which, monkeypatch):
+    """state_dict() of the fused optimizers carries the bank's quantized state as plain tensors: a run
+    resumed from a checkpoint (written and read with weights_only=True for the bank part) continues
+    exactly like the uninterrupted one."""
+    import io
+    S1 = setup[0]
+    import optimizers.matrix_functions as MF
+    real_rand = torch.rand
+    monkeypatch.setattr(MF.torch, "rand", lambda *size, **kw: torch.full(size, 0.75, **kw))
+    g = torch.Generator().manual_seed(6)
+    init = [real_rand(s, generator=g) for s in SHAPES]
+    gs = [[0.02 * torch.randn(s, generator=g) for s in SHAPES] for _ in range(5)]
+
+    def make(params):
+        common = dict(start_prec_step=2, stat_compute_steps=1, prec_compute_steps=2, fused=True, **KW)
+        return (S1.ShampooAdamW(params, lr=1e-2, weight_decay=0.05, **common) if which == "adamw"
+                else S1.ShampooSGD(params, lr=1e-2, momentum=0.9, **common))
+
+    def run(opt, params, steps):
+        for st in steps:
+            for p, gr in zip(params, gs[st]):
+                p.grad = gr.clone().cuda()
+            opt.step()
+
+    straight = [torch.nn.Parameter(t.clone().cuda()) for t in init]
+    run(make(straight), straight, range(5))
+
+    first = [torch.nn.Parameter(t.clone().cuda()) for t in init]
+    opt = make(first)
+    run(opt, first, range(3))
+    sd = opt.state_dict()
+    bank = sd["shampoo_bank"]
+    assert len(bank) == 1 and int(bank[0]["step"]) == 3 and bank[0]["block_table"].shape[1] == 5
+    assert all(isinstance(v, (torch.Tensor, bool)) for v in bank[0].values())
+    buf = io.BytesIO()
+    torch.save(bank, buf)
+    buf.seek(0)
+    sd["shampoo_bank"] = torch.load(buf, weights_only=True, map_location="cpu")
+    resumed = [torch.nn.Parameter(p.detach().clone()) for p in first]
+    opt2 = make(resumed)
+    opt2.load_state_dict(sd)
+    run(opt2, resumed, range(3, 5))
+    for a, b in zip(straight, resumed):
+        assert torch.equal(a.detach(), b.detach())
+    # a checkpoint for other shapes is refused
+    other = [torch.nn.Parameter(torch.zeros(128, 64, device="cuda"))]
+    opt3 = make(other)
+    bad = opt3.state_dict()
+    bad["shampoo_bank"] = sd["shampoo_bank"]
+    opt3.load_state_dict(bad)
+    other[0].grad = torch.ones(128, 64, device="cuda")
+    with pytest.raises(ValueError):
+        opt3.step()
