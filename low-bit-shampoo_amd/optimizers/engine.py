@@ -73,15 +73,14 @@ class ShampooBank:
             for side, order in enumerate((g.bm, g.bn)):
                 g.slot[side] = (order, per_order[order])
                 per_order[order] += len(g)
-        self.stats, self.precs = {}, {}
+        self.per_order = dict(per_order)
+        self.precs = {}
         for order, count in per_order.items():
             eye = torch.eye(order, device=self.device).expand(count, order, order)
-            self.stats[order] = X.quantize_stack((matrix_eps * eye).contiguous(),
-                                                 X.empty_quantized(count, order, quan_blocksize, prec_bits, self.code, True))
             self.precs[order] = X.quantize_stack(eye.contiguous(),
                                                  X.empty_quantized(count, order, quan_blocksize, prec_bits, self.code, True))
-        for g in self.groups:       # fp32 landing areas of the updated statistics and of P_L G, per group
-            g.scratch = [torch.empty(len(g), o, o, device=self.device) for o in (g.bm, g.bn)]
+        self._init_statistics()
+        for g in self.groups:       # fp32 landing area of P_L G, per group
             g.half = torch.empty(len(g), g.bm, g.bn, device=self.device)
         self.outputs = [torch.empty(m, n, device=self.device) for m, n in self.shapes]
         for g in self.groups:
@@ -93,6 +92,16 @@ class ShampooBank:
         self.groups.sort(key=lambda g: -len(g) * g.bm * g.bn * (g.bm + g.bn))
         streams = self.DEFAULT_STREAMS if streams is None else streams
         self.streams = [torch.cuda.Stream(device=self.device) for _ in range(min(streams, len(self.groups)))]
+
+    def _init_statistics(self):
+        """Statistics start as matrix_eps * I, stored quantized with an exact diagonal."""
+        self.stats = {}
+        for order, count in self.per_order.items():
+            eye = torch.eye(order, device=self.device).expand(count, order, order)
+            self.stats[order] = X.quantize_stack((self.matrix_eps * eye).contiguous(),
+                                                 X.empty_quantized(count, order, self.blocksize, self.bits, self.code, True))
+        for g in self.groups:       # fp32 landing areas of the updated statistics, per group and side
+            g.scratch = [torch.empty(len(g), o, o, device=self.device) for o in (g.bm, g.bn)]
 
     def _fan_out(self, jobs):
         """Run the callables round-robin on the side streams, after everything already queued on the
@@ -240,8 +249,9 @@ class ShampooBank:
                     rows.append((pi, j, side, order, first + i))
         return rows
 
-    def state_dict(self):
-        out = {"active": self._active}
+    def _tensors(self):
+        """name -> tensor of everything a checkpoint has to hold."""
+        out = {}
         for name, table in (("stats", self.stats), ("precs", self.precs)):
             for order, q in table.items():
                 out[f"{name}.{order}.codes"] = q.codes
@@ -249,10 +259,10 @@ class ShampooBank:
                 out[f"{name}.{order}.diag"] = q.diag
         return out
 
+    def state_dict(self):
+        return {"active": self._active, **self._tensors()}
+
     def load_state_dict(self, sd):
         self._active = bool(sd["active"])
-        for name, table in (("stats", self.stats), ("precs", self.precs)):
-            for order, q in table.items():
-                q.codes.copy_(sd[f"{name}.{order}.codes"])
-                q.absmax.copy_(sd[f"{name}.{order}.absmax"])
-                q.diag.copy_(sd[f"{name}.{order}.diag"])
+        for name, t in self._tensors().items():
+            t.copy_(sd[name])

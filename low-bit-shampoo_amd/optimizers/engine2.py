@@ -1,0 +1,197 @@
+"""Batched execution of the eigenbasis variant of low-bit Shampoo (the reference's shampoo2.py)
+over all parameters at once.
+
+Every statistic L is held as the reference's QTensorSVDFast holds it (qtensor/utils.py:124-236):
+the quantized matrix Vt whose rows approximate eigenvectors, the smaller half of the Rayleigh
+quotients, the rows they belong to and the largest quotient.  One statistics update is one step
+of subspace iteration per matrix (shampoo2.py:185-200, utils.py:156-203):
+
+    Vt <- 1.5 Vt - 0.5 Vt Vt^T Vt            (rect_t1 times, after dequantizing)
+    L  <- b * Vt[keep]^T diag(S) Vt[keep] + (1 - b) * G G^T
+    V  <- orthonormal basis of L Vt^T, columns in order (QR)
+    quotients <- diag(V^T L V); keep the smaller half; store V^T quantized
+
+Here all statistics of one order form a stack and every line above is one or two launches for
+the whole stack: the products run on the matrix cores through qtensor.fused.gemm (symmetric
+ones compute half and mirror), and the QR factorisation -- 20 ms per 1024 x 1024 matrix through
+the vendor's Householder routine, 5 s per step for a ViT-B/32 -- is replaced by a shifted
+Cholesky QR (rounds of  G = Q^T Q,  R = chol(G + s I),  Q <- Q R^-1  on the column-scaled
+matrix until Q is orthonormal), which yields the same factor Q up to column signs.  Matrices it
+cannot finish are redone with torch.linalg.qr.
+"""
+import torch
+
+from optimizers.engine import ShampooBank
+from optimizers.matrix_functions import ComputePowerBatched
+from qtensor import fused as X
+
+
+_householder_qr = torch.linalg.qr
+
+
+def _fenced(fn, *args, **kwargs):
+    """Call a torch.linalg routine with the device idle before and after.  On this PyTorch-ROCm
+    build a chain  solve_triangular -> matmul -> cholesky_ex  issued back to back on one stream
+    returns wrong factors now and then (torch-only reproduction: the second cholesky_ex of such a
+    chain reports a non-positive minor for a well-conditioned matrix; any synchronisation in between
+    cures it), so these calls are not trusted to be stream-ordered."""
+    torch.cuda.synchronize()
+    out = fn(*args, **kwargs)
+    torch.cuda.synchronize()
+    return out
+
+
+def cholesky_qr(Y, max_rounds=12, shift=1e-3, tolerance=2e-5):
+    """Orthonormal Q [B, n, n] with span(Q[:, :, :k]) == span(Y[:, :, :k]) for every k (the Q factor
+    of a QR factorisation with positive diagonal of R), by rounds of  G = Q^T Q,  R = chol(G + s I),
+    Q <- Q R^-1  on the column-scaled matrix; every R is upper triangular, so the nested spans
+    survive each round.  A matrix far from orthonormal (||G - I||_F >= 0.5) gets the shift s, which
+    lifts its small singular values by 1 / sqrt(s) per round -- a numerically singular Y ends, like
+    with Householder reflections, in a completion fixed by rounding noise; once ||G - I||_F < 0.5 an
+    unshifted round finishes it.  Matrices that are not orthonormal to `tolerance` (max |G - I|)
+    after max_rounds go through torch.linalg.qr.  Returns (Q, number of those)."""
+    B, n, _ = Y.shape
+    scale = torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)
+    Q = (Y / scale).contiguous()                  # unit columns: the Gram matrix has a unit diagonal
+    failed = torch.zeros(B, dtype=torch.bool, device=Y.device)
+    done = failed
+    for _ in range(max_rounds + 1):
+        gram = X.gemm(Q, Q, trans_a=True, symmetric=True)
+        diag = gram.diagonal(dim1=1, dim2=2)
+        diag.sub_(1.0)
+        done = gram.abs().amax(dim=(1, 2)) < tolerance                         # False for NaN as well
+        if bool(done.all()):                                                   # host synchronisation
+            break
+        far = ~(torch.linalg.matrix_norm(gram) < 0.5)
+        diag.add_(1.0 + shift * far.to(gram.dtype).unsqueeze(1))
+        R, info = _fenced(torch.linalg.cholesky_ex, gram, upper=True)
+        failed = failed | (info != 0)
+        Q = _fenced(torch.linalg.solve_triangular, R, Q, upper=True, left=False).contiguous()
+    redo = torch.nonzero(failed | ~done).flatten()
+    if redo.numel():
+        Q[redo] = _fenced(_householder_qr, Y[redo])[0]
+    return Q, int(redo.numel())
+
+
+class ShampooBank2(ShampooBank):
+    def __init__(self, params, name2qmap, code, *, rect_t1=1, rect_t2=4, inv_root_mode=0, **kwargs):
+        self.rect_t1, self.rect_t2, self.inv_root_mode = rect_t1, rect_t2, inv_root_mode
+        self.qr_fallbacks = 0                     # matrices that went through torch.linalg.qr so far
+        super().__init__(params, name2qmap, code, **kwargs)
+
+    def _init_statistics(self):
+        """Basis = quantized identity, every kept quotient and the largest one = matrix_eps
+        (reference: utils.py:134-153 with var = matrix_eps * I)."""
+        self.basis, self.svalue, self.keep, self.max_eig = {}, {}, {}, {}
+        for order, count in self.per_order.items():
+            eye = torch.eye(order, device=self.device).expand(count, order, order).contiguous()
+            self.basis[order] = X.quantize_stack(eye, X.empty_quantized(count, order, self.blocksize, self.bits, self.code, False))
+            half = max(1, order // 2)
+            self.keep[order] = torch.arange(half, device=self.device).expand(count, half).contiguous()
+            self.svalue[order] = torch.full((count, half), self.matrix_eps, device=self.device)
+            self.max_eig[order] = torch.full((count,), self.matrix_eps, device=self.device)
+
+    # ---- pieces of QTensorSVDFast, for a whole stack ---------------------------------------------
+    def _rectified_basis(self, order):
+        """Dequantized Vt after rect_t1 Bjorck steps (utils.py:194-198)."""
+        vt = X.dequantize_stack(self.basis[order])
+        for _ in range(self.rect_t1):
+            vvt = X.gemm(vt, vt, trans_b=True, symmetric=True)
+            vt = X.gemm(vvt, vt, addend=vt, alpha=-0.5, beta=1.5)
+        return vt
+
+    def _kept_rows(self, order, vt):
+        n = vt.shape[2]
+        return torch.gather(vt, 1, self.keep[order].unsqueeze(2).expand(-1, -1, n))
+
+    def _statistic(self, order, vt, out=None):
+        """Vt[keep]^T diag(S) Vt[keep] (utils.py:200-203)."""
+        rows = self._kept_rows(order, vt)
+        return X.gemm(rows * self.svalue[order].unsqueeze(2), rows, trans_a=True, symmetric=True, out=out)
+
+    # ---- the operations of the reference's Preconditioner ----------------------------------------
+    @torch.no_grad()
+    def add_statistics(self, grads):
+        self._check(grads)
+        w1 = self.stat_decay
+        w2 = 1.0 if w1 == 1.0 else 1.0 - w1
+        orders = sorted(self.per_order, key=lambda o: -o ** 3 * self.per_order[o])
+        # buffers that cross the phases below belong to the current stream
+        stat = {o: torch.empty(self.per_order[o], o, o, device=self.device) for o in orders}
+        basis = {}
+        for g in self.groups:
+            self._grad_list(g, grads)
+
+        def rebuild(order):
+            def run():
+                basis[order] = self._rectified_basis(order)
+                self._statistic(order, basis[order], out=stat[order])
+            return run
+
+        def accumulate(g, side):
+            def run():
+                order, first = g.slot[side]
+                seg = stat[order][first:first + len(g)]
+                G = self._grad_list(g, grads)
+                X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, out=seg, symmetric=True)
+            return run
+
+        def iterate(order):
+            def run():
+                L, vt = stat[order], basis[order]
+                Q, redone = cholesky_qr(X.gemm(L, vt, trans_b=True))
+                self.qr_fallbacks += redone
+                quotients = (Q * X.gemm(L, Q)).sum(dim=1)                      # diag(Q^T L Q)
+                ascending, where = torch.sort(quotients, dim=1)
+                half = self.keep[order].shape[1]
+                self.keep[order] = where[:, :half].contiguous()
+                self.svalue[order] = ascending[:, :half].contiguous()
+                self.max_eig[order] = quotients.amax(dim=1)
+                X.quantize_stack(Q.transpose(1, 2).contiguous(), self.basis[order])
+            return run
+
+        self._fan_out([rebuild(o) for o in orders])
+        self._fan_out([accumulate(g, side) for g in self.groups for side in (0, 1)])
+        self._fan_out([iterate(o) for o in orders])
+
+    @torch.no_grad()
+    def compute_preconditioners(self, v0=None):
+        """inv_root_mode 0: inverse 4th root from the stored eigenpairs (functional.py:749-762 through
+        utils.py:205-227); 1: coupled Newton on the rebuilt statistic.  v0 as in ShampooBank."""
+        orders = sorted(self.per_order, key=lambda o: -o ** 3 * self.per_order[o])
+        starts = {}
+        if self.inv_root_mode != 0:
+            starts = {o: (torch.rand(self.per_order[o], o, device=self.device) * 2 - 1) if v0 is None else v0[o]
+                      for o in self.per_order}
+
+        def job(order):
+            def run():
+                if self.inv_root_mode == 0:
+                    rows = self._kept_rows(order, X.dequantize_stack(self.basis[order]))
+                    for _ in range(self.rect_t2):
+                        vvt = X.gemm(rows, rows, trans_b=True, symmetric=True)
+                        rows = X.gemm(vvt, rows, addend=rows, alpha=-0.5, beta=1.5)
+                    ridge = self.matrix_eps * self.max_eig[order]
+                    weights = 1 / (self.svalue[order] + ridge.unsqueeze(1)).pow(1 / 4)
+                    roots = X.gemm(rows * weights.unsqueeze(2), rows, trans_a=True, symmetric=True)
+                else:
+                    L = self._statistic(order, self._rectified_basis(order))
+                    # L is symmetric up to the rounding inside its diagonal tiles: half products are fine
+                    roots = ComputePowerBatched(L, 4, ridge_epsilon=self.matrix_eps, v0=starts[order], symmetric=True)
+                X.quantize_stack(roots.contiguous(), self.precs[order])
+            return run
+
+        self._fan_out([job(o) for o in orders])
+        self._active = True
+
+    # ---- checkpoints -----------------------------------------------------------------------------
+    def _tensors(self):
+        out = {}
+        for order in self.per_order:
+            q = self.basis[order]
+            out[f"basis.{order}.codes"], out[f"basis.{order}.absmax"] = q.codes, q.absmax
+            out[f"basis.{order}.svalue"], out[f"basis.{order}.keep"] = self.svalue[order], self.keep[order]
+            out[f"basis.{order}.max_eigenvalue"] = self.max_eig[order]
+            p = self.precs[order]
+            out[f"precs.{order}.codes"], out[f"precs.{order}.absmax"], out[f"precs.{order}.diag"] = p.codes, p.absmax, p.diag
+        return out

@@ -8,6 +8,7 @@ import torch
 
 from optimizers.shampoo_common import (CODE, BlockPartitioner, PreconditionerBase, ShampooAdamWBase, ShampooSGDBase,
                                        _DOC, _fusable, dense_gram, newton_inverse_root)
+from optimizers.fused_step import _FusedStep, _adamw_update, _sgd_update
 from qtensor.utils import QTensorDiagReal
 
 __all__ = ["CODE", "BlockPartitioner", "Preconditioner", "ShampooSGD", "ShampooAdamW"]
@@ -41,57 +42,6 @@ class Preconditioner(PreconditionerBase):
         return newton_inverse_root(stat, exp, eps, getattr(self, '_v0', None)).to(stat.dtype)
 
 
-class _FusedStep:
-    """fused=True (not in the reference) runs all eligible GPU parameters through one batched
-    ShampooBank instead of one Preconditioner object per parameter; the arithmetic is the same.
-
-    Checkpoints: state_dict() then carries, next to torch's usual entries, 'shampoo_bank': one
-    dict of plain tensors per parameter group -- per block order n the stacked 4/8-bit statistics
-    and preconditioners ('stats.n.codes' uint8 [count, n*n*bits/8] with the first element of a pair
-    in the high nibble, 'stats.n.absmax' fp32 [count, n*n/blocksize], 'stats.n.diag' fp32 [count, n],
-    the same under 'precs.'), 'block_table' int64 [statistics, 5] = (parameter index in the group,
-    block index within the parameter, side, order, row in that order's stack), and the step count.
-    Nothing in it is a pickled Python object, so torch.load(..., weights_only=True) reads it."""
-
-    _update = None
-
-    def _init_fused(self, fused):
-        self._fused = fused
-        self._pending_bank_state = None
-
-    @torch.no_grad()
-    def step(self, closure=None):
-        if not self._fused:
-            return super().step(closure)
-        for index, group in enumerate(self.param_groups):
-            fused_step(self, group, type(self)._update, index)
-
-    def state_dict(self):
-        sd = super().state_dict()
-        if self._fused:
-            banks = []
-            for group in self.param_groups:
-                entry = self.__dict__.get('_fused_cache', {}).get(id(group))
-                if entry is None:
-                    banks.append(None)
-                    continue
-                one = {'step': torch.tensor(entry['step'])}
-                if entry['bank'] is not None:
-                    one.update(entry['bank'].state_dict())
-                    one['block_table'] = torch.tensor(entry['bank'].block_table(), dtype=torch.int64)
-                banks.append(one)
-            sd['shampoo_bank'] = banks
-        return sd
-
-    def load_state_dict(self, state_dict):
-        state_dict = dict(state_dict)
-        banks = state_dict.pop('shampoo_bank', None)
-        super().load_state_dict(state_dict)
-        if banks is not None:
-            self.__dict__.pop('_fused_cache', None)          # rebuilt, then filled, by the next step
-            self._pending_bank_state = list(banks)              # consumed group by group; the caller's list stays as it is
-
-
 class ShampooSGD(_FusedStep, ShampooSGDBase):
     __doc__ = _FusedStep.__doc__
     preconditioner_class = Preconditioner
@@ -108,126 +58,6 @@ class ShampooAdamW(_FusedStep, ShampooAdamWBase):
     def __init__(self, params, *args, fused=False, **kwargs):
         super().__init__(params, *args, **kwargs)
         self._init_fused(fused)
-
-
-def fused_step(opt, group, update, group_index=0):
-    """One optimizer step of a parameter group with the preconditioner work batched."""
-    from optimizers.engine import ShampooBank
-
-    params = [p for p in group['params'] if p.grad is not None]
-    if not params:
-        return
-    cache = opt.__dict__.setdefault('_fused_cache', {})
-    entry = cache.get(id(group))
-    if entry is None:
-        keys = ('prec_maxorder', 'prec_bits', 'min_lowbit_size', 'quan_blocksize')
-        banked = [p for p in params if ShampooBank.accepts(p, *(group[k] for k in keys))]
-        bank = ShampooBank(banked, opt.name2qmap, CODE, stat_decay=group['stat_decay'], matrix_eps=group['matrix_eps'],
-                           **{k: group[k] for k in keys}) if banked else None
-        entry = cache[id(group)] = dict(bank=bank, banked=banked, ids={id(p) for p in banked}, step=0)
-        for p in params:
-            state = opt.state[p]
-            state.setdefault('step', 0)
-            if id(p) not in entry['ids'] and 'preconditioner' not in state:
-                state['preconditioner'] = opt._make_preconditioner(p, group)
-        pending = getattr(opt, '_pending_bank_state', None)
-        if pending is not None and group_index < len(pending) and pending[group_index] is not None:
-            saved = pending[group_index]
-            entry['step'] = int(saved['step'])
-            if bank is not None:
-                table = torch.tensor(bank.block_table(), dtype=torch.int64)
-                if 'block_table' not in saved or not torch.equal(saved['block_table'].cpu(), table):
-                    raise ValueError("checkpoint was written for other parameter shapes or block sizes")
-                bank.load_state_dict(saved)
-            pending[group_index] = None
-    entry['step'] += 1
-    step, bank, banked = entry['step'], entry['bank'], entry['banked']
-    for p in params:
-        opt.state[p]['step'] = step
-    grads = {id(p): p.grad.contiguous() for p in params}
-    directions, grafted = {}, set()
-    if bank is not None:
-        bgrads = [grads[id(p)] for p in banked]
-        if step % group['stat_compute_steps'] == 0:
-            bank.add_statistics(bgrads)
-        if step % group['prec_compute_steps'] == 0:
-            bank.compute_preconditioners()
-        if step >= group['start_prec_step'] and bank.is_active():
-            # the rescaling to each gradient's norm happens inside the fused update
-            directions = {id(p): o for p, o in zip(banked, bank.preconditioned_grads(bgrads))}
-            grafted = set(directions)
-    for p in params:
-        if id(p) not in entry['ids']:
-            directions[id(p)] = opt._shampoo_direction(p, grads[id(p)], group, opt.state[p])
-    update(opt, group, params, [directions.get(id(p), grads[id(p)]) for p in params], [grads[id(p)] for p in params],
-           [id(p) in grafted for p in params], step, entry)
-
-
-def _fused_tail_ok(params, dirs):
-    return all(p.is_cuda and p.dtype == torch.float32 and p.is_contiguous() and d.dtype == torch.float32 and d.is_contiguous()
-               for p, d in zip(params, dirs))
-
-
-def _tail_plan(entry):
-    from optimizers.tail import TailPlan
-    if entry.get('tail') is None:
-        entry['tail'] = TailPlan()
-    return entry['tail']
-
-
-def _graft(dirs, grads, graft):
-    # keep each gradient's norm (reference: shampoo1.py:421)
-    for d, g, f in zip(dirs, grads, graft):
-        if f:
-            d.mul_(g.norm() / (d.norm() + 1e-12))
-
-
-def _adamw_update(opt, group, params, dirs, grads, graft, step, entry):
-    import math
-    for p in params:
-        state = opt.state[p]
-        if 'exp_avg' not in state:
-            state['exp_avg'] = torch.zeros_like(p, memory_format=torch.preserve_format)
-            state['exp_avg_sq'] = torch.zeros_like(p, memory_format=torch.preserve_format)
-    m = [opt.state[p]['exp_avg'] for p in params]
-    v = [opt.state[p]['exp_avg_sq'] for p in params]
-    beta1, beta2 = group['betas']
-    if _fused_tail_ok(params, dirs):
-        plan = _tail_plan(entry)
-        plan.adamw(params, dirs, grads, m, v, graft, group['lr'], (beta1, beta2), group['eps'], group['weight_decay'], step)
-        return
-    _graft(dirs, grads, graft)
-    torch._foreach_mul_(params, 1 - group['lr'] * group['weight_decay'])
-    torch._foreach_mul_(m, beta1)
-    torch._foreach_add_(m, dirs, alpha=1 - beta1)
-    torch._foreach_mul_(v, beta2)
-    torch._foreach_addcmul_(v, dirs, dirs, value=1 - beta2)
-    denom = torch._foreach_sqrt(v)
-    torch._foreach_div_(denom, math.sqrt(1 - beta2 ** step))
-    torch._foreach_add_(denom, group['eps'])
-    torch._foreach_addcdiv_(params, m, denom, value=-group['lr'] / (1 - beta1 ** step))
-
-
-def _sgd_update(opt, group, params, dirs, grads, graft, step, entry):
-    for p in params:
-        state = opt.state[p]
-        if 'momentum' not in state:
-            state['momentum'] = torch.zeros_like(p, memory_format=torch.preserve_format)
-    bufs = [opt.state[p]['momentum'] for p in params]
-    if _fused_tail_ok(params, dirs):
-        plan = _tail_plan(entry)
-        plan.sgd(params, dirs, grads, bufs, graft, group['lr'], group['momentum'], group['weight_decay'], group['nesterov'])
-        return
-    _graft(dirs, grads, graft)
-    if group['weight_decay'] != 0.0:
-        torch._foreach_add_(dirs, params, alpha=group['weight_decay'])
-    torch._foreach_mul_(bufs, group['momentum'])
-    torch._foreach_add_(bufs, dirs)
-    if group['nesterov']:
-        dirs = torch._foreach_add(dirs, bufs, alpha=group['momentum'])
-    else:
-        dirs = bufs
-    torch._foreach_add_(params, dirs, alpha=-group['lr'])
 
 
 ShampooSGD._update = staticmethod(_sgd_update)

@@ -11,6 +11,7 @@ import torch
 
 from optimizers.shampoo_common import (CODE, BlockPartitioner, PreconditionerBase, ShampooAdamWBase, ShampooSGDBase,
                                        _DOC, dense_gram, newton_inverse_root)
+from optimizers.fused_step import _FusedStep, _adamw_update, _sgd_update
 from qtensor.utils import QTensorSVDFast
 
 __all__ = ["CODE", "BlockPartitioner", "Preconditioner", "ShampooSGD", "ShampooAdamW"]
@@ -51,14 +52,25 @@ class Preconditioner(PreconditionerBase):
         return newton_inverse_root(stat, exp, eps, getattr(self, '_v0', None)).to(stat.dtype)
 
 
-class ShampooSGD(ShampooSGDBase):
+class _Fused2(_FusedStep):
+    bank_keys = ('rect_t1', 'rect_t2', 'inv_root_mode')
+
+    @staticmethod
+    def bank_class():
+        from optimizers.engine2 import ShampooBank2
+        return ShampooBank2
+
+
+class ShampooSGD(_Fused2, ShampooSGDBase):
     preconditioner_class = Preconditioner
     extra_keys = ('rect_t1', 'rect_t2', 'inv_root_mode')
+    _update = staticmethod(_sgd_update)
 
     def __init__(self, params, lr=0.1, momentum=0.9, weight_decay=0.0, nesterov=False, start_prec_step=1,
                  stat_compute_steps=100, prec_compute_steps=500, stat_decay=0.95, matrix_eps=1e-6,
                  prec_maxorder=1200, prec_bits=32, min_lowbit_size=4096, quan_blocksize=64,
-                 rect_t1=1, rect_t2=4, inv_root_mode=0):
+                 rect_t1=1, rect_t2=4, inv_root_mode=0, fused=False):
+        self._init_fused(fused)
         super().__init__(params, lr=lr, momentum=momentum, weight_decay=weight_decay, nesterov=nesterov,
                          start_prec_step=start_prec_step, stat_compute_steps=stat_compute_steps,
                          prec_compute_steps=prec_compute_steps, stat_decay=stat_decay, matrix_eps=matrix_eps,
@@ -66,14 +78,16 @@ class ShampooSGD(ShampooSGDBase):
                          quan_blocksize=quan_blocksize, rect_t1=rect_t1, rect_t2=rect_t2, inv_root_mode=inv_root_mode)
 
 
-class ShampooAdamW(ShampooAdamWBase):
+class ShampooAdamW(_Fused2, ShampooAdamWBase):
     preconditioner_class = Preconditioner
     extra_keys = ('rect_t1', 'rect_t2', 'inv_root_mode')
+    _update = staticmethod(_adamw_update)
 
     def __init__(self, params, lr=0.001, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0, start_prec_step=1,
                  stat_compute_steps=100, prec_compute_steps=500, stat_decay=0.95, matrix_eps=1e-6,
                  prec_maxorder=1200, prec_bits=32, min_lowbit_size=4096, quan_blocksize=64,
-                 rect_t1=1, rect_t2=4, inv_root_mode=0):
+                 rect_t1=1, rect_t2=4, inv_root_mode=0, fused=False):
+        self._init_fused(fused)
         super().__init__(params, lr=lr, betas=betas, eps=eps, weight_decay=weight_decay,
                          start_prec_step=start_prec_step, stat_compute_steps=stat_compute_steps,
                          prec_compute_steps=prec_compute_steps, stat_decay=stat_decay, matrix_eps=matrix_eps,
@@ -85,5 +99,5 @@ _MORE = """
         rect_t1 (int): number of iterations t1 for rectification
         rect_t2 (int): number of iterations t2 for rectification
         inv_root_mode(int): "0" for SVD computation and "1" for Schur-Newton iteration"""
-ShampooSGD.__doc__ = _DOC.format(base="SGD", more=_MORE)
-ShampooAdamW.__doc__ = _DOC.format(base="AdamW", more=_MORE)
+ShampooSGD.__doc__ = _DOC.format(base="SGD", more=_MORE) + _FusedStep.__doc__
+ShampooAdamW.__doc__ = _DOC.format(base="AdamW", more=_MORE) + _FusedStep.__doc__
