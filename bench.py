@@ -76,21 +76,28 @@ STEP_KW = dict(stat_decay=0.95, matrix_eps=1e-6, prec_maxorder=1024, prec_bits=4
                quan_blocksize=64)
 
 
-def precond_step_gpu(torch):
-    """ms per full 4-bit Shampoo (statistics stored quantized, Newton inverse roots) + AdamW step over the
-    ViT-B/32 shapes: statistics every step, inverse 4th roots every 10th step, preconditioned and
-    norm-grafted update every step.  Ten untimed steps bring the preconditioners into use."""
-    from optimizers import shampoo1 as S1
+def precond_step_gpu(torch, variant="shampoo1"):
+    """ms per full 4-bit Shampoo + AdamW step over the ViT-B/32 shapes: statistics every step, inverse 4th
+    roots (coupled Newton) every 10th step, preconditioned and norm-grafted update every step.  Ten untimed
+    steps bring the preconditioners into use.  variant "shampoo1": the statistics themselves are stored
+    quantized; "shampoo2": their eigenvector matrices are (one subspace-iteration step per update).
+    Gradients cycle through four independent N(0, 0.02^2) sets, copied into fixed buffers between steps."""
+    import importlib
+    S = importlib.import_module("optimizers." + variant)
 
     g = torch.Generator(device="cuda").manual_seed(1)
     params = [torch.nn.Parameter(0.02 * torch.randn(s, device="cuda", generator=g)) for s in vit_b32_shapes()]
-    grads = [0.02 * torch.randn(p.shape, device="cuda", generator=g) for p in params]
-    opt = S1.ShampooAdamW(params, lr=1e-3, weight_decay=0.05, start_prec_step=1, stat_compute_steps=1,
-                          prec_compute_steps=10, fused=True, **STEP_KW)
-    for p, gr in zip(params, grads):
-        p.grad = gr
+    grad_sets = [[0.02 * torch.randn(p.shape, device="cuda", generator=g) for p in params] for _ in range(4)]
+    extra = dict(inv_root_mode=1) if variant == "shampoo2" else {}
+    opt = S.ShampooAdamW(params, lr=1e-3, weight_decay=0.05, start_prec_step=1, stat_compute_steps=1,
+                         prec_compute_steps=10, fused=True, **STEP_KW, **extra)
+    for p, gr in zip(params, grad_sets[0]):
+        p.grad = gr.clone()
+    calls = [0]
 
     def timed_step():
+        torch._foreach_copy_([p.grad for p in params], grad_sets[calls[0] % 4])
+        calls[0] += 1
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -114,11 +121,18 @@ def precond_step_gpu(torch):
         rows = [1024] * ((m - 1) // 1024) + [m - 1024 * ((m - 1) // 1024)]
         cols = [1024] * ((n - 1) // 1024) + [n - 1024 * ((n - 1) // 1024)]
         gram_flop += sum(2 * a * a * b + 2 * a * b * b for a in rows for b in cols)
+    more = {}
+    if variant == "shampoo2":
+        bank = next(iter(opt._fused_cache.values()))["bank"]
+        more["matrices_redone_with_library_qr"] = bank.qr_fallbacks
+        more["subspace_iteration_updates"] = 30 * sum(bank.per_order.values())
     return {
+        **more,
         "workload": "ViT-B/32 2-D weights (50 parameters, %d blocks of at most 1024, %d quantized statistics and as many "
                     "preconditioners), fp32 N(0,0.02^2) gradients, 4-bit linear-2 blocksize 64, beta 0.95, statistics "
                     "every step, coupled-Newton inverse 4th roots every 10th step, AdamW update; "
-                    "optimizers.shampoo1.ShampooAdamW(fused=True)" % (blocks, 2 * blocks, ),
+                    "optimizers.%s.ShampooAdamW(fused=True%s)" % (blocks, 2 * blocks, variant,
+                                                                   ", inv_root_mode=1" if variant == "shampoo2" else ""),
         "ms_per_step_regular": round(reg, 3),
         "ms_per_step_with_inverse_roots": round(new, 3),
         "ms_per_step_amortized_over_10": round((9 * reg + new) / 10, 3),
@@ -240,7 +254,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--section", choices=["all", "quant", "gemm", "step"], default="all",
+    ap.add_argument("--section", choices=["all", "quant", "gemm", "step", "step2"], default="all",
                     help="run only one part (for profiling one kernel family); the JSON line then lacks the others")
     ap.add_argument("--bank-streams", type=int, default=None,
                     help="side streams of the batched preconditioner engine (0 serialises its launches, which "
@@ -263,9 +277,14 @@ def main():
     if args.bank_streams is not None:
         from optimizers.engine import ShampooBank
         ShampooBank.DEFAULT_STREAMS = args.bank_streams
-    if args.section in ("gemm", "step"):
-        part = fused_gemm_gpu(torch, code) if args.section == "gemm" else precond_step_gpu(torch)
-        print(json.dumps({"section": args.section, "n_gpus": 1, ("fused_gemm" if args.section == "gemm" else "precond_step"): part}))
+    if args.section in ("gemm", "step", "step2"):
+        if args.section == "gemm":
+            part = {"fused_gemm": fused_gemm_gpu(torch, code)}
+        elif args.section == "step":
+            part = {"precond_step": precond_step_gpu(torch)}
+        else:
+            part = {"precond_step_shampoo2": precond_step_gpu(torch, "shampoo2")}
+        print(json.dumps({"section": args.section, "n_gpus": 1, **part}))
         return
     if args.section == "quant":
         args.no_step = args.no_cpu_baseline = True
@@ -361,6 +380,7 @@ def main():
     if not args.no_step:
         result["fused_gemm"] = fused_gemm_gpu(torch, code)
         result["precond_step"] = precond_step_gpu(torch)
+        result["precond_step_shampoo2"] = precond_step_gpu(torch, "shampoo2")
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch, x_slice, code_host)
         if not args.no_step:
