@@ -171,6 +171,23 @@ typedef struct {
  * (DENSE_T, DENSE, STORE|AXPBY_*), (DENSE, DENSE, STORE|AXPBY_DENSE|NEWTON); anything else is an error. */
 void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
 
+/* ---- batched Cholesky factorisation and triangular solve (Cholesky QR) ---------------------------
+ * Replace, for a whole stack of statistics at once, the QR factorisation the reference calls per
+ * matrix in QTensorSVDFast.quantize (torch.linalg.qr, qtensor/utils.py:157): one round of
+ *   G = Q^T Q (qtensor_hip_gemm, symmetric);  U = chol(G);  Q <- Q U^-1
+ * keeps span(Q[:, :k]) for every k, so repeating it until Q is orthonormal yields the Q factor.
+ * Stacks are contiguous [batch, n, n] fp32 with n a multiple of 64; everything runs on `stream`.
+ *
+ * cholesky_upper: gram (upper triangle read, contents destroyed) = U^T U.  u receives the block
+ *   rows of U on and above the diagonal (the part below the diagonal blocks is not written),
+ *   inv [batch, n/64, 64, 64] the inverses of U's diagonal blocks.  info[b] (zeroed by the caller)
+ *   is set to 1 when matrix b has a non-positive pivot (its factor is then meaningless but finite).
+ * solve_upper_right: x = q U^-1 for q, x [batch, rows, n] with u, inv from cholesky_upper;
+ *   panel is scratch of batch * rows * 64 floats.  x must not alias q. */
+void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float *inv, int *info, int n, int batch, qtensor_stream_t stream);
+void qtensor_hip_solve_upper_right_batched(const float *q, const float *u, const float *inv, float *panel, float *x,
+                                           int rows, int n, int batch, qtensor_stream_t stream);
+
 /* ---- the elementwise end of an optimizer step for all parameters at once -------------------------
  * Replaces the per-parameter torch calls of the reference's step():
  *   grafting   direction.mul_(grad.norm() / (direction.norm() + 1e-12))   optimizers/shampoo1.py:421, shampoo2.py:453

@@ -15,9 +15,10 @@ Here all statistics of one order form a stack and every line above is one or two
 the whole stack: the products run on the matrix cores through qtensor.fused.gemm (symmetric
 ones compute half and mirror), and the QR factorisation -- 20 ms per 1024 x 1024 matrix through
 the vendor's Householder routine, 5 s per step for a ViT-B/32 -- is replaced by a shifted
-Cholesky QR (rounds of  G = Q^T Q,  R = chol(G + s I),  Q <- Q R^-1  on the column-scaled
-matrix until Q is orthonormal), which yields the same factor Q up to column signs.  Matrices it
-cannot finish are redone with torch.linalg.qr.
+Cholesky QR (rounds of  G = Q^T Q,  U = chol(G + s I),  Q <- Q U^-1  on the column-scaled
+matrix until Q is orthonormal; the factorisation and the solve are blocked, batched launches of
+libqtensor_hip.so), which yields the same factor Q up to column signs.  Matrices it cannot
+finish are redone with torch.linalg.qr.
 """
 import torch
 
@@ -29,32 +30,24 @@ from qtensor import fused as X
 _householder_qr = torch.linalg.qr
 
 
-def _fenced(fn, *args, **kwargs):
-    """Call a torch.linalg routine with the device idle before and after.  On this PyTorch-ROCm
-    build a chain  solve_triangular -> matmul -> cholesky_ex  issued back to back on one stream
-    returns wrong factors now and then (torch-only reproduction: the second cholesky_ex of such a
-    chain reports a non-positive minor for a well-conditioned matrix; any synchronisation in between
-    cures it), so these calls are not trusted to be stream-ordered."""
-    torch.cuda.synchronize()
-    out = fn(*args, **kwargs)
-    torch.cuda.synchronize()
-    return out
-
-
 def cholesky_qr(Y, max_rounds=12, shift=1e-3, tolerance=2e-5):
     """Orthonormal Q [B, n, n] with span(Q[:, :, :k]) == span(Y[:, :, :k]) for every k (the Q factor
-    of a QR factorisation with positive diagonal of R), by rounds of  G = Q^T Q,  R = chol(G + s I),
-    Q <- Q R^-1  on the column-scaled matrix; every R is upper triangular, so the nested spans
+    of a QR factorisation with positive diagonal of R), by rounds of  G = Q^T Q,  U = chol(G + s I),
+    Q <- Q U^-1  on the column-scaled matrix; every U is upper triangular, so the nested spans
     survive each round.  A matrix far from orthonormal (||G - I||_F >= 0.5) gets the shift s, which
     lifts its small singular values by 1 / sqrt(s) per round -- a numerically singular Y ends, like
     with Householder reflections, in a completion fixed by rounding noise; once ||G - I||_F < 0.5 an
     unshifted round finishes it.  Matrices that are not orthonormal to `tolerance` (max |G - I|)
-    after max_rounds go through torch.linalg.qr.  Returns (Q, number of those)."""
+    after max_rounds go through torch.linalg.qr.  n must be a multiple of 64.
+    Returns (Q, number of matrices redone by the library)."""
     B, n, _ = Y.shape
     scale = torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)
     Q = (Y / scale).contiguous()                  # unit columns: the Gram matrix has a unit diagonal
-    failed = torch.zeros(B, dtype=torch.bool, device=Y.device)
-    done = failed
+    other = torch.empty_like(Q)
+    U, inv = torch.empty_like(Q), torch.empty(B, n // 64, 64, 64, device=Y.device)
+    panel = torch.empty(B, n, 64, device=Y.device)
+    info = torch.zeros(B, dtype=torch.int32, device=Y.device)
+    done = None
     for _ in range(max_rounds + 1):
         gram = X.gemm(Q, Q, trans_a=True, symmetric=True)
         diag = gram.diagonal(dim1=1, dim2=2)
@@ -64,12 +57,14 @@ def cholesky_qr(Y, max_rounds=12, shift=1e-3, tolerance=2e-5):
             break
         far = ~(torch.linalg.matrix_norm(gram) < 0.5)
         diag.add_(1.0 + shift * far.to(gram.dtype).unsqueeze(1))
-        R, info = _fenced(torch.linalg.cholesky_ex, gram, upper=True)
-        failed = failed | (info != 0)
-        Q = _fenced(torch.linalg.solve_triangular, R, Q, upper=True, left=False).contiguous()
-    redo = torch.nonzero(failed | ~done).flatten()
+        X.cholesky_upper(gram, U, inv, info)
+        X.solve_upper_right(Q, U, inv, panel, other)
+        Q, other = other, Q
+    redo = torch.nonzero((info != 0) | ~done).flatten()
     if redo.numel():
-        Q[redo] = _fenced(_householder_qr, Y[redo])[0]
+        torch.cuda.synchronize()                  # the library routine is not trusted to be stream-ordered here
+        Q[redo] = _householder_qr(Y[redo])[0]
+        torch.cuda.synchronize()
     return Q, int(redo.numel())
 
 

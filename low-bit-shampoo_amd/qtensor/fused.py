@@ -272,3 +272,41 @@ def dequantize_stack(q: Quantized, out: Optional[Tensor] = None, outdtype=torch.
     F._call(F.lib.qtensor_hip_dequantize_batched, out.device, q.codes.data_ptr(), q.code.data_ptr(), q.bits, q.order,
             q.batch, q.absmax.data_ptr(), None if q.diag is None else q.diag.data_ptr(), out.data_ptr(), slot, q.blocksize)
     return out
+
+
+# --------------------------------------------------------------------------- Cholesky QR pieces
+if F.lib is not None:
+    F.lib.qtensor_hip_cholesky_upper_batched.restype = None
+    F.lib.qtensor_hip_cholesky_upper_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int,
+                                                         ct.c_void_p]
+    F.lib.qtensor_hip_solve_upper_right_batched.restype = None
+    F.lib.qtensor_hip_solve_upper_right_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int,
+                                                            ct.c_int, ct.c_int, ct.c_void_p]
+
+
+def _stack(t: Tensor, name: str, shape=None) -> Tensor:
+    if not t.is_cuda or t.dtype != torch.float32 or not t.is_contiguous() or (shape is not None and tuple(t.shape) != tuple(shape)):
+        raise ValueError(f"{name} must be a contiguous fp32 GPU tensor" + (f" of shape {tuple(shape)}" if shape else ""))
+    return t
+
+
+def cholesky_upper(gram: Tensor, u: Tensor, inv: Tensor, info: Tensor) -> None:
+    """gram [B, n, n] (destroyed) = U^T U: block rows of U into u, inverses of its 64 x 64 diagonal blocks
+    into inv [B, n/64, 64, 64]; info int32 [B] (zeroed by the caller) flags non-positive pivots."""
+    B, n, _ = gram.shape
+    _stack(gram, "gram", (B, n, n)), _stack(u, "u", (B, n, n)), _stack(inv, "inv", (B, n // 64, 64, 64))
+    if info.dtype != torch.int32 or info.numel() != B or not info.is_cuda:
+        raise ValueError("info must be an int32 GPU vector with one entry per matrix")
+    F._call(F.lib.qtensor_hip_cholesky_upper_batched, gram.device, gram.data_ptr(), u.data_ptr(), inv.data_ptr(), info.data_ptr(), n, B)
+
+
+def solve_upper_right(q: Tensor, u: Tensor, inv: Tensor, panel: Tensor, out: Tensor) -> Tensor:
+    """out = q U^-1 for q [B, rows, n] with u, inv from cholesky_upper; panel: scratch [B, rows, 64]."""
+    B, rows, n = q.shape
+    _stack(q, "q"), _stack(u, "u", (B, n, n)), _stack(inv, "inv", (B, n // 64, 64, 64))
+    _stack(panel, "panel", (B, rows, 64)), _stack(out, "out", (B, rows, n))
+    if out.data_ptr() == q.data_ptr():
+        raise ValueError("out must not alias q")
+    F._call(F.lib.qtensor_hip_solve_upper_right_batched, q.device, q.data_ptr(), u.data_ptr(), inv.data_ptr(), panel.data_ptr(),
+            out.data_ptr(), rows, n, B)
+    return out

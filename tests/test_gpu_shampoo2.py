@@ -30,6 +30,41 @@ def mods():
     return S2, E2
 
 
+@pytest.mark.parametrize("n,batch,rows", [(64, 3, 64), (256, 4, 256), (768, 2, 100)])
+def test_blocked_cholesky_and_right_solve_against_float64(mods, n, batch, rows):
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(n)
+    A = torch.randn(batch, n, n, generator=g)
+    G = (A.transpose(1, 2) @ A / n + 0.1 * torch.eye(n)).cuda()
+    gram, U = G.clone(), torch.full((batch, n, n), 7.0, device="cuda")
+    inv = torch.empty(batch, n // 64, 64, 64, device="cuda")
+    info = torch.zeros(batch, dtype=torch.int32, device="cuda")
+    X.cholesky_upper(gram, U, inv, info)
+    assert info.tolist() == [0] * batch
+    blocks = torch.arange(n) // 64
+    keep = (blocks[:, None] <= blocks[None, :]).cuda()            # block rows on and above the diagonal are written
+    Ut = torch.where(keep, U, torch.zeros_like(U)).double()
+    assert bool((torch.tril(Ut, -1) == 0).all())
+    want = torch.linalg.cholesky(G.double().cpu(), upper=True)
+    assert rel(Ut, want) <= 1e-5
+    for j in range(n // 64):
+        blk = want[:, 64 * j:64 * j + 64, 64 * j:64 * j + 64]
+        assert rel(inv[:, j], torch.linalg.inv(blk)) <= 1e-4
+    Q = torch.randn(batch, rows, n, generator=g).cuda()
+    out = torch.empty_like(Q)
+    X.solve_upper_right(Q, U, inv, torch.empty(batch, rows, 64, device="cuda"), out)
+    assert rel(out, torch.linalg.solve_triangular(want, Q.double().cpu(), upper=True, left=False)) <= 1e-4
+    # a non-positive pivot is flagged, and only for its matrix
+    bad = G.clone()
+    bad[0, 5, 5] = -1.0
+    info.zero_()
+    X.cholesky_upper(bad, U, inv, info)
+    assert info.tolist() == [1] + [0] * (batch - 1) and bool(torch.isfinite(U[keep.expand_as(U)]).all())
+    with pytest.raises((RuntimeError, ValueError)):
+        X.cholesky_upper(torch.zeros(1, 100, 100, device="cuda"), torch.zeros(1, 100, 100, device="cuda"),
+                         torch.zeros(1, 1, 64, 64, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda"))
+
+
 def test_cholesky_qr_gives_the_householder_factor_up_to_signs(mods):
     _, E2 = mods
     g = torch.Generator().manual_seed(3)
