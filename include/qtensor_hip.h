@@ -181,7 +181,7 @@ void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
  * cholesky_upper: gram (upper triangle read, contents destroyed) = U^T U.  u receives the block
  *   rows of U on and above the diagonal (the part below the diagonal blocks is not written),
  *   inv [batch, n/64, 64, 64] the inverses of U's diagonal blocks.  info[b] (zeroed by the caller)
- *   is set to 1 when matrix b has a non-positive pivot (its factor is then meaningless but finite).
+ *   is set to 1 when matrix b has a non-positive pivot (its factor is then meaningless).
  * solve_upper_right: x = q U^-1 for q, x [batch, rows, n] with u, inv from cholesky_upper;
  *   panel is scratch of batch * rows * 64 floats.  x must not alias q. */
 void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float *inv, int *info, int n, int batch, qtensor_stream_t stream);

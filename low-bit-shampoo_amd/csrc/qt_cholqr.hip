@@ -21,48 +21,58 @@ namespace {
 constexpr int NB = 64;
 
 // One wave per matrix: upper Cholesky factor U (G = U^T U) of a 64 x 64 block and U^-1.
-// Reads the upper triangle of G only.  A non-positive pivot sets info[b] = 1 and is replaced by 1
-// so that everything stays finite.
+// Reads the upper triangle of G only.  A non-positive (or NaN) pivot sets info[b] = 1 and is
+// replaced by 1; the factor of that matrix is then meaningless.
+//
+// Lane i keeps row i of the (full, symmetric) trailing matrix in registers.  Because the matrix
+// stays symmetric, column k of step k is row k, i.e. the registers of lane k: they are broadcast
+// with v_readlane, so the whole factorisation and the inversion of the factor run without LDS
+// traffic or barriers (LDS only stages the block on the way in).
+__device__ __forceinline__ float lane_value(float x, int lane) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(x), lane));
+}
+
 __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long long g_stride, int ldg, float *u,
                                                         long long u_stride, int ldu, float *inv, long long inv_stride,
                                                         int *info) {
-    __shared__ float a[NB][NB + 1];      // lower factor L = U^T, built in place
-    __shared__ float m[NB][NB + 1];      // L^-1
+    __shared__ float stage[NB][NB + 1];
     const int b = blockIdx.x, lane = threadIdx.x;
     const float *G = gram + (long long)b * g_stride;
-    for (int r = 0; r < NB; ++r) a[r][lane] = G[(long long)r * ldg + lane];
+    for (int r = 0; r < NB; ++r) stage[r][lane] = G[(long long)r * ldg + lane];
     __syncthreads();
-    for (int r = 0; r < NB; ++r)
-        if (r > lane) a[r][lane] = a[lane][r];           // mirror the upper triangle
-    __syncthreads();
+    float row[NB];                               // row `lane` of the symmetric matrix; ends as row `lane` of L = U^T
+#pragma unroll
+    for (int j = 0; j < NB; ++j) row[j] = j >= lane ? stage[lane][j] : stage[j][lane];
     bool ok = true;
+#pragma unroll
     for (int k = 0; k < NB; ++k) {
-        float d = a[k][k];
+        float d = lane_value(row[k], k);
         if (!(d > 0.0f)) { ok = false; d = 1.0f; }
-        const float root = sqrtf(d);
-        const float lik = lane > k ? a[lane][k] / root : 0.0f;
-        __syncthreads();
-        if (lane == k) a[k][k] = root;
-        if (lane > k) a[lane][k] = lik;
-        __syncthreads();
-        for (int j = k + 1; j < NB; ++j)
-            if (j <= lane) a[lane][j] -= lik * a[j][k];
-        __syncthreads();
+        const float scale = 1.0f / sqrtf(d);
+        const float lik = row[k] * scale;        // L[lane][k] (lanes above k: unused values)
+#pragma unroll
+        for (int j = k + 1; j < NB; ++j) {
+            const float ljk = lane_value(row[j], k) * scale;     // L[j][k] from row k
+            row[j] -= lik * ljk;
+        }
+        row[k] = lik;
     }
-    // column `lane` of L^-1 by forward substitution
+    // column `lane` of L^-1 by forward substitution; L[i][k] sits in lane i
+    float x[NB];
+#pragma unroll
     for (int i = 0; i < NB; ++i) {
         float s = i == lane ? 1.0f : 0.0f;
-        for (int k = 0; k < i; ++k)
-            if (k >= lane) s -= a[i][k] * m[k][lane];
-        m[i][lane] = i >= lane ? s / a[i][i] : 0.0f;
+#pragma unroll
+        for (int k = 0; k < i; ++k) s -= lane_value(row[k], i) * x[k];
+        x[i] = i >= lane ? s / lane_value(row[i], i) : 0.0f;
     }
-    __syncthreads();
     float *U = u + (long long)b * u_stride;
-    float *I = inv + (long long)b * inv_stride;
-    for (int r = 0; r < NB; ++r) {
-        U[(long long)r * ldu + lane] = r <= lane ? a[lane][r] : 0.0f;     // U = L^T
-        I[r * NB + lane] = r <= lane ? m[lane][r] : 0.0f;                 // U^-1 = (L^-1)^T
-    }
+    float *I = inv + (long long)b * inv_stride + lane * NB;
+#pragma unroll
+    for (int r = 0; r < NB; ++r) U[(long long)r * ldu + lane] = r <= lane ? row[r] : 0.0f;        // U[r][lane] = L[lane][r]
+#pragma unroll
+    for (int c = 0; c < NB; c += 4)              // U^-1[lane][c] = L^-1[c][lane] = x[c] of this lane
+        *reinterpret_cast<float4 *>(I + c) = make_float4(x[c], x[c + 1], x[c + 2], x[c + 3]);
     if (!ok && lane == 0) info[b] = 1;
 }
 

@@ -27,45 +27,7 @@ from optimizers.matrix_functions import ComputePowerBatched
 from qtensor import fused as X
 
 
-_householder_qr = torch.linalg.qr
-
-
-def cholesky_qr(Y, max_rounds=12, shift=1e-3, tolerance=2e-5):
-    """Orthonormal Q [B, n, n] with span(Q[:, :, :k]) == span(Y[:, :, :k]) for every k (the Q factor
-    of a QR factorisation with positive diagonal of R), by rounds of  G = Q^T Q,  U = chol(G + s I),
-    Q <- Q U^-1  on the column-scaled matrix; every U is upper triangular, so the nested spans
-    survive each round.  A matrix far from orthonormal (||G - I||_F >= 0.5) gets the shift s, which
-    lifts its small singular values by 1 / sqrt(s) per round -- a numerically singular Y ends, like
-    with Householder reflections, in a completion fixed by rounding noise; once ||G - I||_F < 0.5 an
-    unshifted round finishes it.  Matrices that are not orthonormal to `tolerance` (max |G - I|)
-    after max_rounds go through torch.linalg.qr.  n must be a multiple of 64.
-    Returns (Q, number of matrices redone by the library)."""
-    B, n, _ = Y.shape
-    scale = torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)
-    Q = (Y / scale).contiguous()                  # unit columns: the Gram matrix has a unit diagonal
-    other = torch.empty_like(Q)
-    U, inv = torch.empty_like(Q), torch.empty(B, n // 64, 64, 64, device=Y.device)
-    panel = torch.empty(B, n, 64, device=Y.device)
-    info = torch.zeros(B, dtype=torch.int32, device=Y.device)
-    done = None
-    for _ in range(max_rounds + 1):
-        gram = X.gemm(Q, Q, trans_a=True, symmetric=True)
-        diag = gram.diagonal(dim1=1, dim2=2)
-        diag.sub_(1.0)
-        done = gram.abs().amax(dim=(1, 2)) < tolerance                         # False for NaN as well
-        if bool(done.all()):                                                   # host synchronisation
-            break
-        far = ~(torch.linalg.matrix_norm(gram) < 0.5)
-        diag.add_(1.0 + shift * far.to(gram.dtype).unsqueeze(1))
-        X.cholesky_upper(gram, U, inv, info)
-        X.solve_upper_right(Q, U, inv, panel, other)
-        Q, other = other, Q
-    redo = torch.nonzero((info != 0) | ~done).flatten()
-    if redo.numel():
-        torch.cuda.synchronize()                  # the library routine is not trusted to be stream-ordered here
-        Q[redo] = _householder_qr(Y[redo])[0]
-        torch.cuda.synchronize()
-    return Q, int(redo.numel())
+cholesky_qr = X.cholesky_qr
 
 
 class ShampooBank2(ShampooBank):
