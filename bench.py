@@ -125,6 +125,7 @@ def precond_step_gpu(torch, variant="shampoo1"):
     if variant == "shampoo2":
         bank = next(iter(opt._fused_cache.values()))["bank"]
         more["matrices_redone_with_library_qr"] = bank.qr_fallbacks
+        more["cholesky_qr_rounds_per_stack_and_update"] = round(bank.qr_rounds / (30 * len(bank.per_order)), 2)
         more["subspace_iteration_updates"] = 30 * sum(bank.per_order.values())
     return {
         **more,

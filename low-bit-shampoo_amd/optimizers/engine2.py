@@ -93,11 +93,28 @@ class ShampooBank2(ShampooBank):
                 X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, out=seg, symmetric=True)
             return run
 
+        def project(order):
+            def run():
+                solver[order] = X.CholeskyQR(X.gemm(stat[order], basis[order], trans_b=True))     # L Vt^T
+            return run
+
+        def check(order):
+            return lambda: None if solver[order].finished else solver[order].check()
+
+        def poll(order):
+            return lambda: None if solver[order].finished else solver[order].poll()
+
+        def advance(order):
+            return lambda: None if solver[order].finished else solver[order].advance()
+
+        self.qr_rounds = getattr(self, "qr_rounds", 0)
+
         def iterate(order):
             def run():
-                L, vt = stat[order], basis[order]
-                Q, redone = cholesky_qr(X.gemm(L, vt, trans_b=True))
+                L = stat[order]
+                Q, redone = solver[order].result()
                 self.qr_fallbacks += redone
+                self.qr_rounds += solver[order].rounds
                 quotients = (Q * X.gemm(L, Q)).sum(dim=1)                      # diag(Q^T L Q)
                 ascending, where = torch.sort(quotients, dim=1)
                 half = self.keep[order].shape[1]
@@ -109,6 +126,14 @@ class ShampooBank2(ShampooBank):
 
         self._fan_out([rebuild(o) for o in orders])
         self._fan_out([accumulate(g, side) for g in self.groups for side in (0, 1)])
+        # The Cholesky QR of every order advances on its own stream; the host waits once per round.
+        # (_fan_out gives job i the stream i % streams, so an order keeps its stream from call to call.)
+        solver = {}
+        self._fan_out([project(o) for o in orders])
+        while not all(solver[o].finished for o in orders):
+            self._fan_out([check(o) for o in orders])
+            self._fan_out([poll(o) for o in orders])
+            self._fan_out([advance(o) for o in orders])
         self._fan_out([iterate(o) for o in orders])
 
     @torch.no_grad()

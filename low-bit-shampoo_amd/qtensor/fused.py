@@ -315,50 +315,115 @@ def solve_upper_right(q: Tensor, u: Tensor, inv: Tensor, panel: Tensor, out: Ten
 _householder_qr = torch.linalg.qr
 
 
-def cholesky_qr(Y, max_rounds=12, shift=1e-3, tolerance=2e-5):
+class CholeskyQR:
     """Orthonormal Q [B, n, n] with span(Q[:, :, :k]) == span(Y[:, :, :k]) for every k (the Q factor
     of a QR factorisation with positive diagonal of R), by rounds of  G = Q^T Q,  U = chol(G + s I),
     Q <- Q U^-1  on the column-scaled matrix; every U is upper triangular, so the nested spans
     survive each round.  A matrix far from orthonormal (||G - I||_F >= 0.5) gets the shift s, which
     lifts its small singular values by 1 / sqrt(s) per round -- a numerically singular Y ends, like
-    with Householder reflections, in a completion fixed by rounding noise; once ||G - I||_F < 0.5 an
-    unshifted round finishes it.  Matrices that are not orthonormal to `tolerance` (max |G - I|)
-    after max_rounds go through torch.linalg.qr.  Orders that are not a multiple of 64 are padded with
-    an identity block (QR of diag(Y, I) is diag(Q, I)).
-    Returns (Q, number of matrices redone by the library)."""
-    if Y.dim() != 3 or Y.shape[1] != Y.shape[2] or Y.dtype != torch.float32 or not Y.is_cuda:
-        raise ValueError("cholesky_qr takes an fp32 GPU stack [B, n, n]")
-    B, true_n, _ = Y.shape
-    if true_n % 64:
-        n = -(-true_n // 64) * 64
-        padded = torch.zeros(B, n, n, device=Y.device)
-        padded[:, :true_n, :true_n] = Y
-        padded.diagonal(dim1=1, dim2=2)[:, true_n:] = 1.0
-        Q, redone = cholesky_qr(padded, max_rounds, shift, tolerance)
-        return Q[:, :true_n, :true_n].contiguous(), redone
-    n = true_n
-    scale = torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)
-    Q = (Y / scale).contiguous()                  # unit columns: the Gram matrix has a unit diagonal
-    other = torch.empty_like(Q)
-    U, inv = torch.empty_like(Q), torch.empty(B, n // 64, 64, 64, device=Y.device)
-    panel = torch.empty(B, n, 64, device=Y.device)
-    info = torch.zeros(B, dtype=torch.int32, device=Y.device)
-    done = None
-    for _ in range(max_rounds + 1):
-        gram = gemm(Q, Q, trans_a=True, symmetric=True)
-        diag = gram.diagonal(dim1=1, dim2=2)
-        diag.sub_(1.0)
-        done = gram.abs().amax(dim=(1, 2)) < tolerance                         # False for NaN as well
-        if bool((done | (info != 0)).all()):                                   # host synchronisation
-            break
-        far = ~(torch.linalg.matrix_norm(gram) < 0.5)
-        diag.add_(1.0 + shift * far.to(gram.dtype).unsqueeze(1))
-        cholesky_upper(gram, U, inv, info)
-        solve_upper_right(Q, U, inv, panel, other)
-        Q, other = other, Q
-    redo = torch.nonzero((info != 0) | ~done).flatten()
-    if redo.numel():
-        torch.cuda.synchronize()                  # the library routine is not trusted to be stream-ordered here
-        Q[redo] = _householder_qr(Y[redo])[0]
-        torch.cuda.synchronize()
-    return Q, int(redo.numel())
+    with Householder reflections, in a completion fixed by rounding noise.  Once ||G - I||_F < 0.5
+    (all singular values of Q within [0.7, 1.23]) one unshifted round makes Q orthonormal to fp32
+    rounding and the matrix leaves the working set; matrices that still are far after max_rounds, or
+    whose factorisation hits a non-positive pivot, go through torch.linalg.qr.  Orders that are not
+    a multiple of 64 are padded with an identity block (QR of diag(Y, I) is diag(Q, I)).
+
+    The object is a small state machine so that several stacks can advance on their own streams while
+    the host waits only once per round for all of them:  check() enqueues the orthonormality test,
+    poll() reads its outcome (the only host synchronisation), advance() enqueues one round for the
+    matrices still in the working set, result() returns (Q, number of matrices redone by the
+    library).  All calls for one object must be made with the same current stream."""
+
+    def __init__(self, Y, max_rounds=12, shift=1e-3, tolerance=2e-5):
+        if Y.dim() != 3 or Y.shape[1] != Y.shape[2] or Y.dtype != torch.float32 or not Y.is_cuda:
+            raise ValueError("CholeskyQR takes an fp32 GPU stack [B, n, n]")
+        B, self.true_n, _ = Y.shape
+        n = -(-self.true_n // 64) * 64
+        if n != self.true_n:
+            padded = torch.zeros(B, n, n, device=Y.device)
+            padded[:, :self.true_n, :self.true_n] = Y
+            padded.diagonal(dim1=1, dim2=2)[:, self.true_n:] = 1.0
+            Y = padded
+        self.Y, self.shift, self.tolerance, self.rounds_left = Y, shift, tolerance, max_rounds
+        scale = torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)
+        self.Q = (Y / scale).contiguous()             # working set; unit columns: the Gram matrix has a unit diagonal
+        self.ids = torch.arange(B, device=Y.device)   # which matrix of the stack each working-set entry is
+        self.U, self.inv = torch.empty_like(self.Q), torch.empty(B, n // 64, 64, 64, device=Y.device)
+        self.panel = torch.empty(B, n, 64, device=Y.device)
+        self.info = torch.zeros(B, dtype=torch.int32, device=Y.device)
+        self.final = torch.empty_like(self.Q)
+        self.redo = []                                # matrices handed to the library at the end
+        self.finished = False
+        self.rounds = 0                               # factorisation rounds enqueued so far
+        self.gram = self.flags = self.near = None
+
+    def _keep(self, keep):
+        """Shrink the working set to the entries of the host mask `keep`."""
+        if bool(keep.all()):
+            return
+        index = torch.nonzero(keep).flatten().to(self.Q.device)
+        self.Q, self.ids = self.Q[index], self.ids[index]
+        if self.gram is not None:
+            self.gram = self.gram[index]
+
+    def check(self):
+        k = self.Q.shape[0]
+        self.gram = gemm(self.Q, self.Q, trans_a=True, symmetric=True)
+        self.gram.diagonal(dim1=1, dim2=2).sub_(1.0)
+        done = self.gram.abs().amax(dim=(1, 2)) < self.tolerance                # False for NaN as well
+        near = torch.linalg.matrix_norm(self.gram) < 0.5
+        self.flags = torch.stack([done, near, self.info[:k] != 0])
+
+    def poll(self):
+        done, near, failed = self.flags.cpu()                                   # the host synchronisation
+        if self.rounds_left == 0:
+            failed = failed | ~done
+        done = done & ~failed
+        if bool(failed.any()):
+            self.redo += self.ids[failed.to(self.Q.device)].tolist()
+        if bool(done.any()):
+            sel = done.to(self.Q.device)
+            self.final[self.ids[sel]] = self.Q[sel]
+        keep = ~(done | failed)
+        self.near = near[keep]
+        self._keep(keep)
+        self.finished = self.Q.shape[0] == 0
+        return self.finished
+
+    def advance(self):
+        k = self.Q.shape[0]
+        near = self.near.to(self.Q.device)
+        self.gram.diagonal(dim1=1, dim2=2).add_(1.0 + self.shift * (~near).to(self.gram.dtype).unsqueeze(1))
+        self.info[:k].zero_()
+        cholesky_upper(self.gram, self.U[:k], self.inv[:k], self.info[:k])
+        out = torch.empty_like(self.Q)
+        solve_upper_right(self.Q, self.U[:k], self.inv[:k], self.panel[:k], out)
+        self.Q, self.gram = out, None
+        self.rounds_left -= 1
+        self.rounds += 1
+        if bool(self.near.any()):
+            # ||G - I||_F < 0.5 before an unshifted round: G was positive definite with eigenvalues in
+            # (0.5, 1.5), the round cannot fail and leaves Q orthonormal to rounding
+            self.final[self.ids[near]] = self.Q[near]
+            self._keep(~self.near)
+            self.finished = self.Q.shape[0] == 0
+
+    def result(self):
+        if self.redo:
+            redo = torch.tensor(self.redo, device=self.Y.device)
+            torch.cuda.synchronize()              # the library routine is not trusted to be stream-ordered here
+            self.final[redo] = _householder_qr(self.Y[redo])[0]
+            torch.cuda.synchronize()
+        Q = self.final
+        if Q.shape[1] != self.true_n:
+            Q = Q[:, :self.true_n, :self.true_n].contiguous()
+        return Q, len(self.redo)
+
+
+def cholesky_qr(Y, max_rounds=12, shift=1e-3, tolerance=2e-5):
+    """(Q, number of matrices redone by the library) for one stack; see CholeskyQR."""
+    state = CholeskyQR(Y, max_rounds, shift, tolerance)
+    while not state.finished:
+        state.check()
+        if not state.poll():
+            state.advance()
+    return state.result()
