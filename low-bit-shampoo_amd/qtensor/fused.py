@@ -319,8 +319,9 @@ class CholeskyQR:
     """Orthonormal Q [B, n, n] with span(Q[:, :, :k]) == span(Y[:, :, :k]) for every k (the Q factor
     of a QR factorisation with positive diagonal of R), by rounds of  G = Q^T Q,  U = chol(G + s I),
     Q <- Q U^-1  on the column-scaled matrix; every U is upper triangular, so the nested spans
-    survive each round.  A matrix far from orthonormal (||G - I||_F >= 0.5) gets the shift s, which
-    lifts its small singular values by 1 / sqrt(s) per round -- a numerically singular Y ends, like
+    survive each round.  A matrix far from orthonormal (||G - I||_F >= 0.5) gets the shift s (a few
+    times the rounding error of an fp32 Gram matrix of unit columns, so that G + s I stays positive
+    definite), which lifts its small singular values by 1 / sqrt(s) per round -- a numerically singular Y ends, like
     with Householder reflections, in a completion fixed by rounding noise.  Once ||G - I||_F < 0.5
     (all singular values of Q within [0.7, 1.23]) one unshifted round makes Q orthonormal to fp32
     rounding and the matrix leaves the working set; matrices that still are far after max_rounds, or
@@ -333,7 +334,7 @@ class CholeskyQR:
     matrices still in the working set, result() returns (Q, number of matrices redone by the
     library).  All calls for one object must be made with the same current stream."""
 
-    def __init__(self, Y, max_rounds=12, shift=1e-3, tolerance=2e-5):
+    def __init__(self, Y, max_rounds=12, shift=2e-4, tolerance=2e-5):
         if Y.dim() != 3 or Y.shape[1] != Y.shape[2] or Y.dtype != torch.float32 or not Y.is_cuda:
             raise ValueError("CholeskyQR takes an fp32 GPU stack [B, n, n]")
         B, self.true_n, _ = Y.shape
@@ -419,7 +420,7 @@ class CholeskyQR:
         return Q, len(self.redo)
 
 
-def cholesky_qr(Y, max_rounds=12, shift=1e-3, tolerance=2e-5):
+def cholesky_qr(Y, max_rounds=12, shift=2e-4, tolerance=2e-5):
     """(Q, number of matrices redone by the library) for one stack; see CholeskyQR."""
     state = CholeskyQR(Y, max_rounds, shift, tolerance)
     while not state.finished:
