@@ -14,10 +14,11 @@
 //              Newton: C = acc, T = (1 - w) I + w * acc, err = max |acc - I|.
 //
 // Tiling: workgroup = 4 waves in a 2 x 2 grid, block tile BM x BN x 16, each wave owns
-// (BM/2) x (BN/2) as 32 x 32 MFMA blocks.  Both operand tiles sit in LDS k-major ([k][row], row
-// stride rows + 4) so the per-lane fragment reads (row = lane % 32, k = lane / 32) are
-// consecutive words and row-contiguous sources are written with 16-byte stores.  Global loads
-// run two tiles ahead of the MFMAs; the LDS commit sits in the middle of the MFMA stream.
+// (BM/2) x (BN/2) as 32 x 32 MFMA blocks.  An operand tile sits in LDS the way its source is
+// contiguous -- [row][k] (stride 20) when k is, [k][row] (stride rows + 4) otherwise -- so every
+// commit is a 16-byte store; fragments come out as one 16-byte read per four MFMA steps or as
+// consecutive words per step.  Global loads run two tiles ahead of the MFMAs; the LDS commit sits
+// in the middle of the MFMA stream.
 #include "qt_common.h"
 
 #include <cmath>
@@ -67,7 +68,9 @@ namespace {
 
 constexpr int BK = 16;
 constexpr uint32_t kDies = 8;          // accelerator dies (XCDs) of an MI355X
-constexpr int LDS_PAD = 4;   // row stride = rows + 4 floats: k-major tiles, 16-byte aligned rows
+constexpr int LDS_PAD = 4;   // k-major tiles ([k][row]): row stride = rows + 4 floats, 16-byte aligned rows
+constexpr int LDK = BK + 4;  // row-major tiles ([row][k], for sources whose k is contiguous): 20 floats per row, so
+                             // that the 16-byte fragment reads of 8 consecutive lanes cover all 32 banks
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 // Pointers that arrive inside a by-value struct or from a pointer table are "generic" to the
 // compiler, which then emits flat_* instructions (slower, and they also count on the LDS wait
@@ -139,13 +142,30 @@ __device__ __forceinline__ void dequant_four(const uint8_t *codes, const float *
 // Dense, k contiguous in memory: element (row, k) at base[row * ld + k].
 template <int ROWS>
 struct LoadKContig {
+    static constexpr bool kRowMajor = true;                  // lands in LDS as [row][k]
     static constexpr int VEC = ROWS * BK / 4 / 256;          // float4 per thread
     float4 v[VEC];
+    int off[VEC];
+    // Fast path (whole k tiles, 16-byte aligned rows): per-thread offsets are fixed for the whole
+    // product, rows beyond the matrix are clamped (their results are never stored), and a tile
+    // load is `uniform tile base + offset` with no predicate.
+    __device__ __forceinline__ void prepare(int ld, int row0, int rows) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const int f = threadIdx.x + i * 256;
+            const int r = f / (BK / 4), kq = (f % (BK / 4)) << 2;
+            off[i] = min(row0 + r, rows - 1) * ld + kq;
+        }
+    }
+    __device__ __forceinline__ void fetch_fast(const float *tile_base) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = gload4(tile_base + off[i]);
+    }
     __device__ __forceinline__ void fetch(const float *base, int ld, int row0, int k0, int rows, int K, bool vec_ok) {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const int f = threadIdx.x + i * 256;
-            const int r = f >> 2, kq = (f & 3) << 2;
+            const int r = f / (BK / 4), kq = (f % (BK / 4)) << 2;
             const int gr = row0 + r, gk = k0 + kq;
             float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
             if (gr < rows) {
@@ -162,13 +182,11 @@ struct LoadKContig {
         }
     }
     __device__ __forceinline__ void commit(float *lds, const float *) const {
-        constexpr int LD = ROWS + LDS_PAD;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
             const int f = threadIdx.x + i * 256;
-            const int r = f >> 2, kq = (f & 3) << 2;
-            float *d = lds + kq * LD + r;
-            d[0] = v[i].x; d[LD] = v[i].y; d[2 * LD] = v[i].z; d[3 * LD] = v[i].w;
+            const int r = f / (BK / 4), kq = (f % (BK / 4)) << 2;
+            *reinterpret_cast<float4 *>(lds + r * LDK + kq) = v[i];
         }
     }
 };
@@ -176,8 +194,22 @@ struct LoadKContig {
 // Dense, row index contiguous in memory: element (row, k) at base[k * ld + row].
 template <int ROWS>
 struct LoadRowContig {
+    static constexpr bool kRowMajor = false;                 // lands in LDS as [k][row]
     static constexpr int VEC = ROWS * BK / 4 / 256;
     float4 v[VEC];
+    int off[VEC];
+    __device__ __forceinline__ void prepare(int ld, int row0, int rows) {      // rows is a multiple of 4 here
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const int f = threadIdx.x + i * 256;
+            const int kk = f / (ROWS / 4), rq = (f % (ROWS / 4)) << 2;
+            off[i] = kk * ld + min(row0 + rq, rows - 4);
+        }
+    }
+    __device__ __forceinline__ void fetch_fast(const float *tile_base) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = gload4(tile_base + off[i]);
+    }
     __device__ __forceinline__ void fetch(const float *base, int ld, int row0, int k0, int rows, int K, bool vec_ok) {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
@@ -213,6 +245,7 @@ struct LoadRowContig {
 // factor).  Each thread expands 8 consecutive codes of one matrix row.
 template <int ROWS, int BITS, bool ALONG_K>
 struct LoadQuant {
+    static constexpr bool kRowMajor = ALONG_K;               // 8 consecutive k of one row: [row][k]; else [k][row]
     static constexpr int TOTAL = ROWS * BK / 8;              // 8-element groups in the tile
     static constexpr int GROUPS = (TOTAL + 255) / 256;       // per thread
     // `fetch` only issues the global loads (packed codes, the segment maximum, the exact diagonal
@@ -285,16 +318,10 @@ struct LoadQuant {
             locate(g, tr, tc);
             float v[8];
             expand(g, s_code, v);
-            constexpr int LD = ROWS + LDS_PAD;
-            if (ALONG_K) {
-                float *d = lds + tc * LD + tr;                // consecutive lanes: consecutive words
-#pragma unroll
-                for (int e = 0; e < 8; ++e) d[e * LD] = v[e];
-            } else {
-                float4 *d = reinterpret_cast<float4 *>(lds + tr * LD + tc);
-                d[0] = make_float4(v[0], v[1], v[2], v[3]);
-                d[1] = make_float4(v[4], v[5], v[6], v[7]);
-            }
+            constexpr int LD = ALONG_K ? LDK : ROWS + LDS_PAD;
+            float4 *d = reinterpret_cast<float4 *>(lds + tr * LD + tc);
+            d[0] = make_float4(v[0], v[1], v[2], v[3]);
+            d[1] = make_float4(v[4], v[5], v[6], v[7]);
         }
     }
 };
@@ -326,9 +353,21 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     }
     if (args.skip != nullptr && args.skip[b] != 0) return;
 
+    using LoaderA = typename std::conditional<KA == kDense, LoadKContig<BM>,
+        typename std::conditional<KA == kDenseT, LoadRowContig<BM>,
+            LoadQuant<BM, KA == kQuant4 ? 4 : 8, true>>::type>::type;
+    using LoaderB = typename std::conditional<KB == kDense, LoadRowContig<BN>,
+        typename std::conditional<KB == kDenseT, LoadKContig<BN>,
+            LoadQuant<BN, KB == kQuant4 ? 4 : 8, false>>::type>::type;
+    // An operand whose k is contiguous at the source sits in LDS as [row][k] (16-byte commits, one
+    // 16-byte fragment read per four MFMA steps); the others as [k][row] (16-byte commits, one word
+    // per step).  Which k a lane feeds into which step is free as long as both operands agree:
+    // step s of a tile takes k = 8 (s / 4) + 4 (lane / 32) + s % 4.
+    constexpr bool A_RM = LoaderA::kRowMajor, B_RM = LoaderB::kRowMajor;
     constexpr int LDA = BM + LDS_PAD, LDB = BN + LDS_PAD;
-    __shared__ __attribute__((aligned(16))) float s_a[2][BK * LDA];
-    __shared__ __attribute__((aligned(16))) float s_b[2][BK * LDB];
+    constexpr int SIZE_A = A_RM ? BM * LDK : BK * LDA, SIZE_B = B_RM ? BN * LDK : BK * LDB;
+    __shared__ __attribute__((aligned(16))) float s_a[2][SIZE_A];
+    __shared__ __attribute__((aligned(16))) float s_b[2][SIZE_B];
     __shared__ float s_code[256];
     constexpr bool kNeedCode = KA >= kQuant4 || KB >= kQuant4 || EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8;
     if (kNeedCode) {
@@ -346,18 +385,32 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     const bool a_vec = KA < kQuant4 && (args.lda & 3) == 0 && is_aligned16(A);
     const bool b_vec = KB < kQuant4 && (args.ldb & 3) == 0 && is_aligned16(B);
 
-    typename std::conditional<KA == kDense, LoadKContig<BM>,
-        typename std::conditional<KA == kDenseT, LoadRowContig<BM>,
-            LoadQuant<BM, KA == kQuant4 ? 4 : 8, true>>::type>::type la;
-    typename std::conditional<KB == kDense, LoadRowContig<BN>,
-        typename std::conditional<KB == kDenseT, LoadKContig<BN>,
-            LoadQuant<BN, KB == kQuant4 ? 4 : 8, false>>::type>::type lb;
+    LoaderA la;
+    LoaderB lb;
 
+    // whole k tiles, aligned rows, extents that keep a clamped 16-byte load inside the matrix and
+    // offsets inside 31 bits: the loads of the main loop then need no predicates at all
+    const bool whole_k = args.K % BK == 0;
+    bool a_fast = false, b_fast = false;
+    if constexpr (KA < kQuant4) {
+        a_fast = whole_k && a_vec && (KA == kDense || (args.M & 3) == 0) &&
+                 (long long)(KA == kDense ? args.M : args.K) * args.lda < 0x7fffffffLL;
+        if (a_fast) la.prepare(args.lda, m0, args.M);
+    }
+    if constexpr (KB < kQuant4) {
+        b_fast = whole_k && b_vec && (KB == kDenseT || (args.N & 3) == 0) &&
+                 (long long)(KB == kDenseT ? args.N : args.K) * args.ldb < 0x7fffffffLL;
+        if (b_fast) lb.prepare(args.ldb, n0, args.N);
+    }
     auto fetch = [&](int k0) {
-        if constexpr (KA < kQuant4) la.fetch(A, args.lda, m0, k0, args.M, args.K, a_vec);
-        else la.fetch(args.Aq, b, s_code, m0, k0);
-        if constexpr (KB < kQuant4) lb.fetch(B, args.ldb, n0, k0, args.N, args.K, b_vec);
-        else lb.fetch(args.Bq, b, s_code, n0, k0);
+        if constexpr (KA < kQuant4) {
+            if (a_fast) la.fetch_fast(A + (KA == kDense ? (long long)k0 : (long long)k0 * args.lda));
+            else la.fetch(A, args.lda, m0, k0, args.M, args.K, a_vec);
+        } else la.fetch(args.Aq, b, s_code, m0, k0);
+        if constexpr (KB < kQuant4) {
+            if (b_fast) lb.fetch_fast(B + (KB == kDenseT ? (long long)k0 : (long long)k0 * args.ldb));
+            else lb.fetch(B, args.ldb, n0, k0, args.N, args.K, b_vec);
+        } else lb.fetch(args.Bq, b, s_code, n0, k0);
     };
 
     f32x16 acc[MI][NI];
@@ -377,27 +430,48 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     lb.commit(s_b[0], s_code);
     if (n_tiles > 1) fetch(BK);
     __syncthreads();
-    const int frag_row = lane & 31, frag_k = lane >> 5;
+    const int frag_row = lane & 31, half = lane >> 5;
+    constexpr int STEPS = BK / 2;
     for (int t = 0; t < n_tiles; ++t) {
         const int cur = t & 1;
-        const float *pa = s_a[cur] + frag_k * LDA + wm + frag_row;
-        const float *pb = s_b[cur] + frag_k * LDB + wn + frag_row;
-        // fragments for step ks+1 are read from LDS before the MFMAs of step ks are issued
+        const float *pa = s_a[cur] + (A_RM ? (wm + frag_row) * LDK + 4 * half : 4 * half * LDA + wm + frag_row);
+        const float *pb = s_b[cur] + (B_RM ? (wn + frag_row) * LDK + 4 * half : 4 * half * LDB + wn + frag_row);
+        // fragments are read from LDS ahead of the MFMAs that use them: the next step's words for a
+        // [k][row] operand, the next group of four steps for a [row][k] operand
         float fa[2][MI], fb[2][NI];
+        qt_f32x4 qa[2][MI], qb[2][NI];
+        auto load_a = [&](int step) {
+            if constexpr (A_RM) {
+                if (step % 4 == 0)
 #pragma unroll
-        for (int i = 0; i < MI; ++i) fa[0][i] = pa[i * 32];
+                    for (int i = 0; i < MI; ++i)
+                        qa[(step / 4) & 1][i] = *reinterpret_cast<const qt_f32x4 *>(pa + i * 32 * LDK + 8 * (step / 4));
+            } else {
 #pragma unroll
-        for (int j = 0; j < NI; ++j) fb[0][j] = pb[j * 32];
-#pragma unroll
-        for (int ks = 0; ks < BK / 2; ++ks) {
-            const int now = ks & 1, nxt = now ^ 1;
-            if (ks + 1 < BK / 2) {
-#pragma unroll
-                for (int i = 0; i < MI; ++i) fa[nxt][i] = pa[i * 32 + 2 * (ks + 1) * LDA];
-#pragma unroll
-                for (int j = 0; j < NI; ++j) fb[nxt][j] = pb[j * 32 + 2 * (ks + 1) * LDB];
+                for (int i = 0; i < MI; ++i) fa[step & 1][i] = pa[i * 32 + (8 * (step / 4) + step % 4) * LDA];
             }
-            if (ks == BK / 4 && t + 1 < n_tiles) {
+        };
+        auto load_b = [&](int step) {
+            if constexpr (B_RM) {
+                if (step % 4 == 0)
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+                        qb[(step / 4) & 1][j] = *reinterpret_cast<const qt_f32x4 *>(pb + j * 32 * LDK + 8 * (step / 4));
+            } else {
+#pragma unroll
+                for (int j = 0; j < NI; ++j) fb[step & 1][j] = pb[j * 32 + (8 * (step / 4) + step % 4) * LDB];
+            }
+        };
+        load_a(0);
+        load_b(0);
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            // [row][k] operands fetch a whole group ahead (at the first step of the previous group)
+            if (A_RM && s % 4 == 0 && s + 4 < STEPS) load_a(s + 4);
+            if (B_RM && s % 4 == 0 && s + 4 < STEPS) load_b(s + 4);
+            if (!A_RM && s + 1 < STEPS) load_a(s + 1);
+            if (!B_RM && s + 1 < STEPS) load_b(s + 1);
+            if (s == STEPS / 2 && t + 1 < n_tiles) {
                 la.commit(s_a[cur ^ 1], s_code);
                 lb.commit(s_b[cur ^ 1], s_code);
                 if (t + 2 < n_tiles) fetch((t + 2) * BK);
@@ -405,8 +479,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
-                for (int j = 0; j < NI; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[now][i], fb[now][j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < NI; ++j) {
+                    const float av = A_RM ? qa[(s / 4) & 1][i][s % 4] : fa[s & 1][i];
+                    const float bv = B_RM ? qb[(s / 4) & 1][j][s % 4] : fb[s & 1][j];
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
+                }
         }
         __syncthreads();
     }
