@@ -249,47 +249,64 @@ struct LoadQuant {
     static constexpr int TOTAL = ROWS * BK / 8;              // 8-element groups in the tile
     static constexpr int GROUPS = (TOTAL + 255) / 256;       // per thread
     // `fetch` only issues the global loads (packed codes, the segment maximum, the exact diagonal
-    // entry if the group crosses the diagonal); the table lookups wait until `commit`, one tile
-    // later, when the loads have long landed.
+    // entry); the table lookups wait until `commit`, one tile later, when the loads have long
+    // landed.  The order is a multiple of 64, hence of the tile depth: no k bounds; groups beyond the
+    // matrix are clamped into it (their products are never stored).  Offsets are split into a fixed
+    // per-thread part (`prepare`) and a part that is uniform over the workgroup per tile.
     uint2 raw[GROUPS];
     float amax[GROUPS];
     float dval[GROUPS];
-    int dpos[GROUPS];                                        // element of the group on the diagonal, -1: none, -2: outside
+    int dpos[GROUPS];                                        // element of the group on the diagonal, if in 0..7
+    int code_off[GROUPS], amax_off[GROUPS], d0[GROUPS], drow[GROUPS];
+    const uint8_t *codes;
+    const float *absmax, *diag;
+    int order, per_row, shift;
     __device__ __forceinline__ bool active(int g) const { return (int)threadIdx.x + g * 256 < TOTAL; }
     __device__ __forceinline__ void locate(int g, int &mr, int &mc) const {
         const int f = threadIdx.x + g * 256;
         if (ALONG_K) { mr = f % ROWS; mc = (f / ROWS) << 3; }               // tile row = matrix row, 2 groups per row
         else { mr = f / (ROWS / 8); mc = (f % (ROWS / 8)) << 3; }           // tile k = matrix row
     }
-    __device__ __forceinline__ void fetch(const QuantRef &q, int b, const float *s_code, int row0, int k0) {
-        (void)s_code;
-        const uint8_t *codes = batch_ptr<uint8_t>(q.codes, b);
-        const float *absmax = batch_ptr<float>(q.absmax, b);
-        const float *diag = has_ptr(q.diag) ? batch_ptr<float>(q.diag, b) : nullptr;
+    __device__ __forceinline__ void prepare(const QuantRef &q, int b, int row0) {
+        codes = batch_ptr<uint8_t>(q.codes, b);
+        absmax = batch_ptr<float>(q.absmax, b);
+        diag = has_ptr(q.diag) ? batch_ptr<float>(q.diag, b) : nullptr;
+        order = q.order; shift = q.bs_shift; per_row = q.order >> q.bs_shift;
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            int tr, tc;
+            locate(g, tr, tc);
+            // matrix row / first column of the group at k0 = 0
+            const int mr = ALONG_K ? min(row0 + tr, order - 1) : tr;
+            const int mc = ALONG_K ? tc : min(row0 + tc, order - 8);
+            const int k = mr * order + mc;                   // below 2^31: checked on the host
+            code_off[g] = BITS == 4 ? k >> 1 : k;
+            amax_off[g] = mr * per_row + (mc >> shift);
+            d0[g] = mr - mc;
+            drow[g] = mr;
+            if (ALONG_K) dval[g] = diag != nullptr ? gload(diag + mr) : 0.0f;
+        }
+    }
+    __device__ __forceinline__ void fetch(int k0) {
+        // uniform parts of the addresses for this tile
+        const long long step = ALONG_K ? k0 : (long long)k0 * order;
+        const uint8_t *c = codes + (BITS == 4 ? step >> 1 : step);
+        const float *a = absmax + (ALONG_K ? k0 >> shift : k0 * per_row);
 #pragma unroll
         for (int g = 0; g < GROUPS; ++g) {
             if (!active(g)) continue;
-            int tr, tc;
-            locate(g, tr, tc);
-            const int mr = ALONG_K ? row0 + tr : k0 + tr;     // matrix row
-            const int mc = ALONG_K ? k0 + tc : row0 + tc;     // first matrix column of the group
-            dpos[g] = -2;
-            if (mr < q.order && mc < q.order) {               // order is a multiple of 64: whole group inside
-                const long long k = (long long)mr * q.order + mc;
-                amax[g] = gload(absmax + (k >> q.bs_shift));
-                if (BITS == 4) raw[g].x = gload_u32(codes + (k >> 1));
-                else raw[g] = gload_u32x2(codes + k);
-                dpos[g] = -1;
-                if (diag != nullptr && mr >= mc && mr < mc + 8) { dpos[g] = mr - mc; dval[g] = gload(diag + mr); }
+            amax[g] = gload(a + amax_off[g]);
+            if (BITS == 4) raw[g].x = gload_u32(c + code_off[g]);
+            else raw[g] = gload_u32x2(c + code_off[g]);
+            if (ALONG_K) {
+                dpos[g] = diag != nullptr ? d0[g] - k0 : -1;
+            } else {
+                dpos[g] = diag != nullptr ? d0[g] + k0 : -1;
+                if (diag != nullptr) dval[g] = gload(diag + min(drow[g] + k0, order - 1));
             }
         }
     }
     __device__ __forceinline__ void expand(int g, const float *s_code, float v[8]) const {
-        if (dpos[g] == -2) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = 0.0f;
-            return;
-        }
         uint32_t id[8];
         if (BITS == 4) {
             const uint32_t w = raw[g].x;
@@ -402,15 +419,17 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
                  (long long)(KB == kDenseT ? args.N : args.K) * args.ldb < 0x7fffffffLL;
         if (b_fast) lb.prepare(args.ldb, n0, args.N);
     }
+    if constexpr (KA >= kQuant4) la.prepare(args.Aq, b, m0);
+    if constexpr (KB >= kQuant4) lb.prepare(args.Bq, b, n0);
     auto fetch = [&](int k0) {
         if constexpr (KA < kQuant4) {
             if (a_fast) la.fetch_fast(A + (KA == kDense ? (long long)k0 : (long long)k0 * args.lda));
             else la.fetch(A, args.lda, m0, k0, args.M, args.K, a_vec);
-        } else la.fetch(args.Aq, b, s_code, m0, k0);
+        } else la.fetch(k0);
         if constexpr (KB < kQuant4) {
             if (b_fast) lb.fetch_fast(B + (KB == kDenseT ? (long long)k0 : (long long)k0 * args.ldb));
             else lb.fetch(B, args.ldb, n0, k0, args.N, args.K, b_vec);
-        } else lb.fetch(args.Bq, b, s_code, n0, k0);
+        } else lb.fetch(k0);
     };
 
     f32x16 acc[MI][NI];
@@ -593,6 +612,10 @@ bool valid_quant(const QuantRef &q, int bits, const char *what) {
     }
     if (!has_host_ptr(q.codes) || !has_host_ptr(q.absmax)) {
         set_error(kNullPointer, "gemm: %s: null codes/absmax pointer", what);
+        return false;
+    }
+    if ((long long)q.order * q.order > 0x7fffffffLL) {
+        set_error(kBadArgument, "gemm: %s: order * order must stay below 2^31 (order %d)", what, q.order);
         return false;
     }
     (void)bits;
