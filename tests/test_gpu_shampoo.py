@@ -71,8 +71,11 @@ def test_per_parameter_low_bit_path_follows_the_oracle(setup):
             assert rel(h.dequantize(), slot.get()) <= 2e-3
 
 
-def test_bank_equals_per_parameter_path(setup):
+@pytest.mark.parametrize("bits", [4, 8])
+def test_bank_equals_per_parameter_path(setup, code_maps, bits):
     S1, ShampooBank, grads, code = setup
+    code = code_maps[("linear-2", bits)]
+    KW = dict(globals()["KW"], prec_bits=bits)
     mats = [s for s in SHAPES if len([d for d in s if d != 1]) > 1]
     params = [torch.zeros(s, device="cuda") for s in mats]
     kw = {k: v for k, v in KW.items() if k in ("prec_maxorder", "prec_bits", "min_lowbit_size", "quan_blocksize")}
@@ -105,7 +108,7 @@ def test_bank_equals_per_parameter_path(setup):
             pre.compute_preconditioners([v.cuda() for v in v0_pre[pi]])
             want = pre.preconditioned_grad(gl[pi])
             assert outs[pi].shape == want.shape
-            assert rel(outs[pi], want) <= 1e-4
+            assert rel(outs[pi], want) <= (1e-4 if bits == 4 else 5e-4)      # more, smaller code flips on the finer grid
     for (pi, j, side, order, row) in table:
         h = pres[pi].statistics[2 * j + side]              # statistics: same kernels, bit-identical
         assert torch.equal(bank.stats[order].codes[row], h.var)
@@ -115,8 +118,8 @@ def test_bank_equals_per_parameter_path(setup):
         # for a stack of one and a stack of many, so agreement is to rounding, not to the bit
         h = pres[pi].preconditioners[2 * j + side]
         got, want = bank.precs[order].codes[row], h.var
-        differing = int(((got >> 4) != (want >> 4)).sum() + ((got & 15) != (want & 15)).sum())
-        assert differing <= 1e-3 * 2 * got.numel()
+        differing = int(((got >> 4) != (want >> 4)).sum() + ((got & 15) != (want & 15)).sum()) if bits == 4 else int((got != want).sum())
+        assert differing <= (1e-3 * 2 if bits == 4 else 2e-2) * got.numel()      # 8-bit steps are 16 times finer
         assert rel(bank.precs[order].absmax[row], h.absmax) <= 1e-5
         assert rel(bank.precs[order].diag[row], h.diag) <= 1e-5
     sd = bank.state_dict()
