@@ -164,6 +164,11 @@ typedef struct {
         int symmetric;          /* != 0: A B is known to be symmetric (M == N, dense operands): only the tiles
                                  * on and above the diagonal are multiplied out and every off-diagonal
                                  * tile is also stored mirrored; an addend is read at the mirrored place   */
+        float *workspace;       /* optional scratch (16-byte aligned) of workspace_floats floats: a plain-store
+                                 * product with few output tiles and a long k range is then cut along k into
+                                 * slices whose partial products land here and are summed in a fixed order    */
+        long long workspace_floats;
+        int split_k_;           /* ignored (set by the library)                                             */
     } args;
 } qtensor_gemm_desc;
 

@@ -62,6 +62,9 @@ struct GemmArgs {
     const float *code;            // code table for quantized operands / addend
     int symmetric;                // != 0: the product is symmetric (M == N); only tiles on or above the
                                   // diagonal are computed and every off-diagonal tile is also written mirrored
+    float *workspace;             // optional scratch for splitting k (plain-store products only)
+    long long workspace_floats;
+    int split_k;                  // set by the library: slices of the k range (1 = no split)
 };
 
 namespace {
@@ -354,6 +357,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     const uint32_t die = blockIdx.x % kDies, slot = blockIdx.x / kDies;
     const uint32_t per = total / kDies, extra = total % kDies;
     uint32_t id = die * per + min(die, extra) + slot;
+    const int slices = EPI == kStore ? args.split_k : 1;
+    const int slice = id % slices;
+    id /= slices;
     int tile_m, tile_n, b;
     if (args.symmetric) {                  // row-major walk over the tiles on and above the diagonal
         const uint32_t upper = (uint32_t)tiles_n * (tiles_n + 1) / 2;
@@ -443,11 +449,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     // Pipeline: tile t is multiplied out of one LDS buffer while tile t+1 (already in registers,
     // its loads were issued a whole tile earlier) is written to the other buffer half-way through
     // the MFMA stream and the loads of tile t+2 are issued right after.  One barrier per tile.
-    const int n_tiles = (args.K + BK - 1) / BK;
-    fetch(0);
+    // (with k split into slices -- the host makes them equal -- this workgroup owns one of them)
+    const int n_tiles = (args.K + BK - 1) / BK / slices;
+    const int k_begin = slice * n_tiles * BK;
+    fetch(k_begin);
     la.commit(s_a[0], s_code);
     lb.commit(s_b[0], s_code);
-    if (n_tiles > 1) fetch(BK);
+    if (n_tiles > 1) fetch(k_begin + BK);
     __syncthreads();
     const int frag_row = lane & 31, half = lane >> 5;
     constexpr int STEPS = BK / 2;
@@ -493,7 +501,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
             if (s == STEPS / 2 && t + 1 < n_tiles) {
                 la.commit(s_a[cur ^ 1], s_code);
                 lb.commit(s_b[cur ^ 1], s_code);
-                if (t + 2 < n_tiles) fetch((t + 2) * BK);
+                if (t + 2 < n_tiles) fetch(k_begin + (t + 2) * BK);
             }
 #pragma unroll
             for (int i = 0; i < MI; ++i)
@@ -509,6 +517,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
 
     // ---- epilogue: accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
     float *C = const_cast<float *>(batch_ptr<float>(args.C, b));
+    int ldc = args.ldc;
+    if (slices > 1) {                              // partial product of this slice: summed by reduce_slices_kernel
+        C = args.workspace + ((long long)b * slices + slice) * args.M * args.N;
+        ldc = args.N;
+    }
     float *T = EPI == kNewton ? const_cast<float *>(batch_ptr<float>(args.T, b)) : nullptr;
     const float *E = EPI == kAxpbyDense ? batch_ptr<float>(args.E, b) : nullptr;
     constexpr bool kQuantAddend = EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8;
@@ -519,7 +532,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     // an off-diagonal tile of a symmetric product also provides its mirror image; the addend is
     // read at the mirrored position, so an addend that is not exactly symmetric is honoured
     const bool mirror = args.symmetric != 0 && tile_n != tile_m;
-    const bool mirror_vec = (args.M & 3) == 0 && (args.ldc & 3) == 0 && is_aligned16(C) &&
+    const bool mirror_vec = (args.M & 3) == 0 && (ldc & 3) == 0 && is_aligned16(C) &&
                             (EPI != kNewton || ((args.ldt & 3) == 0 && is_aligned16(T))) &&
                             (EPI != kAxpbyDense || ((args.lde & 3) == 0 && is_aligned16(E)));
     float local_err = 0.0f;
@@ -548,7 +561,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
                         local_err = fmaxf(local_err, fabsf(y - eye));
                         gstore(T + (long long)row * args.ldt + col, (1.0f - args.newton_w) * eye + args.newton_w * y);
                     }
-                    gstore(C + (long long)row * args.ldc + col, y);
+                    gstore(C + (long long)row * ldc + col, y);
                 }
                 if (!mirror || col >= args.N || row4 >= args.M) continue;
                 // mirrored: elements (col, row4 .. row4+3), never on the diagonal
@@ -570,7 +583,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
                     else if (kQuantAddend) y[q] = __builtin_fmaf(args.alpha, a, args.beta * e[q]);
                     else y[q] = a;
                 }
-                float *cm = C + (long long)col * args.ldc + row4;
+                float *cm = C + (long long)col * ldc + row4;
                 if (whole) gstore4(cm, y);
                 else
 #pragma unroll
@@ -594,13 +607,47 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
 }
 
 
+// out[b][m][n] = sum over slices of workspace[b][slice][m][n], slices added in order
+__global__ __launch_bounds__(256) void reduce_slices_kernel(const float *workspace, int slices, BatchPtr C, int ldc, int M, int N) {
+    const int b = blockIdx.y;
+    const long long plane = (long long)M * N;
+    const float *w = workspace + (long long)b * slices * plane;
+    float *out = const_cast<float *>(batch_ptr<float>(C, b));
+    const bool vec = (N & 3) == 0 && (ldc & 3) == 0 && is_aligned16(out) && is_aligned16(w);
+    if (vec) {
+        const long long quads = plane >> 2;
+        for (long long q = blockIdx.x * 256ll + threadIdx.x; q < quads; q += (long long)gridDim.x * 256) {
+            const long long e = q << 2;
+            float4 sum = gload4(w + e);
+            for (int s = 1; s < slices; ++s) {
+                const float4 x = gload4(w + s * plane + e);
+                sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+            }
+            const int m = (int)(e / N), n = (int)(e % N);
+            float *o = out + (long long)m * ldc + n;
+            gstore(o, sum.x); gstore(o + 1, sum.y); gstore(o + 2, sum.z); gstore(o + 3, sum.w);
+        }
+    } else {
+        for (long long e = blockIdx.x * 256ll + threadIdx.x; e < plane; e += (long long)gridDim.x * 256) {
+            float sum = gload(w + e);
+            for (int s = 1; s < slices; ++s) sum += gload(w + s * plane + e);
+            gstore(out + (e / N) * ldc + e % N, sum);
+        }
+    }
+}
+
 template <int BM, int BN, int KA, int KB, int EPI>
 void launch_gemm(const GemmArgs &a, int batch, hipStream_t stream) {
     const long long tn = (a.N + BN - 1) / BN, tm = (a.M + BM - 1) / BM;
     if (a.symmetric && BM != BN) { set_error(kBadArgument, "gemm: symmetric products need square tiles"); return; }
-    const long long blocks = (a.symmetric ? tn * (tn + 1) / 2 : tn * tm) * batch;
+    const long long blocks = (a.symmetric ? tn * (tn + 1) / 2 : tn * tm) * batch * (EPI == kStore ? a.split_k : 1);
     if (blocks > 0x7fffffffLL) { set_error(kBadArgument, "gemm: too many tiles (%lld)", blocks); return; }
     hipLaunchKernelGGL((gemm_kernel<BM, BN, KA, KB, EPI>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    if (EPI == kStore && a.split_k > 1) {
+        const long long quads = ((long long)a.M * a.N + 1023) / 1024;
+        const unsigned grid = (unsigned)(quads < 4096 ? quads : 4096);
+        hipLaunchKernelGGL(reduce_slices_kernel, dim3(grid, batch), dim3(256), 0, stream, a.workspace, a.split_k, a.C, a.ldc, a.M, a.N);
+    }
 }
 
 bool valid_quant(const QuantRef &q, int bits, const char *what) {
@@ -702,6 +749,30 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
         }
     }
     if (a.symmetric && shapes[pick].bm != shapes[pick].bn) pick = 0;
+    // Few tiles and a long k range: cut k into equal slices (whole k tiles each) that write partial products
+    // to the caller's workspace and are summed in order afterwards.  Same cost model, with a fixed cost per
+    // workgroup (prologue, epilogue, the extra pass over the output) worth about 64 k steps.
+    a.split_k = 1;
+    if (ep == kStore && !a.symmetric && a.workspace != nullptr && d->K % 16 == 0 && is_aligned(a.workspace, 16)) {
+        const Shape &sh = shapes[pick];
+        const double units = compute_units();
+        const long long tm = (d->M + sh.bm - 1) / sh.bm, tn = (d->N + sh.bn - 1) / sh.bn;
+        const double tiles = (double)tm * tn * d->batch;
+        const int k_tiles = d->K / 16;
+        const double fixed = 64.0;
+        const double whole = ceil(tiles / units) * (d->K + fixed);
+        double best = whole;
+        int best_split = 1;
+        static const char *forced_split = getenv("QT_GEMM_SPLIT");
+        for (int sp = 2; sp <= 8; ++sp) {
+            if (k_tiles % sp != 0 || k_tiles / sp < 8) continue;
+            if ((long long)sp * d->batch * d->M * d->N > a.workspace_floats) continue;
+            const double cost = ceil(tiles * sp / units) * ((double)d->K / sp + fixed);
+            if (forced_split != nullptr) { if (sp == atoi(forced_split)) best_split = sp; }
+            else if (cost < best) { best = cost; best_split = sp; }
+        }
+        if (forced_split != nullptr || best < 0.95 * whole) a.split_k = best_split;
+    }
     const int combo = ka * 100 + kb * 10 + ep;
 #define QT_GEMM_CASE(KA, KB, EP)                                                                             \
     case (KA) * 100 + (KB) * 10 + (EP):                                                                      \

@@ -88,6 +88,9 @@ def ComputePower(mat_g, p, iter_count=10, error_tolerance=1e-6, ridge_epsilon=1e
     return root
 
 
+_LAST_ROUNDS = {}                                  # order -> int32 [B], for diagnostics
+
+
 @torch.no_grad()
 def PowerIterBatched(mats, error_tolerance=1e-6, num_iters=10, v0=None):
     """PowerIter for a stack [B, n, n]; every matrix follows its own stopping rule (entries that
@@ -177,5 +180,6 @@ def ComputePowerBatched(mats, p=4, iter_count=10, error_tolerance=1e-6, ridge_ep
         err = torch.where(accept, new_err, err)
         rounds = rounds + accept.to(torch.int32)
         done = done | ~accept | (err <= error_tolerance) | (rounds >= iter_count)
+    _LAST_ROUNDS[n] = rounds                       # accepted rounds per matrix of the last stack of this order
     res = torch.where(side.view(B, 1, 1), R[1], R[0])
     return res if out is None else out.copy_(res)

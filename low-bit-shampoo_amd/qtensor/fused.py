@@ -37,7 +37,8 @@ class GemmArgs(ct.Structure):
                 ("Eq", QuantRef),
                 ("T", BatchPtr), ("ldt", ct.c_int),
                 ("newton_w", ct.c_float),
-                ("err", ct.c_void_p), ("skip", ct.c_void_p), ("code", ct.c_void_p), ("symmetric", ct.c_int)]
+                ("err", ct.c_void_p), ("skip", ct.c_void_p), ("code", ct.c_void_p), ("symmetric", ct.c_int),
+                ("workspace", ct.c_void_p), ("workspace_floats", ct.c_longlong), ("split_k_", ct.c_int)]
 
 
 class GemmDesc(ct.Structure):
@@ -113,6 +114,17 @@ def _dense(t):
     if t.dim() != 3 or t.stride(2) != 1:
         raise ValueError("expected [rows, cols] or [batch, rows, cols] with a contiguous last dimension")
     return BatchPtr(t.data_ptr(), None, t.stride(0)), t.stride(1), t.shape[0], t.shape[1], t.shape[2]
+
+
+_WORKSPACE = {}                 # (device index, stream) -> fp32 scratch for products that are split along k
+_WORKSPACE_FLOATS = 1 << 24     # 64 MiB
+
+
+def _workspace(device: torch.device) -> Tensor:
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    if key not in _WORKSPACE:
+        _WORKSPACE[key] = torch.empty(_WORKSPACE_FLOATS, dtype=torch.float32, device=device)
+    return _WORKSPACE[key]
 
 
 def _launch(desc: GemmDesc, device: torch.device) -> None:
@@ -206,6 +218,10 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
         if m != n or isinstance(A, Quantized) or isinstance(B, Quantized):
             raise ValueError("symmetric products are square with dense operands")
         a.symmetric = 1
+    if d.epilogue == EPI_STORE and not symmetric and k >= 256 and batch * m * n <= _WORKSPACE_FLOATS // 2:
+        # few output tiles, long k: the library may cut k into slices (one scratch area per stream)
+        scratch = _workspace(dev)
+        a.workspace, a.workspace_floats = scratch.data_ptr(), scratch.numel()
     _launch(d, dev)
     return out
 

@@ -238,3 +238,24 @@ def test_stack_quantize_dequantize_equal_per_matrix_calls(mods, code_maps, bits,
                 assert np.array_equal(back[b].cpu().numpy(), want)
                 want16 = Q.dequantize_c(o[0], code, n, o[1], bs, bits, diag=o[2] if diag else None, to_bf16=True)
                 assert np.array_equal(back16[b].float().cpu().numpy(), want16)
+
+
+@pytest.mark.parametrize("m,n,k,batch", [(768, 3072, 3072, 1), (256, 256, 2048, 2), (100, 260, 1024, 1)])
+def test_products_split_along_k_equal_the_unsplit_ones_to_rounding(mods, m, n, k, batch, monkeypatch):
+    """Few output tiles and a long k range: the library cuts k into slices whose partial products go through
+    a scratch area and are summed in a fixed order (deterministic: two runs agree bit for bit)."""
+    _, X = mods
+    g = torch.Generator().manual_seed(k + m)
+    A = torch.randn(batch, m, k, generator=g)
+    B = torch.randn(batch, k, n, generator=g)
+    want = A.double() @ B.double()
+    Ad, Bd = A.cuda(), B.cuda()
+    first = X.gemm(Ad, Bd)
+    assert rel_err(first, want) <= TOL
+    assert torch.equal(first, X.gemm(Ad, Bd))
+    monkeypatch.setattr(X, "_WORKSPACE_FLOATS", 0)                 # no scratch: no split
+    assert rel_err(X.gemm(Ad, Bd), want) <= TOL
+    out = torch.full((batch, m, n + 3), 7.0, device="cuda")          # a strided destination keeps its padding
+    monkeypatch.setattr(X, "_WORKSPACE_FLOATS", 1 << 24)
+    X.gemm(Ad, Bd, out=out[:, :, :n])
+    assert rel_err(out[:, :, :n], want) <= TOL and bool((out[:, :, n:] == 7.0).all())
