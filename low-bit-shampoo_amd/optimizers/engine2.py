@@ -34,6 +34,7 @@ class ShampooBank2(ShampooBank):
     def __init__(self, params, name2qmap, code, *, rect_t1=1, rect_t2=4, inv_root_mode=0, **kwargs):
         self.rect_t1, self.rect_t2, self.inv_root_mode = rect_t1, rect_t2, inv_root_mode
         self.qr_fallbacks = 0                     # matrices that went through torch.linalg.qr so far
+        self.qr_rounds = 0                        # Cholesky QR rounds so far, summed over the stacks
         super().__init__(params, name2qmap, code, **kwargs)
 
     def _init_statistics(self):
@@ -107,7 +108,6 @@ class ShampooBank2(ShampooBank):
         def advance(order):
             return lambda: None if solver[order].finished else solver[order].advance()
 
-        self.qr_rounds = getattr(self, "qr_rounds", 0)
 
         def iterate(order):
             def run():

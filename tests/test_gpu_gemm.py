@@ -259,3 +259,33 @@ def test_products_split_along_k_equal_the_unsplit_ones_to_rounding(mods, m, n, k
     monkeypatch.setattr(X, "_WORKSPACE_FLOATS", 1 << 24)
     X.gemm(Ad, Bd, out=out[:, :, :n])
     assert rel_err(out[:, :, :n], want) <= TOL and bool((out[:, :, n:] == 7.0).all())
+
+
+def test_random_shapes_strides_and_alignments_all_dense_layouts(mods):
+    """Seeded sweep over odd extents, padded leading dimensions and base addresses that are not 16-byte
+    aligned: exercises the predicate-free tile loads, the guarded ones and the switch between them."""
+    _, X = mods
+    g = torch.Generator().manual_seed(1234)
+    pick = lambda choices: choices[int(torch.randint(len(choices), (1,), generator=g))]      # noqa: E731
+    for case in range(60):
+        m, n = pick([1, 4, 31, 64, 100, 128, 130, 257]), pick([1, 4, 33, 64, 96, 128, 200, 260])
+        k = pick([1, 15, 16, 17, 32, 48, 100, 256, 272])
+        batch, ta, tb = pick([1, 1, 2, 3]), pick([False, True]), pick([False, True])
+        pad_a, pad_b, shift_a, shift_b = pick([0, 0, 4, 3]), pick([0, 0, 4, 1]), pick([0, 0, 1]), pick([0, 0, 2])
+
+        def operand(rows, cols, pad, shift):
+            flat = torch.randn(batch * rows * (cols + pad) + shift, generator=g).cuda()
+            return flat[shift:].view(batch, rows, cols + pad)[:, :, :cols]
+
+        A = operand(k, m, pad_a, shift_a) if ta else operand(m, k, pad_a, shift_a)
+        B = operand(n, k, pad_b, shift_b) if tb else operand(k, n, pad_b, shift_b)
+        Ad = A.double().cpu().transpose(1, 2) if ta else A.double().cpu()
+        Bd = B.double().cpu().transpose(1, 2) if tb else B.double().cpu()
+        want = Ad @ Bd
+        if ta and tb:                                  # A^T B^T is not on the path and not built
+            with pytest.raises(RuntimeError):
+                X.gemm(A, B, trans_a=ta, trans_b=tb)
+            continue
+        got = X.gemm(A, B, trans_a=ta, trans_b=tb)
+        assert got.shape == (batch, m, n)
+        assert rel_err(got, want) <= TOL, (case, m, n, k, batch, ta, tb, pad_a, pad_b, shift_a, shift_b)
