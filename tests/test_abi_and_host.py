@@ -3,6 +3,7 @@ mirror of qtensor behaves like the reference's interface where no GPU is involve
 import ctypes as ct
 import re
 import subprocess
+import sys
 from pathlib import Path
 
 import numpy as np
@@ -152,3 +153,13 @@ def test_svdfast_dense_path_matches_reference_vectors(golden):
     assert float(s.Svalue.min()) >= float(lam[0]) - 1e-5 and float(s.max_eigenvalue) <= float(lam[-1]) + 1e-5
     assert float(s.Svalue.max()) <= float(s.max_eigenvalue) and s.Svalue.numel() == n // 2
     assert torch.allclose(s.var @ s.var.T, torch.eye(n), atol=1e-5)
+
+
+def test_bench_refuses_more_than_one_gpu_and_names_its_sections():
+    """bench.py measures one GPU: --gpus N with N > 1 exits with a message (no GPU is touched for that)."""
+    bench = ROOT / "bench.py"
+    run = subprocess.run([sys.executable, str(bench), "--gpus", "2"], capture_output=True, text=True)
+    assert run.returncode != 0 and "one GPU" in (run.stderr + run.stdout)
+    helptext = subprocess.run([sys.executable, str(bench), "--help"], capture_output=True, text=True, check=True).stdout
+    for flag in ("--gpus", "--steps", "--warmup", "--section", "--no-cpu-baseline"):
+        assert flag in helptext
