@@ -99,8 +99,14 @@ def fused_step(opt, group, update, group_index=0):
     entry['step'] += 1
     step, bank, banked = entry['step'], entry['bank'], entry['banked']
     for p in params:
-        opt.state[p]['step'] = step
+        state = opt.state[p]
+        state['step'] = step
+        if id(p) not in entry['ids'] and 'preconditioner' not in state:      # first gradient after the bank was built
+            state['preconditioner'] = opt._make_preconditioner(p, group)
     grads = {id(p): p.grad.contiguous() for p in params}
+    if any(id(p) not in grads for p in banked):
+        raise RuntimeError("fused=True batches the parameters that had a gradient at the first step; "
+                           "every one of them needs a gradient at every later step")
     directions, grafted = {}, set()
     if bank is not None:
         bgrads = [grads[id(p)] for p in banked]
