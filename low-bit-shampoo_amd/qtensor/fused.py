@@ -372,6 +372,10 @@ class CholeskyQR:
         self.finished = False
         self.rounds = 0                               # factorisation rounds enqueued so far
         self.gram = self.flags = self.near = None
+        # per working-set entry: a factorisation WITH the shift hit a non-positive pivot (hopeless: the
+        # library takes over) / one WITHOUT it did (the entry keeps its Q and gets the shift from now on)
+        self.fatal = torch.zeros(B, dtype=torch.bool, device=Y.device)
+        self.needs_shift = torch.zeros(B, dtype=torch.bool, device=Y.device)
 
     def _keep(self, keep):
         """Shrink the working set to the entries of the host mask `keep`."""
@@ -379,16 +383,16 @@ class CholeskyQR:
             return
         index = torch.nonzero(keep).flatten().to(self.Q.device)
         self.Q, self.ids = self.Q[index], self.ids[index]
+        self.fatal, self.needs_shift = self.fatal[index], self.needs_shift[index]
         if self.gram is not None:
             self.gram = self.gram[index]
 
     def check(self):
-        k = self.Q.shape[0]
         self.gram = gemm(self.Q, self.Q, trans_a=True, symmetric=True)
         self.gram.diagonal(dim1=1, dim2=2).sub_(1.0)
         done = self.gram.abs().amax(dim=(1, 2)) < self.tolerance                # False for NaN as well
         near = torch.linalg.matrix_norm(self.gram) < 0.5
-        self.flags = torch.stack([done, near, self.info[:k] != 0])
+        self.flags = torch.stack([done, near, self.fatal])
 
     def poll(self):
         done, near, failed = self.flags.cpu()                                   # the host synchronisation
@@ -409,12 +413,20 @@ class CholeskyQR:
     def advance(self):
         k = self.Q.shape[0]
         near = self.near.to(self.Q.device)
-        self.gram.diagonal(dim1=1, dim2=2).add_(1.0 + self.shift * (~near).to(self.gram.dtype).unsqueeze(1))
-        self.info[:k].zero_()
-        cholesky_upper(self.gram, self.U[:k], self.inv[:k], self.info[:k])
+        # The first round is tried without the shift: for condition numbers up to about 1e3 that saves a
+        # round, and a matrix for which it fails (non-positive pivot) simply keeps its Q and joins the
+        # shifted rounds.
+        shifted = ~near & (self.needs_shift if self.rounds == 0 else torch.ones_like(near))
+        self.gram.diagonal(dim1=1, dim2=2).add_(1.0 + self.shift * shifted.to(self.gram.dtype).unsqueeze(1))
+        info = self.info[:k]
+        info.zero_()
+        cholesky_upper(self.gram, self.U[:k], self.inv[:k], info)
         out = torch.empty_like(self.Q)
         solve_upper_right(self.Q, self.U[:k], self.inv[:k], self.panel[:k], out)
-        self.Q, self.gram = out, None
+        bad = info != 0
+        self.fatal = self.fatal | (bad & (shifted | near))
+        self.needs_shift = self.needs_shift | bad
+        self.Q, self.gram = torch.where(bad.view(k, 1, 1), self.Q, out), None
         self.rounds_left -= 1
         self.rounds += 1
         if bool(self.near.any()):
