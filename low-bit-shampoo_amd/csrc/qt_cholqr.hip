@@ -48,14 +48,11 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
     for (int k = 0; k < NB; ++k) {
         float d = lane_value(row[k], k);
         if (!(d > 0.0f)) { ok = false; d = 1.0f; }
-        const float scale = 1.0f / sqrtf(d);
-        const float lik = row[k] * scale;        // L[lane][k] (lanes above k: unused values)
+        // a[i][j] -= a[i][k] a[k][j] / d: one multiply per lane, then a broadcast and a multiply-add per column
+        const float t = row[k] / d;
 #pragma unroll
-        for (int j = k + 1; j < NB; ++j) {
-            const float ljk = lane_value(row[j], k) * scale;     // L[j][k] from row k
-            row[j] -= lik * ljk;
-        }
-        row[k] = lik;
+        for (int j = k + 1; j < NB; ++j) row[j] -= t * lane_value(row[j], k);
+        row[k] = row[k] / sqrtf(d);              // L[lane][k] (lanes above k: unused values)
     }
     // column `lane` of L^-1 by forward substitution; L[i][k] sits in lane i
     float x[NB];
