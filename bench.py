@@ -157,6 +157,7 @@ def fused_gemm_gpu(torch, code):
 
     def inverse_root_like(order):
         q, _ = torch.linalg.qr(torch.randn(order, order, device="cuda", generator=g))
+        torch.cuda.synchronize()
         lam = torch.exp(torch.rand(order, device="cuda", generator=g) * (-6.0 * 2.302585093))   # log-uniform in [1e-6, 1]
         return ((q * lam.pow(-0.25)) @ q.T).contiguous()
 

@@ -84,15 +84,15 @@ def test_cholesky_qr_gives_the_householder_factor_up_to_signs(mods):
             R = Q.transpose(1, 2) @ Y                                  # upper triangular, positive diagonal
             assert float(torch.tril(R, -1).abs().max() / R.abs().max()) < 1e-4
             assert bool((torch.diagonal(R, dim1=1, dim2=2) > 0).all())
-            Qh, Rh = torch.linalg.qr(Y.double())
+            Qh, Rh = torch.linalg.qr(Y.double().cpu())                 # the reference factor on the host
             Qh = Qh * torch.sign(torch.diagonal(Rh, dim1=1, dim2=2)).unsqueeze(1)
             # columns belonging to tiny pivots are determined to (rounding / pivot) only
-            assert float(((Q.double() - Qh).abs() * torch.diagonal(Rh, dim1=1, dim2=2).abs().unsqueeze(1)).max()
+            assert float(((Q.double().cpu() - Qh).abs() * torch.diagonal(Rh, dim1=1, dim2=2).abs().unsqueeze(1)).max()
                          / Rh.abs().max()) < 1e-5
     # an order that is not a multiple of 64 is padded with an identity block
     Y = torch.randn(3, 100, 100, generator=g).cuda()
     Q, redone = E2.cholesky_qr(Y)
-    Qh, Rh = torch.linalg.qr(Y.double())
+    Qh, Rh = torch.linalg.qr(Y.double().cpu())
     Qh = Qh * torch.sign(torch.diagonal(Rh, dim1=1, dim2=2)).unsqueeze(1)
     assert redone == 0 and Q.shape == (3, 100, 100) and rel(Q, Qh) <= 1e-4
     # a matrix with a zero column cannot be factorised this way: it is sent to the library routine
@@ -105,7 +105,12 @@ def test_cholesky_qr_gives_the_householder_factor_up_to_signs(mods):
 def run_both(S2, E2, code_maps, mode, same_qr, monkeypatch, steps=3):
     import qtensor.utils as U
     if not same_qr:                      # the per-parameter path with the vendor's Householder QR, as in the reference
-        monkeypatch.setattr(U, "_orthonormal_basis", lambda Y: torch.linalg.qr(Y)[0])
+        def householder(Y):              # (fenced: this build's batched linalg calls are not reliably stream-ordered)
+            torch.cuda.synchronize()
+            Q = torch.linalg.qr(Y)[0]
+            torch.cuda.synchronize()
+            return Q
+        monkeypatch.setattr(U, "_orthonormal_basis", householder)
     g = torch.Generator().manual_seed(21)
     grads = [[0.02 * torch.randn(s, generator=g).cuda() for s in SHAPES] for _ in range(steps)]
     qmap = {"linear-2": torch.from_numpy(code_maps[("linear-2", 4)])}
