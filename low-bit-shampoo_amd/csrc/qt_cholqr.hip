@@ -4,8 +4,8 @@
 // (torch.linalg.qr at qtensor/utils.py:157 of the reference).
 //
 // Both are blocked with 64-wide panels.  The only arithmetic done outside the matrix-core GEMM
-// (qtensor_hip_gemm) is the 64 x 64 diagonal block: one wave per matrix factors it in LDS and also
-// inverts the factor, so that every panel solve becomes a product with that small inverse.
+// (qtensor_hip_gemm) is the 64 x 64 diagonal block: one wave per matrix factors it in registers and
+// also inverts the factor, so that every panel solve becomes a product with that small inverse.
 //   factor:  for each block row j:  U_jj = chol(G_jj);  U_j,> = U_jj^-T G_j,>;  G_>,> -= U_j,>^T U_j,>
 //   solve :  for each block col j:  X_j = (Q_j - X_<j U_<j,j) U_jj^-1
 // All launches go to the caller's stream; nothing is allocated or synchronised here.
@@ -24,10 +24,13 @@ constexpr int NB = 64;
 // Reads the upper triangle of G only.  A non-positive (or NaN) pivot sets info[b] = 1 and is
 // replaced by 1; the factor of that matrix is then meaningless.
 //
-// Lane i keeps row i of the (full, symmetric) trailing matrix in registers.  Because the matrix
-// stays symmetric, column k of step k is row k, i.e. the registers of lane k: they are broadcast
-// with v_readlane, so the whole factorisation and the inversion of the factor run without LDS
-// traffic or barriers (LDS only stages the block on the way in).
+// Lane i keeps row i of the (full, symmetric) trailing matrix in registers.  Step k scales column k
+// (one value per lane) into column k of L = U^T, parks it in LDS, and every lane reads it back as
+// 16-byte broadcasts: the same 64 values update the trailing matrix (a[i][j] -= L[i][k] L[j][k]) and
+// carry the forward substitution for column `lane` of L^-1 (s[j] -= L[j][k] x[k]), so the inverse
+// costs no second pass.  1 / sqrt(pivot) comes from v_rsq_f32 plus one Newton step.
+constexpr int LDC = NB + 4;                      // LDS row stride: rows stay 16-byte aligned
+
 __device__ __forceinline__ float lane_value(float x, int lane) {
     return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(x), lane));
 }
@@ -35,41 +38,53 @@ __device__ __forceinline__ float lane_value(float x, int lane) {
 __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long long g_stride, int ldg, float *u,
                                                         long long u_stride, int ldu, float *inv, long long inv_stride,
                                                         int *info) {
-    __shared__ float stage[NB][NB + 1];
+    __shared__ __attribute__((aligned(16))) float cols[NB][LDC];
     const int b = blockIdx.x, lane = threadIdx.x;
     const float *G = gram + (long long)b * g_stride;
-    for (int r = 0; r < NB; ++r) stage[r][lane] = G[(long long)r * ldg + lane];
+    for (int r = 0; r < NB; ++r) cols[r][lane] = G[(long long)r * ldg + lane];
     __syncthreads();
-    float row[NB];                               // row `lane` of the symmetric matrix; ends as row `lane` of L = U^T
+    float row[NB];                               // row `lane` of the symmetric matrix; ends as row `lane` of L
+    float s[NB];                                 // right-hand side e_lane of the substitution; ends as column `lane` of L^-1
 #pragma unroll
-    for (int j = 0; j < NB; ++j) row[j] = j >= lane ? stage[lane][j] : stage[j][lane];
+    for (int j = 0; j < NB; ++j) {
+        row[j] = j >= lane ? cols[lane][j] : cols[j][lane];
+        s[j] = j == lane ? 1.0f : 0.0f;
+    }
+    __syncthreads();
     bool ok = true;
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
         float d = lane_value(row[k], k);
         if (!(d > 0.0f)) { ok = false; d = 1.0f; }
-        // a[i][j] -= a[i][k] a[k][j] / d: one multiply per lane, then a broadcast and a multiply-add per column
-        const float t = row[k] / d;
+        float r = __builtin_amdgcn_rsqf(d);
+        r = r * __builtin_fmaf(-0.5f * d * r, r, 1.5f);
+        const float l = row[k] * r;              // L[lane][k] (lanes above k: unused values)
+        row[k] = l;
+        s[k] *= r;                               // x[k] = s[k] / L[k][k]
+        if (k + 1 < NB) {
+            cols[k][lane] = l;
+            __syncthreads();
+            const float xk = s[k];
 #pragma unroll
-        for (int j = k + 1; j < NB; ++j) row[j] -= t * lane_value(row[j], k);
-        row[k] = row[k] / sqrtf(d);              // L[lane][k] (lanes above k: unused values)
-    }
-    // column `lane` of L^-1 by forward substitution; L[i][k] sits in lane i
-    float x[NB];
+            for (int j = (k + 1) & ~3; j < NB; j += 4) {
+                const float4 c = *reinterpret_cast<const float4 *>(&cols[k][j]);
+                const float v[4] = {c.x, c.y, c.z, c.w};
 #pragma unroll
-    for (int i = 0; i < NB; ++i) {
-        float s = i == lane ? 1.0f : 0.0f;
-#pragma unroll
-        for (int k = 0; k < i; ++k) s -= lane_value(row[k], i) * x[k];
-        x[i] = i >= lane ? s / lane_value(row[i], i) : 0.0f;
+                for (int e = 0; e < 4; ++e)
+                    if (j + e > k) {
+                        row[j + e] = __builtin_fmaf(-l, v[e], row[j + e]);
+                        s[j + e] = __builtin_fmaf(-v[e], xk, s[j + e]);
+                    }
+            }
+        }
     }
     float *U = u + (long long)b * u_stride;
     float *I = inv + (long long)b * inv_stride + lane * NB;
 #pragma unroll
     for (int r = 0; r < NB; ++r) U[(long long)r * ldu + lane] = r <= lane ? row[r] : 0.0f;        // U[r][lane] = L[lane][r]
 #pragma unroll
-    for (int c = 0; c < NB; c += 4)              // U^-1[lane][c] = L^-1[c][lane] = x[c] of this lane
-        *reinterpret_cast<float4 *>(I + c) = make_float4(x[c], x[c + 1], x[c + 2], x[c + 3]);
+    for (int c = 0; c < NB; c += 4)              // U^-1[lane][c] = L^-1[c][lane] = s[c] of this lane (zero for c < lane)
+        *reinterpret_cast<float4 *>(I + c) = make_float4(s[c], s[c + 1], s[c + 2], s[c + 3]);
     if (!ok && lane == 0) info[b] = 1;
 }
 
