@@ -98,6 +98,12 @@ void qtensor_hip_quantize_batched(const void *A, int a_is_bf16, const float *cod
 void qtensor_hip_dequantize_batched(const unsigned char *q, const float *code, int bits, int order, int batch,
                                     const float *absmax, const float *diag, void *out, int out_is_bf16, int blocksize,
                                     qtensor_stream_t stream);
+/* Plain (no diagonal) quantizer applied to the transpose of every matrix of an fp32 stack, without
+ * writing the transpose out: entry b equals cquantize_blockwise_*bit_fp32 of A[b]^T.  Replaces
+ * `V.T.contiguous()` followed by the quantizer at qtensor/utils.py:169-170 of the reference.
+ * Needs blocksize in {64, 128, 256} dividing order, order a multiple of 64, 16-byte aligned A. */
+void qtensor_hip_quantize_transposed_batched(const float *A, const float *code, int bits, int order, int batch,
+                                             float *absmax, unsigned char *out, int blocksize, qtensor_stream_t stream);
 
 /* ---- self check and calibration (no counterpart in the reference) ------------------------
  * The flat-path quantizer replaces IEEE division by the segment maximum a with r = rcp(a) refined

@@ -293,6 +293,78 @@ __global__ __launch_bounds__(kThreads) void encode_kernel(
     }
 }
 
+// ---- transposed source -----------------------------------------------------------------
+// Quantizes the transpose of every matrix of a stack without writing the transpose out (the
+// reference transposes first: V.T.contiguous() at qtensor/utils.py:169, then the plain quantizer).
+// A workgroup takes BS input rows x 64 input columns, turns the tile around in LDS (row stride
+// BS + 1: the scalar writes and reads below hit distinct banks for BS = 64), and every group of
+// BS/4 lanes encodes one segment of an output row with the arithmetic of the flat path.
+template <int BITS, int BS>
+__global__ __launch_bounds__(kThreads) void quantize_transposed_kernel(
+    const float *__restrict__ A, const float *__restrict__ code, uint32_t order, uint32_t n_tiles, uint32_t tiles_r, uint32_t tiles_c,
+    float *__restrict__ absmax, uint8_t *__restrict__ out) {
+    constexpr int NCODE = 1 << BITS;
+    constexpr int LD = BS + 1;
+    constexpr int G = BS / 4;                    // lanes per segment
+    constexpr int SEGS = 64 / G;                 // segments a wave encodes at a time
+    static_assert(BS == 64 || BS == 128 || BS == 256, "segment of 64, 128 or 256 elements");
+    __shared__ CodeTables<NCODE> tab;
+    __shared__ float tile[64 * LD];
+    build_code_tables<NCODE>(code, tab, nullptr);
+    const bool fast_ok = (tab.flags & kFlagLut) != 0, ascending = (tab.flags & kFlagAscending) != 0;
+    const uint32_t t = threadIdx.x, lane = t & 63u, w = t >> 6;
+    const uint32_t per_matrix = tiles_r * tiles_c;
+    for (uint32_t id = blockIdx.x; id < n_tiles; id += gridDim.x) {
+        const uint32_t b = id / per_matrix, rem = id - b * per_matrix;
+        const uint32_t rb = rem / tiles_c, cb = rem - rb * tiles_c;
+        const float *src = A + ((size_t)b * order + (size_t)rb * BS) * order + cb * 64u;
+        const uint32_t c4 = (t & 15u) * 4u;
+#pragma unroll
+        for (int p = 0; p < BS / 16; ++p) {
+            const uint32_t r = (uint32_t)p * 16u + (t >> 4);
+            const float4 v = *reinterpret_cast<const float4 *>(src + (size_t)r * order + c4);
+            tile[(c4 + 0) * LD + r] = v.x;
+            tile[(c4 + 1) * LD + r] = v.y;
+            tile[(c4 + 2) * LD + r] = v.z;
+            tile[(c4 + 3) * LD + r] = v.w;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 16 / SEGS; ++q) {
+            const uint32_t cl = w * 16u + (uint32_t)q * SEGS + lane / G;       // output row inside the tile
+            const uint32_t e0 = (lane % G) * 4u;                               // first of this lane's four elements
+            float x[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = tile[cl * LD + e0 + e];
+            uint32_t m = max(max(abs_bits(x[0]), abs_bits(x[1])), max(abs_bits(x[2]), abs_bits(x[3])));
+            m = group_max_u32<G>(m);
+            const bool special = !fast_ok || (m - kFastDivLo) > (kFastDivHi - kFastDivLo);
+            uint32_t idx[4];
+            if (__any(special)) {
+                if (m > 0x7f800000u) m = 0x7fc00000u;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) idx[e] = exact_index<NCODE>(x[e], m, tab);
+            } else {
+                const float amax = __uint_as_float(m);
+                const float r = exact_reciprocal(amax);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    idx[e] = fast_index<NCODE, false>(x[e], amax, r, tab, nullptr);
+                    if (!ascending) idx[e] = tab.perm[idx[e]];
+                }
+            }
+            const size_t orow = (size_t)b * order + cb * 64u + cl;            // row of the stack of transposes
+            if (lane % G == 0) absmax[orow * tiles_r + rb] = __uint_as_float(m);
+            const size_t k = orow * order + (size_t)rb * BS + e0;             // flat element index of x[0]
+            if (BITS == 4)
+                *reinterpret_cast<uint16_t *>(out + (k >> 1)) = (uint16_t)(((idx[0] << 4) | idx[1]) | (((idx[2] << 4) | idx[3]) << 8));
+            else
+                *reinterpret_cast<uint32_t *>(out + k) = idx[0] | (idx[1] << 8) | (idx[2] << 16) | (idx[3] << 24);
+        }
+        __syncthreads();                                                       // the next tile rewrites the LDS copy
+    }
+}
+
 int grid_for(uint32_t work_items_per_block_unit, int blocks_per_cu) {
     const int cap = compute_units() * blocks_per_cu;
     const int need = (int)work_items_per_block_unit;
@@ -413,4 +485,35 @@ extern "C" void qtensor_hip_quantize_batched(const void *A, int a_is_bf16, const
     if (a_is_bf16) { if (bits == 4) QT_QB(uint16_t, 4); else QT_QB(uint16_t, 8); }
     else { if (bits == 4) QT_QB(float, 4); else QT_QB(float, 8); }
 #undef QT_QB
+}
+
+extern "C" void qtensor_hip_quantize_transposed_batched(const float *A, const float *code, int bits, int order, int batch,
+                                                        float *absmax, unsigned char *out, int blocksize, void *stream) {
+    using namespace qt;
+    clear_error();
+    if (bits != 4 && bits != 8) { set_error(kBadArgument, "quantize_transposed: bits must be 4 or 8"); return; }
+    if (blocksize != 64 && blocksize != 128 && blocksize != 256) {
+        set_error(kBadBlocksize, "quantize_transposed: blocksize %d is not one of 64,128,256", blocksize);
+        return;
+    }
+    if (order < 1 || batch < 1 || (int64_t)order * order * batch >= (int64_t(1) << 31) || order % blocksize != 0 || order % 64 != 0) {
+        set_error(kBadOrder, "quantize_transposed: order %d (batch %d) must be a multiple of 64 and of the blocksize, batch*order*order < 2^31",
+                  order, batch);
+        return;
+    }
+    if (!A || !code || !absmax || !out) { set_error(kNullPointer, "quantize_transposed: null device pointer"); return; }
+    if (!is_aligned(A, 16) || !is_aligned(out, 4) || !is_aligned(absmax, 4)) {
+        set_error(kBadArgument, "quantize_transposed: A needs 16-byte, out and absmax 4-byte alignment");
+        return;
+    }
+    const uint32_t tiles_r = (uint32_t)(order / blocksize), tiles_c = (uint32_t)(order / 64);
+    const uint32_t n_tiles = tiles_r * tiles_c * (uint32_t)batch;
+    const int grid = grid_for(n_tiles, blocksize == 256 ? 2 : 4);
+#define QT_QT(BITS, BS)                                                                                                  \
+    hipLaunchKernelGGL((quantize_transposed_kernel<BITS, BS>), dim3(grid), dim3(kThreads), 0, (hipStream_t)stream, A, code, \
+                       (uint32_t)order, n_tiles, tiles_r, tiles_c, absmax, out)
+    if (bits == 4) { if (blocksize == 64) QT_QT(4, 64); else if (blocksize == 128) QT_QT(4, 128); else QT_QT(4, 256); }
+    else { if (blocksize == 64) QT_QT(8, 64); else if (blocksize == 128) QT_QT(8, 128); else QT_QT(8, 256); }
+#undef QT_QT
+    launch_ok("quantize_transposed");
 }

@@ -121,7 +121,7 @@ class ShampooBank2(ShampooBank):
                 self.keep[order] = where[:, :half].contiguous()
                 self.svalue[order] = ascending[:, :half].contiguous()
                 self.max_eig[order] = quotients.amax(dim=1)
-                X.quantize_stack(Q.transpose(1, 2).contiguous(), self.basis[order])
+                X.quantize_stack(Q, self.basis[order], transposed=True)                # rows of the stored matrix = columns of Q
             return run
 
         self._fan_out([rebuild(o) for o in orders])

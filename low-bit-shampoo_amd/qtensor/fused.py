@@ -246,6 +246,9 @@ if F.lib is not None:
     F.lib.qtensor_hip_quantize_batched.restype = None
     F.lib.qtensor_hip_quantize_batched.argtypes = [ct.c_void_p, ct.c_int, ct.c_void_p, ct.c_int, ct.c_int, ct.c_int,
                                                    ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_void_p]
+    F.lib.qtensor_hip_quantize_transposed_batched.restype = None
+    F.lib.qtensor_hip_quantize_transposed_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_int,
+                                                              ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_void_p]
     F.lib.qtensor_hip_dequantize_batched.restype = None
     F.lib.qtensor_hip_dequantize_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_int, ct.c_void_p,
                                                      ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
@@ -260,9 +263,12 @@ def empty_quantized(batch: int, order: int, blocksize: int, bits: int, code: Ten
     return Quantized(codes, absmax, diag, order, blocksize, bits, code)
 
 
-def quantize_stack(mats: Tensor, q: Quantized) -> Quantized:
+def quantize_stack(mats: Tensor, q: Quantized, transposed: bool = False) -> Quantized:
     """Quantize the contiguous stack mats [batch, order, order] (fp32 or bf16) into q's buffers in one
-    launch; entry b equals quantize_blockwise(_diagreal)(mats[b])."""
+    launch; entry b equals quantize_blockwise(_diagreal)(mats[b]) -- of mats[b].T with transposed=True,
+    which reads the stack as it lies (one kernel turns 64-column tiles around on the way; reference:
+    V.T.contiguous() before the quantizer, qtensor/utils.py:169-170) when the form is plain, the input
+    fp32, and the blocksize is 64, 128 or 256 and divides an order that is a multiple of 64."""
     if F.lib is None:
         raise RuntimeError("libqtensor_hip.so is not available")
     if not mats.is_cuda or not mats.is_contiguous() or mats.shape != (q.batch, q.order, q.order):
@@ -271,6 +277,13 @@ def quantize_stack(mats: Tensor, q: Quantized) -> Quantized:
     for t in (q.codes, q.absmax) + ((q.diag,) if q.diag is not None else ()):
         if not t.is_contiguous():
             raise ValueError("stacked quantized buffers must be contiguous")
+    if transposed:
+        if (q.diag is None and mats.dtype == torch.float32 and q.blocksize in (64, 128, 256)
+                and q.order % q.blocksize == 0 and q.order % 64 == 0):
+            F._call(F.lib.qtensor_hip_quantize_transposed_batched, mats.device, mats.data_ptr(), q.code.data_ptr(), q.bits,
+                    q.order, q.batch, q.absmax.data_ptr(), q.codes.data_ptr(), q.blocksize)
+            return q
+        mats = mats.transpose(1, 2).contiguous()
     F._call(F.lib.qtensor_hip_quantize_batched, mats.device, mats.data_ptr(), slot, q.code.data_ptr(), q.bits, q.order,
             q.batch, q.absmax.data_ptr(), None if q.diag is None else q.diag.data_ptr(), q.codes.data_ptr(), q.blocksize)
     return q

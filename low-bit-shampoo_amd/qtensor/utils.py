@@ -169,11 +169,14 @@ class QTensorSVDFast(_LowBitState):
         dropped = ascending[keep:].to(var.dtype)
         self.max_eigenvalue = quotients.max().to(var.dtype)
 
-        rows = V.T.contiguous()
-        if self.bits < 16:
-            F.quantize_blockwise(rows, absmax=self.absmax, out=self.var, **self._kw())
+        if self.bits >= 16:
+            self.var = V.T.contiguous()
+        elif V.is_cuda and V.dtype == torch.float32 and V.is_contiguous() and self.var_order % self.blocksize == 0:
+            # the quantizer reads V as it lies and writes the codes of V.T (no transposed copy)
+            from qtensor import fused
+            fused.quantize_stack(V.unsqueeze(0), fused.Quantized.from_holder(self), transposed=True)
         else:
-            self.var = rows
+            F.quantize_blockwise(V.T.contiguous(), absmax=self.absmax, out=self.var, **self._kw())
 
         if self.log_prefix and not self._log_written:
             self._dump_spectrum(self.Svalue.detach().cpu(), dropped.detach().cpu())

@@ -240,6 +240,35 @@ def test_stack_quantize_dequantize_equal_per_matrix_calls(mods, code_maps, bits,
                 assert np.array_equal(back16[b].float().cpu().numpy(), want16)
 
 
+@pytest.mark.parametrize("bits,bs,name,n,batch", [(4, 64, "linear-2", 768, 3), (4, 64, "linear-2", 64, 9), (8, 64, "linear-2", 192, 2),
+                                                   (8, 256, "dynamic", 512, 3), (4, 128, "dynamic", 384, 2), (4, 256, "linear-2", 256, 2)])
+def test_quantizer_reading_the_transpose_equals_the_oracle_on_the_transposed_matrix(mods, code_maps, bits, bs, name, n, batch):
+    """quantize_stack(..., transposed=True) never writes the transpose; codes and maxima must be the oracle's for
+    mats[b].T bit for bit, including zero segments, tiny / huge / NaN maxima (exact-division route) and a
+    table handed over in descending order."""
+    F, X = mods
+    g = torch.Generator().manual_seed(7 * n + batch)
+    mats = torch.randn(batch, n, n, generator=g)
+    mats[0, :64, 3] = 0.0                                        # a zero segment of row 3 of the transpose
+    mats[0, :64, 5] *= 1e-30                                     # maxima outside the fast-division range
+    mats[0, :64, 6] *= 1e30
+    mats[batch - 1, 10, 7] = float("nan")
+    for code in (code_maps[(name, bits)], code_maps[(name, bits)][::-1].copy()):
+        code_d = torch.from_numpy(code).cuda()
+        q = X.quantize_stack(mats.cuda(), X.empty_quantized(batch, n, bs, bits, code_d, False), transposed=True)
+        torch.cuda.synchronize()
+        for b in range(batch):
+            o = Q.quantize_c(mats[b].T.contiguous().numpy(), code, n, bs, bits, False)
+            assert np.array_equal(q.codes[b].cpu().numpy(), o[0])
+            assert np.array_equal(q.absmax[b].cpu().numpy(), o[1], equal_nan=True)
+    # forms the kernel does not take go through a transposed copy and the ordinary quantizer
+    code = code_maps[(name, bits)]
+    code_d = torch.from_numpy(code).cuda()
+    q = X.quantize_stack(mats.cuda(), X.empty_quantized(batch, n, bs, bits, code_d, True), transposed=True)
+    o = Q.quantize_c(mats[0].T.contiguous().numpy(), code, n, bs, bits, True)
+    assert np.array_equal(q.codes[0].cpu().numpy(), o[0]) and np.array_equal(q.diag[0].cpu().numpy(), o[2])
+
+
 @pytest.mark.parametrize("m,n,k,batch", [(768, 3072, 3072, 1), (256, 256, 2048, 2), (100, 260, 1024, 1)])
 def test_products_split_along_k_equal_the_unsplit_ones_to_rounding(mods, m, n, k, batch, monkeypatch):
     """Few output tiles and a long k range: the library cuts k into slices whose partial products go through
