@@ -389,8 +389,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     constexpr bool A_RM = LoaderA::kRowMajor, B_RM = LoaderB::kRowMajor;
     constexpr int LDA = BM + LDS_PAD, LDB = BN + LDS_PAD;
     constexpr int SIZE_A = A_RM ? BM * LDK : BK * LDA, SIZE_B = B_RM ? BN * LDK : BK * LDB;
-    __shared__ __attribute__((aligned(16))) float s_a[2][SIZE_A];
-    __shared__ __attribute__((aligned(16))) float s_b[2][SIZE_B];
+    // one buffer: the two stages of both operand tiles during the main loop, then (symmetric products)
+    // a 32 x 32 staging square per wave that turns accumulator blocks around for the mirrored stores
+    constexpr int STAGE_LD = 36, SIZE_STAGE = 4 * 32 * STAGE_LD, SIZE_MAIN = 2 * SIZE_A + 2 * SIZE_B;
+    __shared__ __attribute__((aligned(16))) float s_mem[SIZE_MAIN > SIZE_STAGE ? SIZE_MAIN : SIZE_STAGE];
+    float (*s_a)[SIZE_A] = reinterpret_cast<float (*)[SIZE_A]>(s_mem);
+    float (*s_b)[SIZE_B] = reinterpret_cast<float (*)[SIZE_B]>(s_mem + 2 * SIZE_A);
     __shared__ float s_code[256];
     constexpr bool kNeedCode = KA >= kQuant4 || KB >= kQuant4 || EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8;
     if (kNeedCode) {
@@ -515,7 +519,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
         __syncthreads();
     }
 
-    // ---- epilogue: accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
+    // ---- epilogue
     float *C = const_cast<float *>(batch_ptr<float>(args.C, b));
     int ldc = args.ldc;
     if (slices > 1) {                              // partial product of this slice: summed by reduce_slices_kernel
@@ -532,29 +536,74 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     // an off-diagonal tile of a symmetric product also provides its mirror image; the addend is
     // read at the mirrored position, so an addend that is not exactly symmetric is honoured
     const bool mirror = args.symmetric != 0 && tile_n != tile_m;
-    const bool mirror_vec = (args.M & 3) == 0 && (ldc & 3) == 0 && is_aligned16(C) &&
-                            (EPI != kNewton || ((args.ldt & 3) == 0 && is_aligned16(T))) &&
-                            (EPI != kAxpbyDense || ((args.lde & 3) == 0 && is_aligned16(E)));
+    const bool vec_ok = (ldc & 3) == 0 && is_aligned16(C) &&
+                        (EPI != kNewton || ((args.ldt & 3) == 0 && is_aligned16(T))) &&
+                        (EPI != kAxpbyDense || ((args.lde & 3) == 0 && is_aligned16(E)));
+    const bool mirror_vec = vec_ok && (args.M & 3) == 0;
+    const bool direct_vec = vec_ok && (args.N & 3) == 0;
     float local_err = 0.0f;
+    // Each wave passes its accumulator blocks (32 x 32) through a staging square of its own in LDS, so that a
+    // lane ends up with four consecutive elements of one output row: 16-byte stores, eight lanes per 128-byte
+    // line, and one packed load per four elements of a quantized addend.
+    float *stage = s_mem + wave * (32 * STAGE_LD);
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
-            const int col = n0 + wn + j * 32 + (lane & 31);
+            if (direct_vec) {
 #pragma unroll
-            for (int rq = 0; rq < 4; ++rq) {
-                const int row4 = m0 + wm + i * 32 + 8 * rq + 4 * (lane >> 5);
+                for (int r = 0; r < 16; ++r)
+                    stage[(8 * (r / 4) + 4 * (lane >> 5) + r % 4) * STAGE_LD + (lane & 31)] = acc[i][j][r];
+                wave_lds_sync();
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int row = row4 + q;
+                for (int p = 0; p < 4; ++p) {
+                    const int ml = p * 8 + (lane >> 3), nl = (lane & 7) * 4;
+                    const float4 a4 = *reinterpret_cast<const float4 *>(stage + ml * STAGE_LD + nl);
+                    float y[4] = {a4.x, a4.y, a4.z, a4.w};
+                    const int row = m0 + wm + i * 32 + ml, col4 = n0 + wn + j * 32 + nl;
+                    if (row >= args.M || col4 >= args.N) continue;           // N % 4 == 0: col4 + 3 < N
+                    if (EPI == kAxpbyDense) {
+                        const float4 x = gload4(E + (long long)row * args.lde + col4);
+                        const float e[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) y[q] = args.beta * e[q] + args.alpha * y[q];
+                    } else if (kQuantAddend) {
+                        float e[4];
+                        dequant_four<EBITS>(e_codes, e_absmax, s_code, args.Eq.order, args.Eq.bs_shift, row, col4, e);
+                        if (e_diag != nullptr && (unsigned)(row - col4) < 4u) {
+                            const float d = gload(e_diag + row);
+#pragma unroll
+                            for (int q = 0; q < 4; ++q) if (row == col4 + q) e[q] = d;
+                        }
+                        // same two roundings as tensor.mul_(beta).add_(S, alpha=1-beta)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) y[q] = __builtin_fmaf(args.alpha, y[q], args.beta * e[q]);
+                    } else if (EPI == kNewton) {
+                        float t[4];
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const float eye = row == col4 + q ? 1.0f : 0.0f;
+                            local_err = fmaxf(local_err, fabsf(y[q] - eye));
+                            t[q] = (1.0f - args.newton_w) * eye + args.newton_w * y[q];
+                        }
+                        gstore4(T + (long long)row * args.ldt + col4, t);
+                    }
+                    gstore4(C + (long long)row * ldc + col4, y);
+                }
+                wave_lds_sync();
+            } else {
+                // accumulator register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the block
+                const int col = n0 + wn + j * 32 + (lane & 31);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int row = m0 + wm + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + r % 4;
                     if (row >= args.M || col >= args.N) continue;
-                    float y = acc[i][j][4 * rq + q];
+                    float y = acc[i][j][r];
                     if (EPI == kAxpbyDense) {
                         y = args.beta * gload(E + (long long)row * args.lde + col) + args.alpha * y;
                     } else if (kQuantAddend) {
                         const float e = dequant_element<EBITS>(e_codes, e_absmax, e_diag, s_code, args.Eq.order,
                                                                args.Eq.bs_shift, row, col);
-                        // same two roundings as tensor.mul_(beta).add_(S, alpha=1-beta)
                         y = __builtin_fmaf(args.alpha, y, args.beta * e);
                     } else if (EPI == kNewton) {
                         const float eye = row == col ? 1.0f : 0.0f;
@@ -563,42 +612,57 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
                     }
                     gstore(C + (long long)row * ldc + col, y);
                 }
-                if (!mirror || col >= args.N || row4 >= args.M) continue;
-                // mirrored: elements (col, row4 .. row4+3), never on the diagonal
+            }
+            if (!mirror) continue;
+            // The mirror image of the block: staged as [column][row], read back as 16 bytes along the row
+            // index, stored as 128-byte runs of the mirrored rows.
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                stage[(lane & 31) * STAGE_LD + 8 * (r / 4) + 4 * (lane >> 5) + r % 4] = acc[i][j][r];
+            wave_lds_sync();
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int nl = p * 8 + (lane >> 3), ml = (lane & 7) * 4;
+                const float4 a4 = *reinterpret_cast<const float4 *>(stage + nl * STAGE_LD + ml);
+                const float a[4] = {a4.x, a4.y, a4.z, a4.w};
+                const int mrow = n0 + wn + j * 32 + nl;         // row of the mirrored elements (a column of the tile)
+                const int mcol = m0 + wm + i * 32 + ml;         // their first column (a row of the tile)
+                if (mrow >= args.N || mcol >= args.M) continue;
+                // elements (mrow, mcol .. mcol+3), never on the diagonal
                 float y[4], e[4] = {0.f, 0.f, 0.f, 0.f};
-                const bool whole = mirror_vec;                  // M % 4 == 0: row4 + 3 < M
+                const bool whole = mirror_vec;                  // M % 4 == 0: mcol + 3 < M
                 if (EPI == kAxpbyDense) {
-                    if (whole) { const float4 x = gload4(E + (long long)col * args.lde + row4); e[0] = x.x; e[1] = x.y; e[2] = x.z; e[3] = x.w; }
+                    if (whole) { const float4 x = gload4(E + (long long)mrow * args.lde + mcol); e[0] = x.x; e[1] = x.y; e[2] = x.z; e[3] = x.w; }
                     else
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) if (row4 + q < args.M) e[q] = gload(E + (long long)col * args.lde + row4 + q);
+                        for (int q = 0; q < 4; ++q) if (mcol + q < args.M) e[q] = gload(E + (long long)mrow * args.lde + mcol + q);
                 } else if (kQuantAddend) {
                     // flat quantized layout: the order is a multiple of 64, so the four codes share a segment
-                    dequant_four<EBITS>(e_codes, e_absmax, s_code, args.Eq.order, args.Eq.bs_shift, col, row4, e);
+                    dequant_four<EBITS>(e_codes, e_absmax, s_code, args.Eq.order, args.Eq.bs_shift, mrow, mcol, e);
                 }
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const float a = acc[i][j][4 * rq + q];
-                    if (EPI == kAxpbyDense) y[q] = args.beta * e[q] + args.alpha * a;
-                    else if (kQuantAddend) y[q] = __builtin_fmaf(args.alpha, a, args.beta * e[q]);
-                    else y[q] = a;
+                    if (EPI == kAxpbyDense) y[q] = args.beta * e[q] + args.alpha * a[q];
+                    else if (kQuantAddend) y[q] = __builtin_fmaf(args.alpha, a[q], args.beta * e[q]);
+                    else y[q] = a[q];
                 }
-                float *cm = C + (long long)col * ldc + row4;
+                float *cm = C + (long long)mrow * ldc + mcol;
                 if (whole) gstore4(cm, y);
                 else
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) if (row4 + q < args.M) gstore(cm + q, y[q]);
+                    for (int q = 0; q < 4; ++q) if (mcol + q < args.M) gstore(cm + q, y[q]);
                 if (EPI == kNewton) {
                     float t[4];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) t[q] = args.newton_w * y[q];
-                    float *tm = T + (long long)col * args.ldt + row4;
+                    float *tm = T + (long long)mrow * args.ldt + mcol;
                     if (whole) gstore4(tm, t);
                     else
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) if (row4 + q < args.M) gstore(tm + q, t[q]);
+                        for (int q = 0; q < 4; ++q) if (mcol + q < args.M) gstore(tm + q, t[q]);
                 }
             }
+            wave_lds_sync();
         }
     if (EPI == kNewton) {
         uint32_t e = group_max_u32<64>(__float_as_uint(local_err));   // non-negative floats order like their bits
