@@ -120,7 +120,12 @@ def fused_step(opt, group, update, group_index=0):
             grafted = set(directions)
     for p in params:
         if id(p) not in entry['ids']:
-            directions[id(p)] = opt._shampoo_direction(p, grads[id(p)], group, opt.state[p])
+            # into a buffer that stays where it is: the fused update keeps a device table of addresses
+            d = opt._shampoo_direction(p, grads[id(p)], group, opt.state[p])
+            kept = entry.setdefault('directions', {})
+            if id(p) not in kept or kept[id(p)].shape != d.shape or kept[id(p)].dtype != d.dtype:
+                kept[id(p)] = torch.empty_like(d, memory_format=torch.contiguous_format)
+            directions[id(p)] = kept[id(p)].copy_(d)
     update(opt, group, params, [directions.get(id(p), grads[id(p)]) for p in params], [grads[id(p)] for p in params],
            [id(p) in grafted for p in params], step, entry)
 

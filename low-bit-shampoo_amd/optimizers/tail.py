@@ -31,6 +31,7 @@ class TailPlan:
         self.chunk = F.lib.qtensor_hip_tail_chunk()
         self.key = None
         self.keep = None
+        self.partial = None
 
     def _prepare(self, params, dirs, grads, m, v, graft):
         key = tuple((p.data_ptr(), d.data_ptr(), g.data_ptr(), a.data_ptr(), 0 if b is None else b.data_ptr(), bool(f))
@@ -49,9 +50,12 @@ class TailPlan:
             owner += [i] * chunks
             first += chunks
         dev = params[0].device
-        self.table = torch.tensor(rows, dtype=torch.int64).to(dev)
-        self.owner = torch.tensor(owner, dtype=torch.int32).to(dev)
-        self.partial = torch.empty(2 * max(first, 1), dtype=torch.float32, device=dev)
+        # through pinned memory and without blocking: a pageable copy would make the host wait for
+        # everything the step has queued so far
+        self.table = torch.tensor(rows, dtype=torch.int64).pin_memory().to(dev, non_blocking=True)
+        self.owner = torch.tensor(owner, dtype=torch.int32).pin_memory().to(dev, non_blocking=True)
+        if self.partial is None or self.partial.numel() != 2 * max(first, 1) or self.partial.device != dev:
+            self.partial = torch.empty(2 * max(first, 1), dtype=torch.float32, device=dev)
         self.n_chunks = first
         self.any_graft = any(graft)
         self.key = key
