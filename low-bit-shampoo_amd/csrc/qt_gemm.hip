@@ -263,7 +263,8 @@ struct LoadQuant {
     int code_off[GROUPS], amax_off[GROUPS], d0[GROUPS], drow[GROUPS];
     const uint8_t *codes;
     const float *absmax, *diag;
-    int order, per_row, shift;
+    int order, per_row, shift, first_row;
+    bool on_diagonal;                                        // the fetched tile holds diagonal entries (uniform over the workgroup)
     __device__ __forceinline__ bool active(int g) const { return (int)threadIdx.x + g * 256 < TOTAL; }
     __device__ __forceinline__ void locate(int g, int &mr, int &mc) const {
         const int f = threadIdx.x + g * 256;
@@ -275,6 +276,8 @@ struct LoadQuant {
         absmax = batch_ptr<float>(q.absmax, b);
         diag = has_ptr(q.diag) ? batch_ptr<float>(q.diag, b) : nullptr;
         order = q.order; shift = q.bs_shift; per_row = q.order >> q.bs_shift;
+        first_row = row0;
+        on_diagonal = false;
 #pragma unroll
         for (int g = 0; g < GROUPS; ++g) {
             int tr, tc;
@@ -295,17 +298,21 @@ struct LoadQuant {
         const long long step = ALONG_K ? k0 : (long long)k0 * order;
         const uint8_t *c = codes + (BITS == 4 ? step >> 1 : step);
         const float *a = absmax + (ALONG_K ? k0 >> shift : k0 * per_row);
+        // the tile spans BK of one index and ROWS of the other: only the few tiles that cross the diagonal
+        // need the exact diagonal entries
+        on_diagonal = diag != nullptr && k0 + BK > first_row && k0 < first_row + ROWS;
 #pragma unroll
         for (int g = 0; g < GROUPS; ++g) {
             if (!active(g)) continue;
             amax[g] = gload(a + amax_off[g]);
             if (BITS == 4) raw[g].x = gload_u32(c + code_off[g]);
             else raw[g] = gload_u32x2(c + code_off[g]);
+            if (!on_diagonal) continue;
             if (ALONG_K) {
-                dpos[g] = diag != nullptr ? d0[g] - k0 : -1;
+                dpos[g] = d0[g] - k0;
             } else {
-                dpos[g] = diag != nullptr ? d0[g] + k0 : -1;
-                if (diag != nullptr) dval[g] = gload(diag + min(drow[g] + k0, order - 1));
+                dpos[g] = d0[g] + k0;
+                dval[g] = gload(diag + min(drow[g] + k0, order - 1));
             }
         }
     }
@@ -323,11 +330,13 @@ struct LoadQuant {
 #pragma unroll
             for (int e = 0; e < 4; ++e) { id[e] = (raw[g].x >> (8 * e)) & 255u; id[4 + e] = (raw[g].y >> (8 * e)) & 255u; }
         }
+        // (a zero maximum gives +-0 here where the dequantizer writes +0: the same contribution to a product)
         const float a = amax[g];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float x = a == 0.0f ? 0.0f : s_code[id[e]] * a;
-            v[e] = e == dpos[g] ? dval[g] : x;
+        for (int e = 0; e < 8; ++e) v[e] = s_code[id[e]] * a;
+        if (on_diagonal) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = e == dpos[g] ? dval[g] : v[e];
         }
     }
     __device__ __forceinline__ void commit(float *lds, const float *s_code) const {
