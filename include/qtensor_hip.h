@@ -175,6 +175,13 @@ typedef struct {
                                  * slices whose partial products land here and are summed in a fixed order    */
         long long workspace_floats;
         int split_k_;           /* ignored (set by the library)                                             */
+        int batch_inner;        /* > 1: two-level batch for the strided dense operands A, B, C, E (blocks inside the
+                                 * matrices of a stack): entry b lives at base + (b / batch_inner) * stride +
+                                 * (b % batch_inner) * inner_x elements; 0 or 1: plain batch                    */
+        long long inner_a, inner_b, inner_c, inner_e;
+        int triangular;         /* bit 0: A is upper triangular (A[m][k] = 0 for k < m), bit 1: B is upper triangular
+                                 * (B[k][n] = 0 for k > n), square in their k index: the zero part of the k range is
+                                 * skipped (dense operands only, not with `symmetric`)                           */
     } args;
 } qtensor_gemm_desc;
 
@@ -190,13 +197,18 @@ void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
  * Stacks are contiguous [batch, n, n] fp32 with n a multiple of 64; everything runs on `stream`.
  *
  * cholesky_upper: gram (upper triangle read, contents destroyed) = U^T U.  u receives the block
- *   rows of U on and above the diagonal (the part below the diagonal blocks is not written),
- *   inv [batch, n/64, 64, 64] the inverses of U's diagonal blocks.  info[b] (zeroed by the caller)
- *   is set to 1 when matrix b has a non-positive pivot (its factor is then meaningless).
- * solve_upper_right: x = q U^-1 for q, x [batch, rows, n] with u, inv from cholesky_upper;
- *   panel is scratch of batch * rows * 64 floats.  x must not alias q. */
-void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float *inv, int *info, int n, int batch, qtensor_stream_t stream);
-void qtensor_hip_solve_upper_right_batched(const float *q, const float *u, const float *inv, float *panel, float *x,
+ *   rows of U on and above the diagonal (the part below the diagonal blocks is not written); the
+ *   64 x 64 diagonal blocks of x [batch, n, n] receive the inverses of U's diagonal blocks (nothing
+ *   else of x is touched).  info[b] (zeroed by the caller) is set to 1 when matrix b has a
+ *   non-positive pivot (its factor is then meaningless).
+ * solve_upper_right: out = q U^-1 for q, out [batch, rows, n] with u, x from cholesky_upper.  x must
+ *   be zero below its diagonal blocks (zero it once before the first factorisation; no call writes
+ *   there).  Its inverted diagonal blocks are doubled level by level (two launches per level for all
+ *   blocks of all matrices) up to 256 x 256; then the column panels of that width are solved in turn,
+ *   out_j = (q_j - out_<j U_<j,j) x_jj.  work is scratch of batch * max(rows, n) * n floats (gram may
+ *   be passed when rows <= n).  out must not alias q. */
+void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float *x, int *info, int n, int batch, qtensor_stream_t stream);
+void qtensor_hip_solve_upper_right_batched(const float *q, const float *u, float *x, float *work, float *out,
                                            int rows, int n, int batch, qtensor_stream_t stream);
 
 /* ---- the elementwise end of an optimizer step for all parameters at once -------------------------

@@ -3,22 +3,26 @@
 // which replaces the QR factorisation the reference calls once per statistic and update
 // (torch.linalg.qr at qtensor/utils.py:157 of the reference).
 //
-// Both are blocked with 64-wide panels.  The only arithmetic done outside the matrix-core GEMM
-// (qtensor_hip_gemm) is the 64 x 64 diagonal block: one wave per matrix factors it in registers and
-// also inverts the factor, so that every panel solve becomes a product with that small inverse.
+// The only arithmetic done outside the matrix-core GEMM (qtensor_hip_gemm) is the 64 x 64 diagonal
+// block: one wave per matrix factors it in registers and also inverts the factor.
 //   factor:  for each block row j:  U_jj = chol(G_jj);  U_j,> = U_jj^-T G_j,>;  G_>,> -= U_j,>^T U_j,>
-//   solve :  for each block col j:  X_j = (Q_j - X_<j U_<j,j) U_jj^-1
+//   solve :  the inverted diagonal blocks are doubled up to 256 x 256 -- with blocks A, C already
+//            inverted and B the block of U between them, [A^-1 B; 0 C^-1] gets -A^-1 B C^-1; every level is
+//            two launches for all pairs of all matrices -- then, for each 256-wide column panel j,
+//            X_j = (Q_j - X_<j U_<j,j) U_jj^-1; products with a triangular factor skip its zero part.
 // All launches go to the caller's stream; nothing is allocated or synchronised here.
 #include "qt_common.h"
 
 #include "qtensor_hip.h"
 
+#include <cstdlib>
 #include <initializer_list>
 
 namespace qt {
 namespace {
 
 constexpr int NB = 64;
+constexpr int kSolvePanel = 256;       // diagonal blocks of the factor are inverted up to this size, then panels of that width are solved
 
 // One wave per matrix: upper Cholesky factor U (G = U^T U) of a 64 x 64 block and U^-1.
 // Reads the upper triangle of G only.  A non-positive (or NaN) pivot sets info[b] = 1 and is
@@ -37,7 +41,7 @@ __device__ __forceinline__ float lane_value(float x, int lane) {
 
 __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long long g_stride, int ldg, float *u,
                                                         long long u_stride, int ldu, float *inv, long long inv_stride,
-                                                        int *info) {
+                                                        int ldi, int *info) {
     __shared__ __attribute__((aligned(16))) float cols[NB][LDC];
     const int b = blockIdx.x, lane = threadIdx.x;
     const float *G = gram + (long long)b * g_stride;
@@ -79,7 +83,7 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
         }
     }
     float *U = u + (long long)b * u_stride;
-    float *I = inv + (long long)b * inv_stride + lane * NB;
+    float *I = inv + (long long)b * inv_stride + (long long)lane * ldi;
 #pragma unroll
     for (int r = 0; r < NB; ++r) U[(long long)r * ldu + lane] = r <= lane ? row[r] : 0.0f;        // U[r][lane] = L[lane][r]
 #pragma unroll
@@ -114,20 +118,18 @@ bool stack_args_ok(const char *what, int n, int batch, std::initializer_list<con
 }  // namespace
 }  // namespace qt
 
-extern "C" void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float *inv, int *info, int n, int batch, void *stream_v) {
+extern "C" void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float *x, int *info, int n, int batch, void *stream_v) {
     using namespace qt;
     clear_error();
-    if (!stack_args_ok("cholesky_upper_batched", n, batch, {gram, u, inv, info})) return;
+    if (!stack_args_ok("cholesky_upper_batched", n, batch, {gram, u, x, info})) return;
     hipStream_t stream = (hipStream_t)stream_v;
     const long long mat = (long long)n * n;
     const int blocks = n / NB;
-    const long long inv_mat = (long long)blocks * NB * NB;
     for (int j = 0; j < blocks; ++j) {
         const int j0 = j * NB, j1 = j0 + NB, rest = n - j1;
         const long long corner = (long long)j0 * n + j0;
-        float *inv_j = inv + (long long)j * NB * NB;
-        hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram + corner, mat, n, u + corner, mat, n, inv_j,
-                           inv_mat, info);
+        hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram + corner, mat, n, u + corner, mat, n, x + corner,
+                           mat, n, info);
         if (!launch_ok("cholesky_upper_batched (diagonal block)")) return;
         if (rest == 0) break;
         const long long row = (long long)j0 * n + j1;
@@ -135,7 +137,7 @@ extern "C" void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float 
         // U_j,> = U_jj^-T G_j,>
         d.M = NB; d.N = rest; d.K = NB; d.batch = batch;
         d.kind_a = QTENSOR_DENSE_T; d.kind_b = QTENSOR_DENSE; d.epilogue = QTENSOR_EPI_STORE;
-        d.args.A = strided(inv_j, inv_mat); d.args.lda = NB;
+        d.args.A = strided(x + corner, mat); d.args.lda = n;
         d.args.B = strided(gram + row, mat); d.args.ldb = n;
         d.args.C = strided(u + row, mat); d.args.ldc = n;
         if (!run(d, stream)) return;
@@ -154,41 +156,80 @@ extern "C" void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float 
     }
 }
 
-extern "C" void qtensor_hip_solve_upper_right_batched(const float *q, const float *u, const float *inv, float *panel, float *x,
+extern "C" void qtensor_hip_solve_upper_right_batched(const float *q, const float *u, float *x, float *work, float *out,
                                                       int rows, int n, int batch, void *stream_v) {
     using namespace qt;
     clear_error();
-    if (!stack_args_ok("solve_upper_right_batched", n, batch, {q, u, inv, panel, x})) return;
+    if (!stack_args_ok("solve_upper_right_batched", n, batch, {q, u, x, work, out})) return;
     if (rows < 1) { set_error(kBadArgument, "solve_upper_right_batched: rows must be positive"); return; }
     hipStream_t stream = (hipStream_t)stream_v;
     const long long mat = (long long)n * n, tall = (long long)rows * n;
-    const int blocks = n / NB;
-    const long long inv_mat = (long long)blocks * NB * NB;
-    for (int j = 0; j < blocks; ++j) {
-        const int j0 = j * NB;
+    static const char *top_env = getenv("QT_SOLVE_PANEL");
+    const int top = top_env != nullptr ? atoi(top_env) : kSolvePanel;
+    // x holds the inverses of the 64 x 64 diagonal blocks; every level doubles the size of the inverted blocks
+    for (int s = NB; s < n && s < top; s *= 2) {
+        const int full = n / (2 * s), rem = n % (2 * s);
+        for (int part = 0; part < 2; ++part) {
+            // part 0: the `full` pairs of two s-blocks of every matrix; part 1: a last pair whose second block is shorter
+            if (part == 0 ? full == 0 : rem <= s) continue;
+            const int c = part == 0 ? s : rem - s;
+            const long long first = part == 0 ? 0 : (long long)full * 2 * s * (n + 1);     // corner of the (first) pair
+            const int pairs = part == 0 ? full : 1;
+            if ((long long)batch * pairs > 65535) { set_error(kBadArgument, "solve_upper_right_batched: too many blocks"); return; }
+            const long long step = (long long)2 * s * (n + 1);
+            // work_B = U_B X_C
+            qtensor_gemm_desc w = {};
+            w.M = s; w.N = c; w.K = c; w.batch = batch * pairs;
+            w.kind_a = QTENSOR_DENSE; w.kind_b = QTENSOR_DENSE; w.epilogue = QTENSOR_EPI_STORE;
+            w.args.A = strided(u + first + s, mat); w.args.lda = n;
+            w.args.B = strided(x + first + (long long)s * (n + 1), mat); w.args.ldb = n;
+            w.args.C = strided(work + first + s, mat); w.args.ldc = n;
+            w.args.batch_inner = pairs;
+            w.args.inner_a = w.args.inner_b = w.args.inner_c = step;
+            w.args.triangular = 2;
+            if (!run(w, stream)) return;
+            // X_B = -X_A work_B
+            qtensor_gemm_desc v = {};
+            v.M = s; v.N = c; v.K = s; v.batch = batch * pairs;
+            v.kind_a = QTENSOR_DENSE; v.kind_b = QTENSOR_DENSE; v.epilogue = QTENSOR_EPI_AXPBY_DENSE;
+            v.args.A = strided(x + first, mat); v.args.lda = n;
+            v.args.B = strided(work + first + s, mat); v.args.ldb = n;
+            v.args.C = strided(x + first + s, mat); v.args.ldc = n;
+            v.args.E = strided(work + first + s, mat); v.args.lde = n;       // finite values; beta = 0
+            v.args.alpha = -1.0f; v.args.beta = 0.0f;
+            v.args.batch_inner = pairs;
+            v.args.inner_a = v.args.inner_b = v.args.inner_c = v.args.inner_e = step;
+            v.args.triangular = 1;
+            if (!run(v, stream)) return;
+        }
+    }
+    // block back-substitution over column panels whose diagonal blocks of x are now inverted:
+    //   out_j = (q_j - out_<j U_<j,j) X_jj
+    const int width = top < n ? top : n;
+    for (int j0 = 0; j0 < n; j0 += width) {
+        const int w = n - j0 < width ? n - j0 : width;
         const float *rhs = q + j0;
         long long rhs_stride = tall;
         int rhs_ld = n;
-        if (j > 0) {
-            // panel = Q_j - X_<j U_<j,j
+        if (j0 > 0) {
             qtensor_gemm_desc d = {};
-            d.M = rows; d.N = NB; d.K = j0; d.batch = batch;
+            d.M = rows; d.N = w; d.K = j0; d.batch = batch;
             d.kind_a = QTENSOR_DENSE; d.kind_b = QTENSOR_DENSE; d.epilogue = QTENSOR_EPI_AXPBY_DENSE;
-            d.args.A = strided(x, tall); d.args.lda = n;
+            d.args.A = strided(out, tall); d.args.lda = n;
             d.args.B = strided(u + j0, mat); d.args.ldb = n;
             d.args.E = strided(q + j0, tall); d.args.lde = n;
-            d.args.C = strided(panel, (long long)rows * NB); d.args.ldc = NB;
+            d.args.C = strided(work, (long long)rows * width); d.args.ldc = width;
             d.args.alpha = -1.0f; d.args.beta = 1.0f;
             if (!run(d, stream)) return;
-            rhs = panel; rhs_stride = (long long)rows * NB; rhs_ld = NB;
+            rhs = work; rhs_stride = (long long)rows * width; rhs_ld = width;
         }
-        // X_j = panel U_jj^-1
-        qtensor_gemm_desc s = {};
-        s.M = rows; s.N = NB; s.K = NB; s.batch = batch;
-        s.kind_a = QTENSOR_DENSE; s.kind_b = QTENSOR_DENSE; s.epilogue = QTENSOR_EPI_STORE;
-        s.args.A = strided(rhs, rhs_stride); s.args.lda = rhs_ld;
-        s.args.B = strided(inv + (long long)j * NB * NB, inv_mat); s.args.ldb = NB;
-        s.args.C = strided(x + j0, tall); s.args.ldc = n;
-        if (!run(s, stream)) return;
+        qtensor_gemm_desc t = {};
+        t.M = rows; t.N = w; t.K = w; t.batch = batch;
+        t.kind_a = QTENSOR_DENSE; t.kind_b = QTENSOR_DENSE; t.epilogue = QTENSOR_EPI_STORE;
+        t.args.A = strided(rhs, rhs_stride); t.args.lda = rhs_ld;
+        t.args.B = strided(x + (long long)j0 * (n + 1), mat); t.args.ldb = n;
+        t.args.C = strided(out + j0, tall); t.args.ldc = n;
+        t.args.triangular = 2;
+        if (!run(t, stream)) return;
     }
 }

@@ -65,6 +65,10 @@ struct GemmArgs {
     float *workspace;             // optional scratch for splitting k (plain-store products only)
     long long workspace_floats;
     int split_k;                  // set by the library: slices of the k range (1 = no split)
+    int batch_inner;              // > 1: batch entry b of the strided dense operands A, B, C, E lives at
+    long long inner_a, inner_b, inner_c, inner_e;   // base + (b / batch_inner) * stride + (b % batch_inner) * inner_x
+    int triangular;               // bit 0: A is upper triangular (A[m][k] = 0 for k < m): k starts at the tile's first row;
+                                  // bit 1: B is upper triangular (B[k][n] = 0 for k > n): k ends with the tile's last column
 };
 
 namespace {
@@ -101,6 +105,13 @@ __device__ __forceinline__ void gstore4(float *p, const float v[4]) {
 template <typename T>
 __device__ __forceinline__ const T *batch_ptr(const BatchPtr &p, int b) {
     return p.list ? reinterpret_cast<const T *>(p.list[b]) : reinterpret_cast<const T *>(p.base) + (long long)b * p.stride;
+}
+
+// Dense operand of batch entry b when the batch has two levels (blocks inside the matrices of a stack).
+__device__ __forceinline__ const float *dense_ptr(const BatchPtr &p, int b, int inner, long long inner_stride) {
+    if (p.list || inner <= 1) return batch_ptr<float>(p, b);
+    const int outer = b / inner;
+    return reinterpret_cast<const float *>(p.base) + outer * p.stride + (b - outer * inner) * inner_stride;
 }
 
 __device__ __forceinline__ bool has_ptr(const BatchPtr &p) { return p.base != nullptr || p.list != nullptr; }
@@ -416,8 +427,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
 
-    const float *A = (KA < kQuant4) ? batch_ptr<float>(args.A, b) : nullptr;
-    const float *B = (KB < kQuant4) ? batch_ptr<float>(args.B, b) : nullptr;
+    const float *A = (KA < kQuant4) ? dense_ptr(args.A, b, args.batch_inner, args.inner_a) : nullptr;
+    const float *B = (KB < kQuant4) ? dense_ptr(args.B, b, args.batch_inner, args.inner_b) : nullptr;
     const bool a_vec = KA < kQuant4 && (args.lda & 3) == 0 && is_aligned16(A);
     const bool b_vec = KB < kQuant4 && (args.ldb & 3) == 0 && is_aligned16(B);
 
@@ -463,8 +474,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     // its loads were issued a whole tile earlier) is written to the other buffer half-way through
     // the MFMA stream and the loads of tile t+2 are issued right after.  One barrier per tile.
     // (with k split into slices -- the host makes them equal -- this workgroup owns one of them)
-    const int n_tiles = (args.K + BK - 1) / BK / slices;
-    const int k_begin = slice * n_tiles * BK;
+    // (a triangular operand shortens the range to where it is not zero: tile origins are multiples of BK)
+    const int k_first = (args.triangular & 1) ? min(m0, args.K) : 0;
+    const int k_last = (args.triangular & 2) ? min(n0 + BN, args.K) : args.K;
+    const int n_tiles = max((k_last - k_first + BK - 1) / BK, 1) / slices;
+    const int k_begin = k_first + slice * n_tiles * BK;
     fetch(k_begin);
     la.commit(s_a[0], s_code);
     lb.commit(s_b[0], s_code);
@@ -529,14 +543,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     }
 
     // ---- epilogue
-    float *C = const_cast<float *>(batch_ptr<float>(args.C, b));
+    float *C = const_cast<float *>(dense_ptr(args.C, b, args.batch_inner, args.inner_c));
     int ldc = args.ldc;
     if (slices > 1) {                              // partial product of this slice: summed by reduce_slices_kernel
         C = args.workspace + ((long long)b * slices + slice) * args.M * args.N;
         ldc = args.N;
     }
     float *T = EPI == kNewton ? const_cast<float *>(batch_ptr<float>(args.T, b)) : nullptr;
-    const float *E = EPI == kAxpbyDense ? batch_ptr<float>(args.E, b) : nullptr;
+    const float *E = EPI == kAxpbyDense ? dense_ptr(args.E, b, args.batch_inner, args.inner_e) : nullptr;
     constexpr bool kQuantAddend = EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8;
     constexpr int EBITS = EPI == kAxpbyQuant8 ? 8 : 4;
     const uint8_t *e_codes = kQuantAddend ? batch_ptr<uint8_t>(args.Eq.codes, b) : nullptr;
@@ -790,6 +804,11 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
     }
     if (ep == kNewton && (!has_host_ptr(a.T) || a.ldt < d->N || !a.err)) { set_error(kBadArgument, "gemm: Newton epilogue needs T and err"); return; }
     a.symmetric = a.symmetric != 0;
+    if (a.triangular != 0 && (ka >= kQuant4 || kb >= kQuant4 || a.symmetric || (a.triangular & ~3) != 0)) {
+        set_error(kBadArgument, "gemm: triangular operands must be dense, in a product that is not marked symmetric");
+        return;
+    }
+    if (a.batch_inner < 0) { set_error(kBadArgument, "gemm: negative inner batch count"); return; }
     if (a.symmetric && (d->M != d->N || ka >= kQuant4 || kb >= kQuant4)) {
         set_error(kBadArgument, "gemm: symmetric products need M == N and dense operands");
         return;
@@ -830,7 +849,8 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
     // to the caller's workspace and are summed in order afterwards.  Same cost model, with a fixed cost per
     // workgroup (prologue, epilogue, the extra pass over the output) worth about 64 k steps.
     a.split_k = 1;
-    if (ep == kStore && !a.symmetric && a.workspace != nullptr && d->K % 16 == 0 && is_aligned(a.workspace, 16)) {
+    if (ep == kStore && !a.symmetric && a.batch_inner <= 1 && a.triangular == 0 && a.workspace != nullptr && d->K % 16 == 0 &&
+        is_aligned(a.workspace, 16)) {
         const Shape &sh = shapes[pick];
         const double units = compute_units();
         const long long tm = (d->M + sh.bm - 1) / sh.bm, tn = (d->N + sh.bn - 1) / sh.bn;

@@ -38,7 +38,9 @@ class GemmArgs(ct.Structure):
                 ("T", BatchPtr), ("ldt", ct.c_int),
                 ("newton_w", ct.c_float),
                 ("err", ct.c_void_p), ("skip", ct.c_void_p), ("code", ct.c_void_p), ("symmetric", ct.c_int),
-                ("workspace", ct.c_void_p), ("workspace_floats", ct.c_longlong), ("split_k_", ct.c_int)]
+                ("workspace", ct.c_void_p), ("workspace_floats", ct.c_longlong), ("split_k_", ct.c_int),
+                ("batch_inner", ct.c_int), ("inner_a", ct.c_longlong), ("inner_b", ct.c_longlong),
+                ("inner_c", ct.c_longlong), ("inner_e", ct.c_longlong), ("triangular", ct.c_int)]
 
 
 class GemmDesc(ct.Structure):
@@ -134,7 +136,8 @@ def _launch(desc: GemmDesc, device: torch.device) -> None:
 
 
 def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, alpha=1.0, beta=0.0,
-         addend=None, newton=None, skip: Optional[Tensor] = None, symmetric: bool = False) -> Tensor:
+         addend=None, newton=None, skip: Optional[Tensor] = None, symmetric: bool = False,
+         upper_a: bool = False, upper_b: bool = False) -> Tensor:
     """out[b] = epilogue(op(A[b]) @ op(B[b])).
 
     A, B: fp32 tensors ([m,k] / [batch,m,k]; with trans_x the stored matrix is the transpose) or a
@@ -145,7 +148,9 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
     skip: optional int32 [batch]; entries with a nonzero flag are not touched.
     symmetric: the caller knows the product to be symmetric (a Gram matrix, a product of commuting
     symmetric matrices): only the tiles on and above the diagonal are multiplied out and mirrored,
-    which halves the work; the result is then symmetric bit for bit outside the diagonal tiles."""
+    which halves the work; the result is then symmetric bit for bit outside the diagonal tiles.
+    upper_a / upper_b: op(A) / op(B) is upper triangular (zero below the diagonal, square in its k
+    index, dense): the part of the k range where it is zero is skipped."""
     d = GemmDesc()
     a = d.args
     dev = None
@@ -218,6 +223,10 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
         if m != n or isinstance(A, Quantized) or isinstance(B, Quantized):
             raise ValueError("symmetric products are square with dense operands")
         a.symmetric = 1
+    if upper_a or upper_b:
+        if symmetric or isinstance(A, Quantized) or isinstance(B, Quantized) or (upper_a and m != k) or (upper_b and n != k):
+            raise ValueError("triangular operands are dense and square, in a product that is not marked symmetric")
+        a.triangular = (1 if upper_a else 0) | (2 if upper_b else 0)
     if d.epilogue == EPI_STORE and not symmetric and k >= 256 and batch * m * n <= _WORKSPACE_FLOATS // 2:
         # few output tiles, long k: the library may cut k into slices (one scratch area per stream)
         scratch = _workspace(dev)
@@ -319,24 +328,28 @@ def _stack(t: Tensor, name: str, shape=None) -> Tensor:
     return t
 
 
-def cholesky_upper(gram: Tensor, u: Tensor, inv: Tensor, info: Tensor) -> None:
+def cholesky_upper(gram: Tensor, u: Tensor, x: Tensor, info: Tensor) -> None:
     """gram [B, n, n] (destroyed) = U^T U: block rows of U into u, inverses of its 64 x 64 diagonal blocks
-    into inv [B, n/64, 64, 64]; info int32 [B] (zeroed by the caller) flags non-positive pivots."""
+    into the diagonal blocks of x [B, n, n] (nothing else of x is written); info int32 [B] (zeroed by the
+    caller) flags non-positive pivots."""
     B, n, _ = gram.shape
-    _stack(gram, "gram", (B, n, n)), _stack(u, "u", (B, n, n)), _stack(inv, "inv", (B, n // 64, 64, 64))
+    _stack(gram, "gram", (B, n, n)), _stack(u, "u", (B, n, n)), _stack(x, "x", (B, n, n))
     if info.dtype != torch.int32 or info.numel() != B or not info.is_cuda:
         raise ValueError("info must be an int32 GPU vector with one entry per matrix")
-    F._call(F.lib.qtensor_hip_cholesky_upper_batched, gram.device, gram.data_ptr(), u.data_ptr(), inv.data_ptr(), info.data_ptr(), n, B)
+    F._call(F.lib.qtensor_hip_cholesky_upper_batched, gram.device, gram.data_ptr(), u.data_ptr(), x.data_ptr(), info.data_ptr(), n, B)
 
 
-def solve_upper_right(q: Tensor, u: Tensor, inv: Tensor, panel: Tensor, out: Tensor) -> Tensor:
-    """out = q U^-1 for q [B, rows, n] with u, inv from cholesky_upper; panel: scratch [B, rows, 64]."""
+def solve_upper_right(q: Tensor, u: Tensor, x: Tensor, work: Tensor, out: Tensor) -> Tensor:
+    """out = q U^-1 for q [B, rows, n] (rows <= n) with u, x from cholesky_upper; the inverted diagonal
+    blocks of x (zero below them) are doubled up to 256 x 256 on the way; work: scratch [B, n, n]."""
     B, rows, n = q.shape
-    _stack(q, "q"), _stack(u, "u", (B, n, n)), _stack(inv, "inv", (B, n // 64, 64, 64))
-    _stack(panel, "panel", (B, rows, 64)), _stack(out, "out", (B, rows, n))
+    _stack(q, "q"), _stack(u, "u", (B, n, n)), _stack(x, "x", (B, n, n)), _stack(work, "work", (B, n, n))
+    _stack(out, "out", (B, rows, n))
     if out.data_ptr() == q.data_ptr():
         raise ValueError("out must not alias q")
-    F._call(F.lib.qtensor_hip_solve_upper_right_batched, q.device, q.data_ptr(), u.data_ptr(), inv.data_ptr(), panel.data_ptr(),
+    if rows > n:
+        raise ValueError("the scratch area covers at most n rows")
+    F._call(F.lib.qtensor_hip_solve_upper_right_batched, q.device, q.data_ptr(), u.data_ptr(), x.data_ptr(), work.data_ptr(),
             out.data_ptr(), rows, n, B)
     return out
 
@@ -377,8 +390,8 @@ class CholeskyQR:
         scale = torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)
         self.Q = (Y / scale).contiguous()             # working set; unit columns: the Gram matrix has a unit diagonal
         self.ids = torch.arange(B, device=Y.device)   # which matrix of the stack each working-set entry is
-        self.U, self.inv = torch.empty_like(self.Q), torch.empty(B, n // 64, 64, 64, device=Y.device)
-        self.panel = torch.empty(B, n, 64, device=Y.device)
+        self.U = torch.empty_like(self.Q)
+        self.X = torch.zeros_like(self.Q)             # inverse factors; the part below the diagonal blocks stays zero
         self.info = torch.zeros(B, dtype=torch.int32, device=Y.device)
         self.final = torch.empty_like(self.Q)
         self.redo = []                                # matrices handed to the library at the end
@@ -433,9 +446,9 @@ class CholeskyQR:
         self.gram.diagonal(dim1=1, dim2=2).add_(1.0 + self.shift * shifted.to(self.gram.dtype).unsqueeze(1))
         info = self.info[:k]
         info.zero_()
-        cholesky_upper(self.gram, self.U[:k], self.inv[:k], info)
+        cholesky_upper(self.gram, self.U[:k], self.X[:k], info)
         out = torch.empty_like(self.Q)
-        solve_upper_right(self.Q, self.U[:k], self.inv[:k], self.panel[:k], out)
+        solve_upper_right(self.Q, self.U[:k], self.X[:k], self.gram, out)      # the Gram matrix is used up: scratch
         bad = info != 0
         self.fatal = self.fatal | (bad & (shifted | near))
         self.needs_shift = self.needs_shift | bad

@@ -269,6 +269,23 @@ def test_quantizer_reading_the_transpose_equals_the_oracle_on_the_transposed_mat
     assert np.array_equal(q.codes[0].cpu().numpy(), o[0]) and np.array_equal(q.diag[0].cpu().numpy(), o[2])
 
 
+@pytest.mark.parametrize("n,rows,batch", [(64, 64, 3), (320, 200, 2), (768, 768, 2)])
+def test_products_with_a_triangular_factor_skip_its_zero_part_and_change_nothing(mods, n, rows, batch):
+    _, X = mods
+    g = torch.Generator().manual_seed(n)
+    U = torch.triu(torch.randn(batch, n, n, generator=g))
+    Q = torch.randn(batch, rows, n, generator=g)
+    W = torch.randn(batch, n, rows, generator=g)
+    Ud, Qd, Wd = U.cuda(), Q.cuda(), W.cuda()
+    assert rel_err(X.gemm(Qd, Ud, upper_b=True), Q.double() @ U.double()) <= TOL
+    assert rel_err(X.gemm(Ud, Wd, upper_a=True), U.double() @ W.double()) <= TOL
+    assert rel_err(X.gemm(Ud, Ud, upper_a=True, upper_b=True), U.double() @ U.double()) <= TOL
+    E = torch.randn(batch, rows, n, generator=g).cuda()
+    assert rel_err(X.gemm(Qd, Ud, upper_b=True, addend=E, alpha=-1.0, beta=0.5), 0.5 * E.cpu().double() - Q.double() @ U.double()) <= TOL
+    with pytest.raises(ValueError):
+        X.gemm(Qd, torch.zeros(batch, n, n + 64, device="cuda"), upper_b=True)        # not square in its k index
+
+
 @pytest.mark.parametrize("m,n,k,batch", [(768, 3072, 3072, 1), (256, 256, 2048, 2), (100, 260, 1024, 1)])
 def test_products_split_along_k_equal_the_unsplit_ones_to_rounding(mods, m, n, k, batch, monkeypatch):
     """Few output tiles and a long k range: the library cuts k into slices whose partial products go through

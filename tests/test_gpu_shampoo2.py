@@ -30,14 +30,14 @@ def mods():
     return S2, E2
 
 
-@pytest.mark.parametrize("n,batch,rows", [(64, 3, 64), (256, 4, 256), (768, 2, 100)])
+@pytest.mark.parametrize("n,batch,rows", [(64, 3, 64), (256, 4, 256), (768, 2, 100), (320, 3, 320), (1024, 2, 130), (576, 1, 64)])
 def test_blocked_cholesky_and_right_solve_against_float64(mods, n, batch, rows):
     import qtensor.fused as X
     g = torch.Generator().manual_seed(n)
     A = torch.randn(batch, n, n, generator=g)
     G = (A.transpose(1, 2) @ A / n + 0.1 * torch.eye(n)).cuda()
     gram, U = G.clone(), torch.full((batch, n, n), 7.0, device="cuda")
-    inv = torch.empty(batch, n // 64, 64, 64, device="cuda")
+    inv = torch.zeros(batch, n, n, device="cuda")               # diagonal blocks: inverses of U's; below them: stays zero
     info = torch.zeros(batch, dtype=torch.int32, device="cuda")
     X.cholesky_upper(gram, U, inv, info)
     assert info.tolist() == [0] * batch
@@ -49,10 +49,18 @@ def test_blocked_cholesky_and_right_solve_against_float64(mods, n, batch, rows):
     assert rel(Ut, want) <= 1e-5
     for j in range(n // 64):
         blk = want[:, 64 * j:64 * j + 64, 64 * j:64 * j + 64]
-        assert rel(inv[:, j], torch.linalg.inv(blk)) <= 1e-4
+        assert rel(inv[:, 64 * j:64 * j + 64, 64 * j:64 * j + 64], torch.linalg.inv(blk)) <= 1e-4
+    off = (blocks[:, None] != blocks[None, :]).cuda()
+    assert bool((torch.where(off, inv, torch.zeros_like(inv)) == 0).all())       # nothing but the diagonal blocks written
     Q = torch.randn(batch, rows, n, generator=g).cuda()
     out = torch.empty_like(Q)
-    X.solve_upper_right(Q, U, inv, torch.empty(batch, rows, 64, device="cuda"), out)
+    X.solve_upper_right(Q, U, inv, gram, out)                  # doubles the inverted diagonal blocks up to 256 x 256
+    for j0 in range(0, n, 256):
+        j1 = min(j0 + 256, n)
+        assert rel(inv[:, j0:j1, j0:j1], torch.linalg.inv(want[:, j0:j1, j0:j1])) <= 1e-4
+    wide = torch.arange(n) // 256
+    assert bool((torch.where((wide[:, None] != wide[None, :]).cuda(), inv, torch.zeros_like(inv)) == 0).all())
+    assert bool((torch.tril(inv, -1) == 0).all())
     assert rel(out, torch.linalg.solve_triangular(want, Q.double().cpu(), upper=True, left=False)) <= 1e-4
     # a non-positive pivot is flagged, and only for its matrix
     bad = G.clone()
@@ -63,7 +71,7 @@ def test_blocked_cholesky_and_right_solve_against_float64(mods, n, batch, rows):
     assert rel(torch.where(keep, U, torch.zeros_like(U))[1:], want[1:]) <= 1e-5          # the others are unaffected
     with pytest.raises((RuntimeError, ValueError)):
         X.cholesky_upper(torch.zeros(1, 100, 100, device="cuda"), torch.zeros(1, 100, 100, device="cuda"),
-                         torch.zeros(1, 1, 64, 64, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda"))
+                         torch.zeros(1, 100, 100, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda"))
 
 
 def test_cholesky_qr_gives_the_householder_factor_up_to_signs(mods):
