@@ -32,7 +32,8 @@ constexpr int kSolvePanel = 256;       // diagonal blocks of the factor are inve
 // (one value per lane) into column k of L = U^T, parks it in LDS, and every lane reads it back as
 // 16-byte broadcasts: the same 64 values update the trailing matrix (a[i][j] -= L[i][k] L[j][k]) and
 // carry the forward substitution for column `lane` of L^-1 (s[j] -= L[j][k] x[k]), so the inverse
-// costs no second pass.  1 / sqrt(pivot) comes from v_rsq_f32 plus one Newton step.
+// costs no second pass.  1 / sqrt(pivot) comes from v_rsq_f32 plus one Newton step.  One block = one
+// wave: the wave-level fence below is all the synchronisation the LDS copy needs.
 constexpr int LDC = NB + 4;                      // LDS row stride: rows stay 16-byte aligned
 
 __device__ __forceinline__ float lane_value(float x, int lane) {
@@ -56,8 +57,17 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
     }
     __syncthreads();
     bool ok = true;
+    // Step k: pivot, column k of L, then the two next columns at once through v_readlane (they carry the
+    // chain from one pivot to the next); all further columns get the update of step k one step later, from
+    // the copy of column k parked in LDS, so that no pivot ever waits for an LDS round trip.
+    float l_prev = 0.0f, x_prev = 0.0f;
 #pragma unroll
     for (int k = 0; k < NB; ++k) {
+        float4 far[NB / 4];                      // column k-1 of L for the columns from k+2 on
+        if (k >= 1) {
+#pragma unroll
+            for (int j = (k + 2) & ~3; j < NB; j += 4) far[j / 4] = *reinterpret_cast<const float4 *>(&cols[k - 1][j]);
+        }
         float d = lane_value(row[k], k);
         if (!(d > 0.0f)) { ok = false; d = 1.0f; }
         float r = __builtin_amdgcn_rsqf(d);
@@ -65,22 +75,29 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
         const float l = row[k] * r;              // L[lane][k] (lanes above k: unused values)
         row[k] = l;
         s[k] *= r;                               // x[k] = s[k] / L[k][k]
-        if (k + 1 < NB) {
-            cols[k][lane] = l;
-            __syncthreads();
-            const float xk = s[k];
+        const float xk = s[k];
+        cols[k][lane] = l;
 #pragma unroll
-            for (int j = (k + 1) & ~3; j < NB; j += 4) {
-                const float4 c = *reinterpret_cast<const float4 *>(&cols[k][j]);
-                const float v[4] = {c.x, c.y, c.z, c.w};
+        for (int j = k + 1; j <= k + 2 && j < NB; ++j) {
+            const float v = lane_value(l, j);    // L[j][k]
+            row[j] = __builtin_fmaf(-l, v, row[j]);
+            s[j] = __builtin_fmaf(-v, xk, s[j]);
+        }
+        if (k >= 1) {
+#pragma unroll
+            for (int j = (k + 2) & ~3; j < NB; j += 4) {
+                const float v[4] = {far[j / 4].x, far[j / 4].y, far[j / 4].z, far[j / 4].w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    if (j + e > k) {
-                        row[j + e] = __builtin_fmaf(-l, v[e], row[j + e]);
-                        s[j + e] = __builtin_fmaf(-v[e], xk, s[j + e]);
+                    if (j + e >= k + 2) {
+                        row[j + e] = __builtin_fmaf(-l_prev, v[e], row[j + e]);
+                        s[j + e] = __builtin_fmaf(-v[e], x_prev, s[j + e]);
                     }
             }
         }
+        l_prev = l;
+        x_prev = xk;
+        wave_lds_sync();                         // column k is readable in the next step
     }
     float *U = u + (long long)b * u_stride;
     float *I = inv + (long long)b * inv_stride + (long long)lane * ldi;
@@ -164,8 +181,13 @@ extern "C" void qtensor_hip_solve_upper_right_batched(const float *q, const floa
     if (rows < 1) { set_error(kBadArgument, "solve_upper_right_batched: rows must be positive"); return; }
     hipStream_t stream = (hipStream_t)stream_v;
     const long long mat = (long long)n * n, tall = (long long)rows * n;
-    static const char *top_env = getenv("QT_SOLVE_PANEL");
-    const int top = top_env != nullptr ? atoi(top_env) : kSolvePanel;
+    // QT_SOLVE_PANEL (a tuning knob): another panel width, 64 times a power of two
+    static const int top = [] {
+        const char *env = getenv("QT_SOLVE_PANEL");
+        const int asked = env != nullptr ? atoi(env) : 0;
+        const bool usable = asked >= NB && asked % NB == 0 && ((asked / NB) & (asked / NB - 1)) == 0;
+        return usable ? asked : kSolvePanel;
+    }();
     // x holds the inverses of the 64 x 64 diagonal blocks; every level doubles the size of the inverted blocks
     for (int s = NB; s < n && s < top; s *= 2) {
         const int full = n / (2 * s), rem = n % (2 * s);
