@@ -208,6 +208,10 @@ void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
  *   out_j = (q_j - out_<j U_<j,j) x_jj.  work is scratch of batch * max(rows, n) * n floats (gram may
  *   be passed when rows <= n).  out must not alias q. */
 void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float *x, int *info, int n, int batch, qtensor_stream_t stream);
+/* The test that ends the rounds: out[2 b] = max |G_b - I|, out[2 b + 1] = ||G_b - I||_F^2 for the stack
+ * gram [batch, n, n], one pass, fixed summation order, NaN if G_b holds one.  partial: scratch of
+ * batch * 64 floats.  (No counterpart in the reference: Householder QR needs no such test.) */
+void qtensor_hip_gram_deviation_batched(const float *gram, float *partial, float *out, int n, int batch, qtensor_stream_t stream);
 void qtensor_hip_solve_upper_right_batched(const float *q, const float *u, float *x, float *work, float *out,
                                            int rows, int n, int batch, qtensor_stream_t stream);
 

@@ -109,6 +109,60 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
     if (!ok && lane == 0) info[b] = 1;
 }
 
+// How far a stack of Gram matrices is from the identity: per matrix max |G - I| and ||G - I||_F^2, in
+// one pass over the stack and in a fixed summation order (each block reduces a band of rows, a second
+// kernel adds the bands of a matrix in order).  A NaN anywhere gives NaN in both.
+constexpr int kBands = 32;
+
+__global__ __launch_bounds__(256) void deviation_bands_kernel(const float *gram, int n, int rows_per_band, float *partial) {
+    const int band = blockIdx.x, b = blockIdx.y;
+    const float *G = gram + (long long)b * n * n;
+    const int r0 = band * rows_per_band, r1 = min(r0 + rows_per_band, n);
+    const int quads = n / 4;                                     // n is a multiple of 64
+    uint32_t worst = 0;                                          // bits of the largest |e| (a NaN has the largest bits)
+    float sum = 0.0f;
+    for (int q = threadIdx.x; q < (r1 - r0) * quads; q += 256) {
+        const int r = r0 + q / quads, c = (q % quads) * 4;
+        const float4 g = *reinterpret_cast<const float4 *>(G + (long long)r * n + c);
+        const float e[4] = {g.x - (r == c ? 1.0f : 0.0f), g.y - (r == c + 1 ? 1.0f : 0.0f), g.z - (r == c + 2 ? 1.0f : 0.0f),
+                            g.w - (r == c + 3 ? 1.0f : 0.0f)};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            worst = max(worst, __float_as_uint(e[k]) & 0x7fffffffu);
+            sum = __builtin_fmaf(e[k], e[k], sum);
+        }
+    }
+    __shared__ uint32_t s_worst[256];
+    __shared__ float s_sum[256];
+    s_worst[threadIdx.x] = worst;
+    s_sum[threadIdx.x] = sum;
+    __syncthreads();
+    for (int step = 128; step >= 1; step >>= 1) {
+        if ((int)threadIdx.x < step) {
+            s_worst[threadIdx.x] = max(s_worst[threadIdx.x], s_worst[threadIdx.x + step]);
+            s_sum[threadIdx.x] += s_sum[threadIdx.x + step];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        partial[((long long)b * kBands + band) * 2] = __uint_as_float(s_worst[0]);
+        partial[((long long)b * kBands + band) * 2 + 1] = s_sum[0];
+    }
+}
+
+__global__ __launch_bounds__(64) void deviation_total_kernel(const float *partial, int bands, int batch, float *out) {
+    const int b = blockIdx.x * 64 + threadIdx.x;
+    if (b >= batch) return;
+    uint32_t worst = 0;
+    float sum = 0.0f;
+    for (int band = 0; band < bands; ++band) {
+        worst = max(worst, __float_as_uint(partial[((long long)b * kBands + band) * 2]));
+        sum += partial[((long long)b * kBands + band) * 2 + 1];
+    }
+    out[2 * b] = __uint_as_float(worst);
+    out[2 * b + 1] = sum;
+}
+
 qtensor_batch_ptr strided(const float *base, long long stride) {
     qtensor_batch_ptr p;
     p.base = base;
@@ -254,4 +308,17 @@ extern "C" void qtensor_hip_solve_upper_right_batched(const float *q, const floa
         t.args.triangular = 2;
         if (!run(t, stream)) return;
     }
+}
+
+extern "C" void qtensor_hip_gram_deviation_batched(const float *gram, float *partial, float *out, int n, int batch, void *stream_v) {
+    using namespace qt;
+    clear_error();
+    if (!stack_args_ok("gram_deviation_batched", n, batch, {gram, partial, out})) return;
+    hipStream_t stream = (hipStream_t)stream_v;
+    const int bands = n / 16 < kBands ? n / 16 : kBands;         // at least 16 rows per band
+    const int rows_per_band = (n + bands - 1) / bands;
+    hipLaunchKernelGGL(deviation_bands_kernel, dim3(bands, batch), dim3(256), 0, stream, gram, n, rows_per_band, partial);
+    if (!launch_ok("gram_deviation_batched (bands)")) return;
+    hipLaunchKernelGGL(deviation_total_kernel, dim3((batch + 63) / 64), dim3(64), 0, stream, partial, bands, batch, out);
+    launch_ok("gram_deviation_batched (totals)");
 }

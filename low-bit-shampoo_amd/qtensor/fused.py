@@ -317,6 +317,8 @@ if F.lib is not None:
     F.lib.qtensor_hip_cholesky_upper_batched.restype = None
     F.lib.qtensor_hip_cholesky_upper_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int,
                                                          ct.c_void_p]
+    F.lib.qtensor_hip_gram_deviation_batched.restype = None
+    F.lib.qtensor_hip_gram_deviation_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
     F.lib.qtensor_hip_solve_upper_right_batched.restype = None
     F.lib.qtensor_hip_solve_upper_right_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int,
                                                             ct.c_int, ct.c_int, ct.c_void_p]
@@ -337,6 +339,17 @@ def cholesky_upper(gram: Tensor, u: Tensor, x: Tensor, info: Tensor) -> None:
     if info.dtype != torch.int32 or info.numel() != B or not info.is_cuda:
         raise ValueError("info must be an int32 GPU vector with one entry per matrix")
     F._call(F.lib.qtensor_hip_cholesky_upper_batched, gram.device, gram.data_ptr(), u.data_ptr(), x.data_ptr(), info.data_ptr(), n, B)
+
+
+def gram_deviation(gram: Tensor) -> Tensor:
+    """[B, 2]: max |G - I| and ||G - I||_F^2 of every matrix of the stack gram [B, n, n] (n a multiple of
+    64), in one pass and a fixed summation order."""
+    B, n, _ = gram.shape
+    _stack(gram, "gram", (B, n, n))
+    out = torch.empty(B, 2, device=gram.device)
+    partial = torch.empty(B, 64, device=gram.device)
+    F._call(F.lib.qtensor_hip_gram_deviation_batched, gram.device, gram.data_ptr(), partial.data_ptr(), out.data_ptr(), n, B)
+    return out
 
 
 def solve_upper_right(q: Tensor, u: Tensor, x: Tensor, work: Tensor, out: Tensor) -> Tensor:
@@ -415,9 +428,9 @@ class CholeskyQR:
 
     def check(self):
         self.gram = gemm(self.Q, self.Q, trans_a=True, symmetric=True)
-        self.gram.diagonal(dim1=1, dim2=2).sub_(1.0)
-        done = self.gram.abs().amax(dim=(1, 2)) < self.tolerance                # False for NaN as well
-        near = torch.linalg.matrix_norm(self.gram) < 0.5
+        far = gram_deviation(self.gram)                                         # max |G - I|, ||G - I||_F^2
+        done = far[:, 0] < self.tolerance                                       # False for NaN as well
+        near = far[:, 1] < 0.25
         self.flags = torch.stack([done, near, self.fatal])
 
     def poll(self):
@@ -443,7 +456,7 @@ class CholeskyQR:
         # round, and a matrix for which it fails (non-positive pivot) simply keeps its Q and joins the
         # shifted rounds.
         shifted = ~near & (self.needs_shift if self.rounds == 0 else torch.ones_like(near))
-        self.gram.diagonal(dim1=1, dim2=2).add_(1.0 + self.shift * shifted.to(self.gram.dtype).unsqueeze(1))
+        self.gram.diagonal(dim1=1, dim2=2).add_(self.shift * shifted.to(self.gram.dtype).unsqueeze(1))
         info = self.info[:k]
         info.zero_()
         cholesky_upper(self.gram, self.U[:k], self.X[:k], info)

@@ -74,6 +74,22 @@ def test_blocked_cholesky_and_right_solve_against_float64(mods, n, batch, rows):
                          torch.zeros(1, 100, 100, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda"))
 
 
+@pytest.mark.parametrize("n,batch", [(64, 5), (320, 3), (1024, 2)])
+def test_distance_of_gram_matrices_from_the_identity_in_one_pass(mods, n, batch):
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(n)
+    G = torch.eye(n) + 0.01 * torch.randn(batch, n, n, generator=g)
+    G[0, 3, n - 1] = -0.75                                     # the largest deviation is negative and off the diagonal
+    out = X.gram_deviation(G.cuda()).cpu()
+    E = G.double() - torch.eye(n, dtype=torch.float64)
+    assert torch.allclose(out[:, 0].double(), E.abs().amax(dim=(1, 2)), rtol=1e-6, atol=0)
+    assert torch.allclose(out[:, 1].double(), (E * E).sum(dim=(1, 2)), rtol=1e-5, atol=0)
+    assert torch.equal(out, X.gram_deviation(G.cuda()).cpu())                  # fixed summation order
+    G[batch - 1, 7, 9] = float("nan")
+    out = X.gram_deviation(G.cuda()).cpu()
+    assert bool(out[batch - 1].isnan().all()) and not bool(out[:batch - 1].isnan().any())
+
+
 def test_cholesky_qr_gives_the_householder_factor_up_to_signs(mods):
     _, E2 = mods
     g = torch.Generator().manual_seed(3)
