@@ -212,6 +212,10 @@ void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float *x, int *in
  * gram [batch, n, n], one pass, fixed summation order, NaN if G_b holds one.  partial: scratch of
  * batch * 64 floats.  (No counterpart in the reference: Householder QR needs no such test.) */
 void qtensor_hip_gram_deviation_batched(const float *gram, float *partial, float *out, int n, int batch, qtensor_stream_t stream);
+/* dst[b] = src[b] (n x n fp32 each) for every b with flags[b] != 0; the other matrices of dst are left
+ * alone.  Puts the previous iterate back where a factorisation failed, without a pass over the whole
+ * stack and without the host knowing which ones failed.  (No counterpart in the reference.) */
+void qtensor_hip_copy_flagged_batched(float *dst, const float *src, const int *flags, int n, int batch, qtensor_stream_t stream);
 void qtensor_hip_solve_upper_right_batched(const float *q, const float *u, float *x, float *work, float *out,
                                            int rows, int n, int batch, qtensor_stream_t stream);
 

@@ -163,6 +163,15 @@ __global__ __launch_bounds__(64) void deviation_total_kernel(const float *partia
     out[2 * b + 1] = sum;
 }
 
+// dst[b] = src[b] for the matrices whose flag is set; the blocks of all others leave at once.
+__global__ __launch_bounds__(256) void copy_flagged_kernel(float *dst, const float *src, const int *flags, long long quads) {
+    const int b = blockIdx.y;
+    if (flags[b] == 0) return;
+    const float4 *s = reinterpret_cast<const float4 *>(src) + (long long)b * quads;
+    float4 *d = reinterpret_cast<float4 *>(dst) + (long long)b * quads;
+    for (long long q = blockIdx.x * 256ll + threadIdx.x; q < quads; q += (long long)gridDim.x * 256) d[q] = s[q];
+}
+
 qtensor_batch_ptr strided(const float *base, long long stride) {
     qtensor_batch_ptr p;
     p.base = base;
@@ -321,4 +330,13 @@ extern "C" void qtensor_hip_gram_deviation_batched(const float *gram, float *par
     if (!launch_ok("gram_deviation_batched (bands)")) return;
     hipLaunchKernelGGL(deviation_total_kernel, dim3((batch + 63) / 64), dim3(64), 0, stream, partial, bands, batch, out);
     launch_ok("gram_deviation_batched (totals)");
+}
+
+extern "C" void qtensor_hip_copy_flagged_batched(float *dst, const float *src, const int *flags, int n, int batch, void *stream_v) {
+    using namespace qt;
+    clear_error();
+    if (!stack_args_ok("copy_flagged_batched", n, batch, {dst, src, flags})) return;
+    const long long quads = (long long)n * n / 4;
+    hipLaunchKernelGGL(copy_flagged_kernel, dim3(64, batch), dim3(256), 0, (hipStream_t)stream_v, dst, src, flags, quads);
+    launch_ok("copy_flagged_batched");
 }

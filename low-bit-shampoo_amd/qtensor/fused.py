@@ -319,6 +319,8 @@ if F.lib is not None:
                                                          ct.c_void_p]
     F.lib.qtensor_hip_gram_deviation_batched.restype = None
     F.lib.qtensor_hip_gram_deviation_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
+    F.lib.qtensor_hip_copy_flagged_batched.restype = None
+    F.lib.qtensor_hip_copy_flagged_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
     F.lib.qtensor_hip_solve_upper_right_batched.restype = None
     F.lib.qtensor_hip_solve_upper_right_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int,
                                                             ct.c_int, ct.c_int, ct.c_void_p]
@@ -350,6 +352,16 @@ def gram_deviation(gram: Tensor) -> Tensor:
     partial = torch.empty(B, 64, device=gram.device)
     F._call(F.lib.qtensor_hip_gram_deviation_batched, gram.device, gram.data_ptr(), partial.data_ptr(), out.data_ptr(), n, B)
     return out
+
+
+def copy_flagged(dst: Tensor, src: Tensor, flags: Tensor) -> Tensor:
+    """dst[b] = src[b] for the matrices of the stacks [B, n, n] with flags[b] != 0 (int32 [B])."""
+    B, n, _ = dst.shape
+    _stack(dst, "dst", (B, n, n)), _stack(src, "src", (B, n, n))
+    if flags.dtype != torch.int32 or flags.numel() != B or not flags.is_cuda:
+        raise ValueError("flags must be an int32 GPU vector with one entry per matrix")
+    F._call(F.lib.qtensor_hip_copy_flagged_batched, dst.device, dst.data_ptr(), src.data_ptr(), flags.data_ptr(), n, B)
+    return dst
 
 
 def solve_upper_right(q: Tensor, u: Tensor, x: Tensor, work: Tensor, out: Tensor) -> Tensor:
@@ -465,7 +477,7 @@ class CholeskyQR:
         bad = info != 0
         self.fatal = self.fatal | (bad & (shifted | near))
         self.needs_shift = self.needs_shift | bad
-        self.Q, self.gram = torch.where(bad.view(k, 1, 1), self.Q, out), None
+        self.Q, self.gram = copy_flagged(out, self.Q, info), None              # a failed matrix keeps its iterate
         self.rounds_left -= 1
         self.rounds += 1
         if bool(self.near.any()):

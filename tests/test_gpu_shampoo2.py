@@ -90,6 +90,16 @@ def test_distance_of_gram_matrices_from_the_identity_in_one_pass(mods, n, batch)
     assert bool(out[batch - 1].isnan().all()) and not bool(out[:batch - 1].isnan().any())
 
 
+def test_flagged_matrices_are_put_back_and_only_those(mods):
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(5)
+    src, dst = torch.randn(5, 128, 128, generator=g).cuda(), torch.randn(5, 128, 128, generator=g).cuda()
+    before = dst.clone()
+    flags = torch.tensor([0, 1, 0, 0, 7], dtype=torch.int32, device="cuda")
+    X.copy_flagged(dst, src, flags)
+    assert torch.equal(dst[[1, 4]], src[[1, 4]]) and torch.equal(dst[[0, 2, 3]], before[[0, 2, 3]])
+
+
 def test_cholesky_qr_gives_the_householder_factor_up_to_signs(mods):
     _, E2 = mods
     g = torch.Generator().manual_seed(3)
