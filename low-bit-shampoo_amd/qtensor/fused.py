@@ -8,6 +8,7 @@ tensors only and launches libqtensor_hip.so's qtensor_hip_gemm on torch's curren
 import ctypes as ct
 from typing import Optional, Sequence
 
+import numpy as np
 import torch
 from torch import Tensor
 
@@ -414,89 +415,119 @@ class CholeskyQR:
         self.Y, self.shift, self.tolerance, self.rounds_left = Y, shift, tolerance, max_rounds
         scale = torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)
         self.Q = (Y / scale).contiguous()             # working set; unit columns: the Gram matrix has a unit diagonal
-        self.ids = torch.arange(B, device=Y.device)   # which matrix of the stack each working-set entry is
         self.U = torch.empty_like(self.Q)
         self.X = torch.zeros_like(self.Q)             # inverse factors; the part below the diagonal blocks stays zero
         self.info = torch.zeros(B, dtype=torch.int32, device=Y.device)
-        self.final = torch.empty_like(self.Q)
+        self.final = None                             # allocated when the first matrix is done
         self.redo = []                                # matrices handed to the library at the end
         self.finished = False
         self.rounds = 0                               # factorisation rounds enqueued so far
-        self.gram = self.flags = self.near = None
-        # per working-set entry: a factorisation WITH the shift hit a non-positive pivot (hopeless: the
-        # library takes over) / one WITHOUT it did (the entry keeps its Q and gets the shift from now on)
-        self.fatal = torch.zeros(B, dtype=torch.bool, device=Y.device)
-        self.needs_shift = torch.zeros(B, dtype=torch.bool, device=Y.device)
+        self.gram = self.far = None
+        # The bookkeeping lives on the host (it waits once per round anyway), per working-set entry:
+        # which matrix of the stack it is, whether it is within ||G - I||_F < 0.5, and whether a factorisation
+        # WITHOUT the shift hit a non-positive pivot (it kept its Q and gets the shift from now on).
+        self.ids = np.arange(B)
+        self.near = np.zeros(B, dtype=bool)
+        self.needs_shift = np.zeros(B, dtype=bool)
+        self.last = None                              # (pivot flags, shifted, near, ids) of the round not yet looked at
+
+    def _index(self, positions):
+        return torch.as_tensor(np.ascontiguousarray(positions), dtype=torch.int64).to(self.Q.device)
+
+    def _finish(self, where, source):
+        """The working-set entries `where` (host positions) of `source` are final."""
+        if where.size == 0:
+            return
+        B = self.Y.shape[0]
+        if self.final is None and where.size == B and source.shape[0] == B and np.array_equal(self.ids, np.arange(B)):
+            self.final = source                       # the whole stack at once: no copy
+            return
+        if self.final is None:
+            self.final = torch.empty_like(self.Y)
+        self.final.index_copy_(0, self._index(self.ids[where]), source.index_select(0, self._index(where)))
 
     def _keep(self, keep):
         """Shrink the working set to the entries of the host mask `keep`."""
-        if bool(keep.all()):
+        if keep.all():
             return
-        index = torch.nonzero(keep).flatten().to(self.Q.device)
-        self.Q, self.ids = self.Q[index], self.ids[index]
-        self.fatal, self.needs_shift = self.fatal[index], self.needs_shift[index]
+        index = self._index(np.nonzero(keep)[0])
+        self.Q = self.Q.index_select(0, index)
         if self.gram is not None:
-            self.gram = self.gram[index]
+            self.gram = self.gram.index_select(0, index)
+        self.ids, self.near, self.needs_shift = self.ids[keep], self.near[keep], self.needs_shift[keep]
 
     def check(self):
         self.gram = gemm(self.Q, self.Q, trans_a=True, symmetric=True)
-        far = gram_deviation(self.gram)                                         # max |G - I|, ||G - I||_F^2
-        done = far[:, 0] < self.tolerance                                       # False for NaN as well
-        near = far[:, 1] < 0.25
-        self.flags = torch.stack([done, near, self.fatal])
+        self.far = gram_deviation(self.gram)                                    # max |G - I|, ||G - I||_F^2
 
     def poll(self):
-        done, near, failed = self.flags.cpu()                                   # the host synchronisation
+        far = self.far.cpu().numpy()                                            # the host synchronisation
+        k = self.ids.size
+        failed = np.zeros(k, dtype=bool)
+        if self.last is not None:
+            # pivot flags of the previous round: a failure with the shift (or of a matrix that was already close:
+            # it has been finalised, wrongly) is hopeless and goes to the library; one without the shift keeps its Q
+            info, shifted, near, ids = self.last
+            bad = info.cpu().numpy()[:shifted.size] != 0
+            self.redo += ids[bad & near].tolist()
+            bad, shifted = bad[~near], shifted[~near]                           # the entries still in the working set
+            failed |= bad & shifted
+            self.needs_shift |= bad
+            self.last = None
+        with np.errstate(invalid="ignore"):
+            done = far[:, 0] < self.tolerance                                   # False for NaN as well
+            self.near = far[:, 1] < 0.25
         if self.rounds_left == 0:
-            failed = failed | ~done
-        done = done & ~failed
-        if bool(failed.any()):
-            self.redo += self.ids[failed.to(self.Q.device)].tolist()
-        if bool(done.any()):
-            sel = done.to(self.Q.device)
-            self.final[self.ids[sel]] = self.Q[sel]
-        keep = ~(done | failed)
-        self.near = near[keep]
-        self._keep(keep)
-        self.finished = self.Q.shape[0] == 0
+            failed |= ~done
+        done &= ~failed
+        self.redo += self.ids[failed].tolist()
+        self._finish(np.nonzero(done)[0], self.Q)
+        self._keep(~(done | failed))
+        self.finished = self.ids.size == 0
         return self.finished
 
     def advance(self):
-        k = self.Q.shape[0]
-        near = self.near.to(self.Q.device)
+        k = self.ids.size
         # The first round is tried without the shift: for condition numbers up to about 1e3 that saves a
         # round, and a matrix for which it fails (non-positive pivot) simply keeps its Q and joins the
         # shifted rounds.
-        shifted = ~near & (self.needs_shift if self.rounds == 0 else torch.ones_like(near))
-        self.gram.diagonal(dim1=1, dim2=2).add_(self.shift * shifted.to(self.gram.dtype).unsqueeze(1))
+        shifted = ~self.near & (self.needs_shift if self.rounds == 0 else True)
+        if shifted.any():
+            add = torch.as_tensor(np.where(shifted, self.shift, 0.0).astype(np.float32)).to(self.Q.device)
+            self.gram.diagonal(dim1=1, dim2=2).add_(add.unsqueeze(1))
         info = self.info[:k]
         info.zero_()
         cholesky_upper(self.gram, self.U[:k], self.X[:k], info)
         out = torch.empty_like(self.Q)
         solve_upper_right(self.Q, self.U[:k], self.X[:k], self.gram, out)      # the Gram matrix is used up: scratch
-        bad = info != 0
-        self.fatal = self.fatal | (bad & (shifted | near))
-        self.needs_shift = self.needs_shift | bad
-        self.Q, self.gram = copy_flagged(out, self.Q, info), None              # a failed matrix keeps its iterate
+        copy_flagged(out, self.Q, info)                                         # a failed matrix keeps its iterate
+        self.Q, self.gram = out, None
+        self.last = (info, shifted, self.near.copy(), self.ids.copy())
         self.rounds_left -= 1
         self.rounds += 1
-        if bool(self.near.any()):
+        if self.near.any():
             # ||G - I||_F < 0.5 before an unshifted round: G was positive definite with eigenvalues in
-            # (0.5, 1.5), the round cannot fail and leaves Q orthonormal to rounding
-            self.final[self.ids[near]] = self.Q[near]
+            # (0.5, 1.5), the round leaves Q orthonormal to rounding
+            self._finish(np.nonzero(self.near)[0], self.Q)
             self._keep(~self.near)
-            self.finished = self.Q.shape[0] == 0
+            self.finished = self.ids.size == 0
 
     def result(self):
+        if self.last is not None:                     # pivot flags of the last round
+            info, shifted, near, ids = self.last
+            self.redo += ids[(info.cpu().numpy()[:shifted.size] != 0) & near].tolist()
+            self.last = None
+        if self.final is None:
+            self.final = torch.empty_like(self.Y)
         if self.redo:
-            redo = torch.tensor(self.redo, device=self.Y.device)
+            redo = torch.tensor(sorted(set(self.redo)), device=self.Y.device)
             torch.cuda.synchronize()              # the library routine is not trusted to be stream-ordered here
             self.final[redo] = _householder_qr(self.Y[redo])[0]
             torch.cuda.synchronize()
         Q = self.final
         if Q.shape[1] != self.true_n:
             Q = Q[:, :self.true_n, :self.true_n].contiguous()
-        return Q, len(self.redo)
+        return Q, len(set(self.redo))
 
 
 def cholesky_qr(Y, max_rounds=12, shift=2e-4, tolerance=2e-5):
