@@ -146,7 +146,12 @@ typedef struct {
 
 enum { QTENSOR_DENSE = 0, QTENSOR_DENSE_T = 1, QTENSOR_QUANT4 = 2, QTENSOR_QUANT8 = 3 };
 enum { QTENSOR_EPI_STORE = 0, QTENSOR_EPI_AXPBY_DENSE = 1, QTENSOR_EPI_AXPBY_QUANT4 = 2,
-       QTENSOR_EPI_AXPBY_QUANT8 = 3, QTENSOR_EPI_NEWTON = 4 };
+       QTENSOR_EPI_AXPBY_QUANT8 = 3, QTENSOR_EPI_NEWTON = 4,
+       /* beta * deq(Eq) + alpha * (A B) re-encoded IN PLACE into Eq's codes, maxima and exact diagonal (C is
+        * not used): the statistics update L <- beta L + (1 - beta) G G^T of optimizers/shampoo1.py:164-178
+        * (dequantize, update, quantize) in one launch.  Blocksize 64; bit-identical to AXPBY_QUANT* followed
+        * by the stack quantizer. */
+       QTENSOR_EPI_REQUANT4 = 5, QTENSOR_EPI_REQUANT8 = 6 };
 
 typedef struct {
     int M, N, K, batch;
@@ -186,7 +191,8 @@ typedef struct {
 } qtensor_gemm_desc;
 
 /* Combinations built: (QUANT*, DENSE, STORE), (DENSE, QUANT*, STORE), (DENSE, DENSE_T, STORE|AXPBY_*),
- * (DENSE_T, DENSE, STORE|AXPBY_*), (DENSE, DENSE, STORE|AXPBY_DENSE|NEWTON); anything else is an error. */
+ * (DENSE_T, DENSE, STORE|AXPBY_*), (DENSE, DENSE, STORE|AXPBY_DENSE|NEWTON), and REQUANT* with
+ * (DENSE, DENSE_T) or (DENSE_T, DENSE); anything else is an error. */
 void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
 
 /* ---- batched Cholesky factorisation and triangular solve (Cholesky QR) ---------------------------

@@ -20,6 +20,7 @@
 // consecutive words per step.  Global loads run two tiles ahead of the MFMAs; the LDS commit sits
 // in the middle of the MFMA stream.
 #include "qt_common.h"
+#include "qt_tables.h"
 
 #include <cmath>
 #include <cstdio>
@@ -29,7 +30,7 @@
 namespace qt {
 
 enum OperandKind : int { kDense = 0, kDenseT = 1, kQuant4 = 2, kQuant8 = 3 };
-enum EpilogueKind : int { kStore = 0, kAxpbyDense = 1, kAxpbyQuant4 = 2, kAxpbyQuant8 = 3, kNewton = 4 };
+enum EpilogueKind : int { kStore = 0, kAxpbyDense = 1, kAxpbyQuant4 = 2, kAxpbyQuant8 = 3, kNewton = 4, kRequant4 = 5, kRequant8 = 6 };
 
 // One matrix argument over the batch: either base + b * stride, or list[b] when list != nullptr.
 struct BatchPtr {
@@ -411,14 +412,20 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     constexpr int SIZE_A = A_RM ? BM * LDK : BK * LDA, SIZE_B = B_RM ? BN * LDK : BK * LDB;
     // one buffer: the two stages of both operand tiles during the main loop, then (symmetric products)
     // a 32 x 32 staging square per wave that turns accumulator blocks around for the mirrored stores
-    constexpr int STAGE_LD = 36, SIZE_STAGE = 4 * 32 * STAGE_LD, SIZE_MAIN = 2 * SIZE_A + 2 * SIZE_B;
+    constexpr bool kRequant = EPI == kRequant4 || EPI == kRequant8;
+    constexpr int STAGE_LD = 36, REQUANT_LD = 68, SIZE_MAIN = 2 * SIZE_A + 2 * SIZE_B;
+    constexpr int SIZE_STAGE = kRequant ? 4 * 32 * REQUANT_LD : 4 * 32 * STAGE_LD;
     __shared__ __attribute__((aligned(16))) float s_mem[SIZE_MAIN > SIZE_STAGE ? SIZE_MAIN : SIZE_STAGE];
     float (*s_a)[SIZE_A] = reinterpret_cast<float (*)[SIZE_A]>(s_mem);
     float (*s_b)[SIZE_B] = reinterpret_cast<float (*)[SIZE_B]>(s_mem + 2 * SIZE_A);
     __shared__ float s_code[256];
-    constexpr bool kNeedCode = KA >= kQuant4 || KB >= kQuant4 || EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8;
+    constexpr bool kNeedCode = KA >= kQuant4 || KB >= kQuant4 || EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8 || kRequant;
+    // a requantizing epilogue searches the table like the quantizer does: thresholds per workgroup
+    constexpr int RCODE = EPI == kRequant8 ? 256 : 16;
+    __shared__ CodeTables<kRequant ? RCODE : 1> tab;
+    if constexpr (kRequant) build_code_tables<RCODE>(args.code, tab, nullptr);
     if (kNeedCode) {
-        constexpr int NCODE = (KA == kQuant8 || KB == kQuant8 || EPI == kAxpbyQuant8) ? 256 : 16;
+        constexpr int NCODE = (KA == kQuant8 || KB == kQuant8 || EPI == kAxpbyQuant8 || EPI == kRequant8) ? 256 : 16;
         if ((int)threadIdx.x < NCODE) s_code[threadIdx.x] = args.code[threadIdx.x];
         __syncthreads();
     }
@@ -551,8 +558,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
     }
     float *T = EPI == kNewton ? const_cast<float *>(batch_ptr<float>(args.T, b)) : nullptr;
     const float *E = EPI == kAxpbyDense ? dense_ptr(args.E, b, args.batch_inner, args.inner_e) : nullptr;
-    constexpr bool kQuantAddend = EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8;
-    constexpr int EBITS = EPI == kAxpbyQuant8 ? 8 : 4;
+    constexpr bool kQuantAddend = EPI == kAxpbyQuant4 || EPI == kAxpbyQuant8 || kRequant;
+    constexpr int EBITS = (EPI == kAxpbyQuant8 || EPI == kRequant8) ? 8 : 4;
     const uint8_t *e_codes = kQuantAddend ? batch_ptr<uint8_t>(args.Eq.codes, b) : nullptr;
     const float *e_absmax = kQuantAddend ? batch_ptr<float>(args.Eq.absmax, b) : nullptr;
     const float *e_diag = kQuantAddend && has_ptr(args.Eq.diag) ? batch_ptr<float>(args.Eq.diag, b) : nullptr;
@@ -564,6 +571,78 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
                         (EPI != kAxpbyDense || ((args.lde & 3) == 0 && is_aligned16(E)));
     const bool mirror_vec = vec_ok && (args.M & 3) == 0;
     const bool direct_vec = vec_ok && (args.N & 3) == 0;
+    if constexpr (kRequant) {
+        // beta * deq(E) + alpha * acc goes straight back into E's codes, maxima and exact diagonal: the fp32
+        // statistic never reaches memory.  A wave's 64 x 64 quadrant holds whole segments (blocksize 64) of 64
+        // rows -- and, mirrored, of 64 rows of the transposed tile -- so it encodes them alone: 32 rows at a
+        // time go through its staging area, 16 lanes take one row (four consecutive elements each), and the
+        // maximum, the division and the table search are those of the flat quantizer.  Each element of E is
+        // read and rewritten by the same wave, all reads of a row before its writes.
+        float *stage = s_mem + wave * (32 * REQUANT_LD);
+        uint8_t *o_codes = const_cast<uint8_t *>(e_codes);
+        float *o_absmax = const_cast<float *>(e_absmax), *o_diag = const_cast<float *>(e_diag);
+        const bool fast_ok = (tab.flags & kFlagLut) != 0, ascending = (tab.flags & kFlagAscending) != 0;
+        const int order = args.Eq.order, per_row = order >> 6;
+        auto encode_rows = [&](int row_base, int col_base) {
+            if (col_base >= order) return;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int rl = q * 4 + (lane >> 4), c4 = (lane & 15) * 4;
+                const float4 a4 = *reinterpret_cast<const float4 *>(stage + rl * REQUANT_LD + c4);
+                const float a[4] = {a4.x, a4.y, a4.z, a4.w};
+                const int row = row_base + rl, col = col_base + c4;
+                if (row >= order) continue;                      // the 16 lanes of a segment share the row
+                float e[4], y[4];
+                dequant_four<EBITS>(e_codes, e_absmax, s_code, order, 6, row, col, e);
+                const bool on_diag = o_diag != nullptr && (unsigned)(row - col) < 4u;
+                if (on_diag) {
+                    const float d = gload(o_diag + row);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) if (row == col + k) e[k] = d;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) y[k] = __builtin_fmaf(args.alpha, a[k], args.beta * e[k]);
+                if (on_diag) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        if (row == col + k) { gstore(o_diag + row, y[k]); y[k] = 0.0f; }
+                }
+                uint32_t idx[4];
+                const uint32_t m = encode_four<RCODE, 16>(y, tab, fast_ok, ascending, idx);
+                if ((lane & 15) == 0) gstore(o_absmax + (long long)row * per_row + (col >> 6), __uint_as_float(m));
+                const long long k0 = (long long)row * order + col;
+                if (EBITS == 4)
+                    *(QT_GLOBAL uint16_t *)(o_codes + (k0 >> 1)) = (uint16_t)(((idx[0] << 4) | idx[1]) | (((idx[2] << 4) | idx[3]) << 8));
+                else
+                    *(QT_GLOBAL uint32_t *)(o_codes + k0) = idx[0] | (idx[1] << 8) | (idx[2] << 16) | (idx[3] << 24);
+            }
+        };
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    stage[(8 * (r / 4) + 4 * (lane >> 5) + r % 4) * REQUANT_LD + j * 32 + (lane & 31)] = acc[i][j][r];
+            wave_lds_sync();
+            encode_rows(m0 + wm + i * 32, n0 + wn);
+            wave_lds_sync();
+        }
+        if (mirror) {
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        stage[(lane & 31) * REQUANT_LD + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + r % 4] = acc[i][j][r];
+                wave_lds_sync();
+                encode_rows(n0 + wn + j * 32, m0 + wm);
+                wave_lds_sync();
+            }
+        }
+        return;
+    }
     float local_err = 0.0f;
     // Each wave passes its accumulator blocks (32 x 32) through a staging square of its own in LDS, so that a
     // lane ends up with four consecutive elements of one output row: 16-byte stores, eight lanes per 128-byte
@@ -778,11 +857,12 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
         return;
     }
     const int ka = d->kind_a, kb = d->kind_b, ep = d->epilogue;
-    if (ka < kDense || ka > kQuant8 || kb < kDense || kb > kQuant8 || ep < kStore || ep > kNewton) {
+    if (ka < kDense || ka > kQuant8 || kb < kDense || kb > kQuant8 || ep < kStore || ep > kRequant8) {
         set_error(kBadArgument, "gemm: unknown operand or epilogue kind (%d, %d, %d)", ka, kb, ep);
         return;
     }
-    if (!has_host_ptr(a.C) || a.ldc < d->N) { set_error(kBadArgument, "gemm: bad C (ldc %d < N %d or null)", a.ldc, d->N); return; }
+    const bool requant = ep == kRequant4 || ep == kRequant8;        // no dense result: the addend is re-encoded in place
+    if (!requant && (!has_host_ptr(a.C) || a.ldc < d->N)) { set_error(kBadArgument, "gemm: bad C (ldc %d < N %d or null)", a.ldc, d->N); return; }
     if (ka < kQuant4) {
         const int need = ka == kDense ? d->K : d->M;
         if (!has_host_ptr(a.A) || a.lda < need) { set_error(kBadArgument, "gemm: bad A (lda %d < %d or null)", a.lda, need); return; }
@@ -798,9 +878,10 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
         if (a.Bq.order != d->N || d->K != d->N) { set_error(kBadArgument, "gemm: quantized B must be square with K == N == order"); return; }
     }
     if (ep == kAxpbyDense && (!has_host_ptr(a.E) || a.lde < d->N)) { set_error(kBadArgument, "gemm: bad dense addend"); return; }
-    if (ep == kAxpbyQuant4 || ep == kAxpbyQuant8) {
-        if (!valid_quant(a.Eq, ep == kAxpbyQuant4 ? 4 : 8, "addend")) return;
+    if (ep == kAxpbyQuant4 || ep == kAxpbyQuant8 || requant) {
+        if (!valid_quant(a.Eq, ep == kAxpbyQuant4 || ep == kRequant4 ? 4 : 8, "addend")) return;
         if (a.Eq.order != d->M || d->M != d->N) { set_error(kBadArgument, "gemm: quantized addend must be M x N square of its order"); return; }
+        if (requant && a.Eq.bs_shift != 6) { set_error(kBadArgument, "gemm: the requantizing epilogue needs blocksize 64"); return; }
     }
     if (ep == kNewton && (!has_host_ptr(a.T) || a.ldt < d->N || !a.err)) { set_error(kBadArgument, "gemm: Newton epilogue needs T and err"); return; }
     a.symmetric = a.symmetric != 0;
@@ -813,7 +894,7 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
         set_error(kBadArgument, "gemm: symmetric products need M == N and dense operands");
         return;
     }
-    const bool need_code = ka >= kQuant4 || kb >= kQuant4 || ep == kAxpbyQuant4 || ep == kAxpbyQuant8;
+    const bool need_code = ka >= kQuant4 || kb >= kQuant4 || ep == kAxpbyQuant4 || ep == kAxpbyQuant8 || requant;
     if (need_code && !a.code) { set_error(kNullPointer, "gemm: code table missing"); return; }
 
     // Tile shape: the one with the smallest estimated makespan.  Workgroups that share a compute unit
@@ -845,6 +926,7 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
         }
     }
     if (a.symmetric && shapes[pick].bm != shapes[pick].bn) pick = 0;
+    if (requant) pick = 0;          // a wave's quadrant must hold whole 64-element segments
     // Few tiles and a long k range: cut k into equal slices (whole k tiles each) that write partial products
     // to the caller's workspace and are summed in order afterwards.  Same cost model, with a fixed cost per
     // workgroup (prologue, epilogue, the extra pass over the output) worth about 64 k steps.
@@ -887,6 +969,10 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
         QT_GEMM_CASE(kDense, kDenseT, kAxpbyDense)
         QT_GEMM_CASE(kDense, kDenseT, kAxpbyQuant4)
         QT_GEMM_CASE(kDense, kDenseT, kAxpbyQuant8)
+        case kDense * 100 + kDenseT * 10 + kRequant4: launch_gemm<128, 128, kDense, kDenseT, kRequant4>(a, d->batch, stream); break;
+        case kDense * 100 + kDenseT * 10 + kRequant8: launch_gemm<128, 128, kDense, kDenseT, kRequant8>(a, d->batch, stream); break;
+        case kDenseT * 100 + kDense * 10 + kRequant4: launch_gemm<128, 128, kDenseT, kDense, kRequant4>(a, d->batch, stream); break;
+        case kDenseT * 100 + kDense * 10 + kRequant8: launch_gemm<128, 128, kDenseT, kDense, kRequant8>(a, d->batch, stream); break;
         QT_GEMM_CASE(kDenseT, kDense, kStore)
         QT_GEMM_CASE(kDenseT, kDense, kAxpbyDense)
         QT_GEMM_CASE(kDenseT, kDense, kAxpbyQuant4)

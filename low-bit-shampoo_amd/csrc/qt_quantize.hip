@@ -47,34 +47,6 @@ template <> struct ElementLoader<uint16_t> {
     static __device__ __forceinline__ float load1(const uint16_t *base, size_t k) { return bf16_bits_to_float(base[k]); }
 };
 
-__device__ __forceinline__ uint32_t abs_bits(float x) { return __float_as_uint(x) & 0x7fffffffu; }
-
-// Index by the exact route: IEEE division, then the threshold count.  amax_bits == 0 -> 0.
-template <int NCODE>
-__device__ __forceinline__ uint32_t exact_index(float x, uint32_t amax_bits, const CodeTables<NCODE> &t) {
-    if (amax_bits == 0u) return 0u;
-    const float q = x / __uint_as_float(amax_bits);
-    return t.perm[count_thresholds<NCODE>(q, t.thr)];
-}
-
-// Bucket of a quotient known to satisfy |q| <= 1 (no upper clamp needed).
-__device__ __forceinline__ int lut_bucket_unit(float q) {
-    const uint32_t b = __float_as_uint(q);
-    int fb = (int)((b & 0x7fffffffu) >> kLutShift) - kLutBias;
-    fb = max(fb, 0);
-    return kLutPerSign + (fb ^ ((int)b >> 31));
-}
-
-template <int NCODE, bool USE_LUT>
-__device__ __forceinline__ uint32_t fast_index(float x, float a, float r, const CodeTables<NCODE> &t, const uint2 *lut) {
-    const float q = quotient(x, a, r);
-    if (USE_LUT) {
-        const uint2 e = lut[lut_bucket_unit(q)];
-        return e.y + (uint32_t)!(q < __uint_as_float(e.x));
-    }
-    return (uint32_t)count_thresholds<NCODE>(q, t.thr);
-}
-
 // Per-wave staging area: packed codes of one step in element order, and its segment maxima.
 template <int BITS>
 struct WaveStage {

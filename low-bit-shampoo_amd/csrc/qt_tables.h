@@ -12,6 +12,7 @@
 #pragma once
 
 #include "qt_common.h"
+#include "qt_divide.h"
 
 namespace qt {
 
@@ -119,6 +120,59 @@ __device__ void build_code_tables(const float *__restrict__ code, CodeTables<NCO
         }
         __syncthreads();
     }
+}
+
+// ---- from one value to its table index -------------------------------------------------------
+__device__ __forceinline__ uint32_t abs_bits(float x) { return __float_as_uint(x) & 0x7fffffffu; }
+
+// Index by the exact route: IEEE division, then the threshold count.  amax_bits == 0 -> 0.
+template <int NCODE>
+__device__ __forceinline__ uint32_t exact_index(float x, uint32_t amax_bits, const CodeTables<NCODE> &t) {
+    if (amax_bits == 0u) return 0u;
+    const float q = x / __uint_as_float(amax_bits);
+    return t.perm[count_thresholds<NCODE>(q, t.thr)];
+}
+
+// Bucket of a quotient known to satisfy |q| <= 1 (no upper clamp needed).
+__device__ __forceinline__ int lut_bucket_unit(float q) {
+    const uint32_t b = __float_as_uint(q);
+    int fb = (int)((b & 0x7fffffffu) >> kLutShift) - kLutBias;
+    fb = max(fb, 0);
+    return kLutPerSign + (fb ^ ((int)b >> 31));
+}
+
+template <int NCODE, bool USE_LUT>
+__device__ __forceinline__ uint32_t fast_index(float x, float a, float r, const CodeTables<NCODE> &t, const uint2 *lut) {
+    const float q = quotient(x, a, r);
+    if (USE_LUT) {
+        const uint2 e = lut[lut_bucket_unit(q)];
+        return e.y + (uint32_t)!(q < __uint_as_float(e.x));
+    }
+    return (uint32_t)count_thresholds<NCODE>(q, t.thr);
+}
+
+// Four consecutive elements per lane, G lanes per segment: the segment maximum (as bits; a NaN
+// becomes the canonical one) and the four table indices, by the arithmetic of the flat quantizer.
+template <int NCODE, int G>
+__device__ __forceinline__ uint32_t encode_four(const float x[4], const CodeTables<NCODE> &tab, bool fast_ok, bool ascending,
+                                                uint32_t idx[4]) {
+    uint32_t m = max(max(abs_bits(x[0]), abs_bits(x[1])), max(abs_bits(x[2]), abs_bits(x[3])));
+    m = group_max_u32<G>(m);
+    // 2^-60 <= maximum <= 2^60, else (zero, huge, tiny, inf, NaN) the exact route
+    if (!fast_ok || (m - kFastDivLo) > (kFastDivHi - kFastDivLo)) {
+        if (m > 0x7f800000u) m = 0x7fc00000u;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) idx[e] = exact_index<NCODE>(x[e], m, tab);
+    } else {
+        const float amax = __uint_as_float(m);
+        const float r = exact_reciprocal(amax);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            idx[e] = fast_index<NCODE, false>(x[e], amax, r, tab, nullptr);
+            if (!ascending) idx[e] = tab.perm[idx[e]];
+        }
+    }
+    return m;
 }
 
 #endif  // __HIPCC__

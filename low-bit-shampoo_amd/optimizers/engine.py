@@ -100,8 +100,12 @@ class ShampooBank:
             eye = torch.eye(order, device=self.device).expand(count, order, order)
             self.stats[order] = X.quantize_stack((self.matrix_eps * eye).contiguous(),
                                                  X.empty_quantized(count, order, self.blocksize, self.bits, self.code, True))
-        for g in self.groups:       # fp32 landing areas of the updated statistics, per group and side
+
+    def _landing(self, g, side):
+        """fp32 landing area of an updated statistic stack (only for blocksizes the requantizing product does not take)."""
+        if getattr(g, "scratch", None) is None:
             g.scratch = [torch.empty(len(g), o, o, device=self.device) for o in (g.bm, g.bn)]
+        return g.scratch[side]
 
     def _fan_out(self, jobs):
         """Run the callables round-robin on the side streams, after everything already queued on the
@@ -186,7 +190,12 @@ class ShampooBank:
             def run():
                 G = self._grad_list(g, grads)
                 seg = self._segment(self.stats, g, side)
-                out = g.scratch[side]
+                if self.blocksize == 64:
+                    # dequantize, update and requantize in one launch: the fp32 statistic never reaches memory
+                    X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, symmetric=True,
+                           requantize=True)
+                    return
+                out = self._landing(g, side)
                 X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, out=out,
                        symmetric=True)
                 X.quantize_stack(out, seg)

@@ -15,7 +15,7 @@ from torch import Tensor
 import qtensor.functional as F
 
 DENSE, DENSE_T, QUANT4, QUANT8 = 0, 1, 2, 3
-EPI_STORE, EPI_AXPBY_DENSE, EPI_AXPBY_QUANT4, EPI_AXPBY_QUANT8, EPI_NEWTON = 0, 1, 2, 3, 4
+EPI_STORE, EPI_AXPBY_DENSE, EPI_AXPBY_QUANT4, EPI_AXPBY_QUANT8, EPI_NEWTON, EPI_REQUANT4, EPI_REQUANT8 = 0, 1, 2, 3, 4, 5, 6
 
 
 class BatchPtr(ct.Structure):
@@ -138,7 +138,7 @@ def _launch(desc: GemmDesc, device: torch.device) -> None:
 
 def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, alpha=1.0, beta=0.0,
          addend=None, newton=None, skip: Optional[Tensor] = None, symmetric: bool = False,
-         upper_a: bool = False, upper_b: bool = False) -> Tensor:
+         upper_a: bool = False, upper_b: bool = False, requantize: bool = False):
     """out[b] = epilogue(op(A[b]) @ op(B[b])).
 
     A, B: fp32 tensors ([m,k] / [batch,m,k]; with trans_x the stored matrix is the transpose) or a
@@ -150,6 +150,9 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
     symmetric: the caller knows the product to be symmetric (a Gram matrix, a product of commuting
     symmetric matrices): only the tiles on and above the diagonal are multiplied out and mirrored,
     which halves the work; the result is then symmetric bit for bit outside the diagonal tiles.
+    requantize (with a `Quantized` addend of blocksize 64): beta*E + alpha*product is encoded straight back
+    into E's buffers (codes, maxima, exact diagonal) -- bit-identical to writing it out and quantizing it, but
+    the fp32 matrix never reaches memory; returns E.
     upper_a / upper_b: op(A) / op(B) is upper triangular (zero below the diagonal, square in its k
     index, dense): the part of the k range where it is zero is skipped."""
     d = GemmDesc()
@@ -180,14 +183,18 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
     if batch_a != batch_b:
         raise ValueError(f"batch sizes differ: {batch_a} vs {batch_b}")
     batch = batch_a
-    if out is None:
-        out = torch.empty((batch, m, n), device=dev, dtype=torch.float32)
-        squeeze = (not isinstance(A, Quantized) and A.dim() == 2) or (not isinstance(B, Quantized) and B.dim() == 2)
-        if squeeze and batch == 1:
-            out = out[0]
-    a.C, a.ldc, batch_c, mc, nc = _dense(out)
-    if (batch_c, mc, nc) != (batch, m, n):
-        raise ValueError(f"out has shape {tuple(out.shape)}, expected batch {batch} x {m} x {n}")
+    if requantize:
+        if not isinstance(addend, Quantized) or addend.blocksize != 64 or out is not None or newton is not None:
+            raise ValueError("requantize needs a quantized addend of blocksize 64 and takes no other output")
+    else:
+        if out is None:
+            out = torch.empty((batch, m, n), device=dev, dtype=torch.float32)
+            squeeze = (not isinstance(A, Quantized) and A.dim() == 2) or (not isinstance(B, Quantized) and B.dim() == 2)
+            if squeeze and batch == 1:
+                out = out[0]
+        a.C, a.ldc, batch_c, mc, nc = _dense(out)
+        if (batch_c, mc, nc) != (batch, m, n):
+            raise ValueError(f"out has shape {tuple(out.shape)}, expected batch {batch} x {m} x {n}")
     d.M, d.N, d.K, d.batch = m, n, k, batch
     d.epilogue = EPI_STORE
     a.alpha, a.beta = alpha, beta
@@ -197,6 +204,8 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
                 raise ValueError("quantized addend must match the batch and be m x m")
             a.Eq = addend.ref()
             d.epilogue = EPI_AXPBY_QUANT4 if addend.bits == 4 else EPI_AXPBY_QUANT8
+            if requantize:
+                d.epilogue = EPI_REQUANT4 if addend.bits == 4 else EPI_REQUANT8
             code = addend.code
         else:
             a.E, a.lde, be, me, ne = _dense(addend)
@@ -233,7 +242,7 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
         scratch = _workspace(dev)
         a.workspace, a.workspace_floats = scratch.data_ptr(), scratch.numel()
     _launch(d, dev)
-    return out
+    return addend if requantize else out
 
 
 def precondition(G: Tensor, left, right, out: Optional[Tensor] = None) -> Tensor:

@@ -269,6 +269,45 @@ def test_quantizer_reading_the_transpose_equals_the_oracle_on_the_transposed_mat
     assert np.array_equal(q.codes[0].cpu().numpy(), o[0]) and np.array_equal(q.diag[0].cpu().numpy(), o[2])
 
 
+@pytest.mark.parametrize("bits,name,n,k,batch,diag", [(4, "linear-2", 768, 256, 3, True), (4, "linear-2", 320, 100, 2, True),
+                                                       (8, "dynamic", 256, 512, 2, True), (4, "dynamic", 128, 64, 5, False),
+                                                       (4, "linear-2", 64, 32, 4, True)])
+def test_statistics_update_encoded_in_place_equals_update_then_quantize_bit_for_bit(mods, code_maps, bits, name, n, k, batch, diag):
+    """L <- beta L + (1 - beta) G G^T (and G^T G) with the result re-encoded inside the product's epilogue: codes,
+    maxima and exact diagonal must be those of the two-step path (fused product to fp32, then the stack quantizer,
+    which the other tests pin to the oracle) -- including zero, tiny, huge and NaN segments."""
+    F, X = mods
+    g = torch.Generator().manual_seed(n + k)
+    code = code_maps[(name, bits)]
+    code_d = torch.from_numpy(code).cuda()
+    L0 = torch.randn(batch, n, n, generator=g)
+    L0 = (L0 @ L0.transpose(1, 2) / n).contiguous()
+    for side in (0, 1):
+        G = (0.3 * torch.randn(batch, n, k, generator=g)) if side == 0 else (0.3 * torch.randn(batch, k, n, generator=g))
+        if side == 0:
+            G[0, 5, :] = 0.0                      # row/column 5 of G G^T is zero
+            G[batch - 1, 7, 3] = float("nan")
+            G[1, 9, :] *= 1e-22                   # maxima below the fast-division range once squared with the addend gone
+        Gd = G.cuda()
+        for beta in (0.95, 0.0):
+            two = X.quantize_stack(L0.cuda(), X.empty_quantized(batch, n, 64, bits, code_d, diag))
+            one = X.quantize_stack(L0.cuda(), X.empty_quantized(batch, n, 64, bits, code_d, diag))
+            kw = dict(trans_b=True) if side == 0 else dict(trans_a=True)
+            half = not (side == 1 and beta == 0.0)          # once with every tile multiplied out
+            dense = X.gemm(Gd, Gd, addend=two, alpha=1.0 - beta, beta=beta, symmetric=True, **kw)
+            X.quantize_stack(dense, two)
+            got = X.gemm(Gd, Gd, addend=one, alpha=1.0 - beta, beta=beta, symmetric=half, requantize=True, **kw)
+            torch.cuda.synchronize()
+            assert got is one
+            assert torch.equal(one.codes, two.codes)
+            assert np.array_equal(one.absmax.cpu().numpy(), two.absmax.cpu().numpy(), equal_nan=True)
+            if diag:
+                assert np.array_equal(one.diag.cpu().numpy(), two.diag.cpu().numpy(), equal_nan=True)
+    with pytest.raises(ValueError):
+        X.gemm(Gd, Gd, trans_a=True, addend=X.empty_quantized(batch, n, 128, bits, code_d, diag) if n % 128 == 0 else None,
+               requantize=True)
+
+
 @pytest.mark.parametrize("n,rows,batch", [(64, 64, 3), (320, 200, 2), (768, 768, 2)])
 def test_products_with_a_triangular_factor_skip_its_zero_part_and_change_nothing(mods, n, rows, batch):
     _, X = mods
