@@ -368,7 +368,7 @@ struct LoadQuant {
 };
 
 template <int BM, int BN, int KA, int KB, int EPI>
-__global__ __launch_bounds__(256) void gemm_kernel(const GemmArgs args) {
+__global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   // three waves per SIMD: at most 168 registers
     constexpr int WM = BM / 2, WN = BN / 2, MI = WM / 32, NI = WN / 32;
     // Workgroups are dealt round-robin to the 8 accelerator dies, each with its own L2.  Renumber
     // them so that every die works through one contiguous run of (batch entry, tile row, tile
