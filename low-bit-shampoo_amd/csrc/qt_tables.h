@@ -30,7 +30,7 @@ constexpr int kLutEntries = 2 * kLutPerSign;
 #if defined(__HIPCC__)
 
 template <int NCODE>
-struct CodeTables {
+struct alignas(16) CodeTables {
     float code[NCODE];     // ascending
     float thr[NCODE];      // thr[i], i < NCODE-1; last slot = +inf
     float raw[NCODE];      // caller's order
@@ -57,11 +57,19 @@ __device__ __forceinline__ int lut_bucket(float v) {
 // #{i < NCODE-1 : !(v < thr[i])}; thr ascending.  NaN counts everything -> NCODE-1.
 template <int NCODE>
 __device__ __forceinline__ int count_thresholds(float v, const float *thr) {
-    int pos = 0;
+    if constexpr (NCODE == 16) {
+        // two levels of four: the quarter from three fixed thresholds (reads that do not depend on v), then the
+        // three thresholds inside it in one 16-byte read -- one dependent LDS access instead of four
+        const int quarter = (int)!(v < thr[3]) + (int)!(v < thr[7]) + (int)!(v < thr[11]);
+        const float4 t = *reinterpret_cast<const float4 *>(thr + 4 * quarter);
+        return 4 * quarter + (int)!(v < t.x) + (int)!(v < t.y) + (int)!(v < t.z);
+    } else {
+        int pos = 0;
 #pragma unroll
-    for (int step = NCODE / 2; step >= 1; step >>= 1)
-        if (!(v < thr[pos + step - 1])) pos += step;
-    return pos;
+        for (int step = NCODE / 2; step >= 1; step >>= 1)
+            if (!(v < thr[pos + step - 1])) pos += step;
+        return pos;
+    }
 }
 
 // All threads of the workgroup call this; ends with a barrier.  lut may be nullptr.
