@@ -6,6 +6,7 @@
 // The only arithmetic done outside the matrix-core GEMM (qtensor_hip_gemm) is the 64 x 64 diagonal
 // block: one wave per matrix factors it in registers and also inverts the factor.
 //   factor:  for each block row j:  U_jj = chol(G_jj);  U_j,> = U_jj^-T G_j,>;  G_>,> -= U_j,>^T U_j,>
+//            (the last step for the rows of the current 256-row panel at once, for the rest per panel)
 //   solve :  the inverted diagonal blocks are doubled up to 256 x 256 -- with blocks A, C already
 //            inverted and B the block of U between them, [A^-1 B; 0 C^-1] gets -A^-1 B C^-1; every level is
 //            two launches for all pairs of all matrices -- then, for each 256-wide column panel j,
@@ -22,6 +23,7 @@ namespace qt {
 namespace {
 
 constexpr int NB = 64;
+constexpr int kFactorPanel = 256;      // rows factored between two updates of the whole trailing matrix
 constexpr int kSolvePanel = 256;       // diagonal blocks of the factor are inverted up to this size, then panels of that width are solved
 
 // One wave per matrix: upper Cholesky factor U (G = U^T U) of a 64 x 64 block and U^-1.
@@ -204,35 +206,56 @@ extern "C" void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float 
     if (!stack_args_ok("cholesky_upper_batched", n, batch, {gram, u, x, info})) return;
     hipStream_t stream = (hipStream_t)stream_v;
     const long long mat = (long long)n * n;
-    const int blocks = n / NB;
-    for (int j = 0; j < blocks; ++j) {
-        const int j0 = j * NB, j1 = j0 + NB, rest = n - j1;
-        const long long corner = (long long)j0 * n + j0;
-        hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram + corner, mat, n, u + corner, mat, n, x + corner,
-                           mat, n, info);
-        if (!launch_ok("cholesky_upper_batched (diagonal block)")) return;
-        if (rest == 0) break;
-        const long long row = (long long)j0 * n + j1;
-        qtensor_gemm_desc d = {};
-        // U_j,> = U_jj^-T G_j,>
-        d.M = NB; d.N = rest; d.K = NB; d.batch = batch;
-        d.kind_a = QTENSOR_DENSE_T; d.kind_b = QTENSOR_DENSE; d.epilogue = QTENSOR_EPI_STORE;
-        d.args.A = strided(x + corner, mat); d.args.lda = n;
-        d.args.B = strided(gram + row, mat); d.args.ldb = n;
-        d.args.C = strided(u + row, mat); d.args.ldc = n;
-        if (!run(d, stream)) return;
-        // G_>,> -= U_j,>^T U_j,>   (symmetric: upper tiles, mirrored)
-        qtensor_gemm_desc t = {};
-        t.M = rest; t.N = rest; t.K = NB; t.batch = batch;
-        t.kind_a = QTENSOR_DENSE_T; t.kind_b = QTENSOR_DENSE; t.epilogue = QTENSOR_EPI_AXPBY_DENSE;
-        t.args.A = strided(u + row, mat); t.args.lda = n;
-        t.args.B = strided(u + row, mat); t.args.ldb = n;
-        const long long next = (long long)j1 * n + j1;
-        t.args.C = strided(gram + next, mat); t.args.ldc = n;
-        t.args.E = strided(gram + next, mat); t.args.lde = n;
-        t.args.alpha = -1.0f; t.args.beta = 1.0f;
-        t.args.symmetric = 1;
-        if (!run(t, stream)) return;
+    // Two levels of blocking: inside a panel of kFactorPanel rows the 64-row steps update only the rest of
+    // the panel's rows (thin strips); the matrix below the panel gets the whole panel at once, with a k
+    // range four times as long -- a quarter of the passes over the trailing matrix.
+    for (int p0 = 0; p0 < n; p0 += kFactorPanel) {
+        const int p1 = p0 + kFactorPanel < n ? p0 + kFactorPanel : n;
+        for (int j0 = p0; j0 < p1; j0 += NB) {
+            const int j1 = j0 + NB, rest = n - j1;
+            const long long corner = (long long)j0 * n + j0;
+            hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram + corner, mat, n, u + corner, mat, n,
+                               x + corner, mat, n, info);
+            if (!launch_ok("cholesky_upper_batched (diagonal block)")) return;
+            if (rest == 0) break;
+            const long long row = (long long)j0 * n + j1;
+            qtensor_gemm_desc d = {};
+            // U_j,> = U_jj^-T G_j,>
+            d.M = NB; d.N = rest; d.K = NB; d.batch = batch;
+            d.kind_a = QTENSOR_DENSE_T; d.kind_b = QTENSOR_DENSE; d.epilogue = QTENSOR_EPI_STORE;
+            d.args.A = strided(x + corner, mat); d.args.lda = n;
+            d.args.B = strided(gram + row, mat); d.args.ldb = n;
+            d.args.C = strided(u + row, mat); d.args.ldc = n;
+            if (!run(d, stream)) return;
+            if (j1 < p1) {
+                // the other rows of the panel: G_[j1,p1),[j1,n) -= U_j,[j1,p1)^T U_j,[j1,n)
+                qtensor_gemm_desc t = {};
+                t.M = p1 - j1; t.N = rest; t.K = NB; t.batch = batch;
+                t.kind_a = QTENSOR_DENSE_T; t.kind_b = QTENSOR_DENSE; t.epilogue = QTENSOR_EPI_AXPBY_DENSE;
+                t.args.A = strided(u + row, mat); t.args.lda = n;
+                t.args.B = strided(u + row, mat); t.args.ldb = n;
+                const long long next = (long long)j1 * n + j1;
+                t.args.C = strided(gram + next, mat); t.args.ldc = n;
+                t.args.E = strided(gram + next, mat); t.args.lde = n;
+                t.args.alpha = -1.0f; t.args.beta = 1.0f;
+                if (!run(t, stream)) return;
+            }
+        }
+        if (p1 < n) {
+            // below the panel: G_>,> -= U_P,>^T U_P,>   (symmetric: upper tiles, mirrored)
+            qtensor_gemm_desc t = {};
+            t.M = n - p1; t.N = n - p1; t.K = p1 - p0; t.batch = batch;
+            t.kind_a = QTENSOR_DENSE_T; t.kind_b = QTENSOR_DENSE; t.epilogue = QTENSOR_EPI_AXPBY_DENSE;
+            const long long rows = (long long)p0 * n + p1;
+            t.args.A = strided(u + rows, mat); t.args.lda = n;
+            t.args.B = strided(u + rows, mat); t.args.ldb = n;
+            const long long next = (long long)p1 * n + p1;
+            t.args.C = strided(gram + next, mat); t.args.ldc = n;
+            t.args.E = strided(gram + next, mat); t.args.lde = n;
+            t.args.alpha = -1.0f; t.args.beta = 1.0f;
+            t.args.symmetric = 1;
+            if (!run(t, stream)) return;
+        }
     }
 }
 
