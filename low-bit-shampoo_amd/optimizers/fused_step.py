@@ -1,9 +1,37 @@
 """One optimizer step with the preconditioner work of all eligible parameters batched in a
 ShampooBank (no counterpart in the reference, whose step() walks the parameters one by one:
 optimizers/shampoo1.py:371-427, shampoo2.py:412-468), and the checkpointing of that bank."""
+import threading
+
 import torch
 
 from optimizers.shampoo_common import CODE
+
+
+class _SideJob:
+    """Runs fn() on a thread and a stream of its own, ordered after what the current stream holds now;
+    join() makes the current stream wait for it and passes an exception on."""
+
+    def __init__(self, device, stream, fn):
+        self.main, self.side, self.error = torch.cuda.current_stream(device), stream, None
+        self.side.wait_stream(self.main)
+
+        def run():
+            try:
+                torch.cuda.set_device(device)
+                with torch.no_grad(), torch.cuda.stream(self.side):       # grad mode and current stream are per thread
+                    fn()
+            except BaseException as exc:                                   # noqa: BLE001 -- handed to join()
+                self.error = exc
+
+        self.thread = threading.Thread(target=run, name="unbatched-statistics")
+        self.thread.start()
+
+    def join(self):
+        self.thread.join()
+        self.main.wait_stream(self.side)
+        if self.error is not None:
+            raise self.error
 
 
 class _FusedStep:
@@ -23,6 +51,9 @@ class _FusedStep:
 
     _update = None                 # _adamw_update or _sgd_update
     bank_keys = ()                 # group entries handed to the bank besides the common ones
+    # True: the statistics update of the parameters the bank does not take runs on a thread of its own while
+    # the bank updates its statistics (worth it where that update waits for the device again and again)
+    overlap_unbatched_statistics = False
 
     @staticmethod
     def bank_class():
@@ -108,10 +139,26 @@ def fused_step(opt, group, update, group_index=0):
         raise RuntimeError("fused=True batches the parameters that had a gradient at the first step; "
                            "every one of them needs a gradient at every later step")
     directions, grafted = {}, set()
+    unbatched = [p for p in params if id(p) not in entry['ids']]
+    side_job = None
+    if (bank is not None and unbatched and opt.overlap_unbatched_statistics and step % group['stat_compute_steps'] == 0
+            and all('preconditioner' in opt.state[p] for p in unbatched)):
+        if entry.get('side_stream') is None:
+            entry['side_stream'] = torch.cuda.Stream(device=unbatched[0].device)
+
+        def update_unbatched():
+            for q in unbatched:
+                opt.state[q]['preconditioner'].add_statistics(grads[id(q)])
+
+        side_job = _SideJob(unbatched[0].device, entry['side_stream'], update_unbatched)
     if bank is not None:
         bgrads = [grads[id(p)] for p in banked]
         if step % group['stat_compute_steps'] == 0:
-            bank.add_statistics(bgrads)
+            try:
+                bank.add_statistics(bgrads)
+            finally:
+                if side_job is not None:
+                    side_job.join()
         if step % group['prec_compute_steps'] == 0:
             bank.compute_preconditioners()
         if step >= group['start_prec_step'] and bank.is_active():
@@ -121,7 +168,7 @@ def fused_step(opt, group, update, group_index=0):
     for p in params:
         if id(p) not in entry['ids']:
             # into a buffer that stays where it is: the fused update keeps a device table of addresses
-            d = opt._shampoo_direction(p, grads[id(p)], group, opt.state[p])
+            d = opt._shampoo_direction(p, grads[id(p)], group, opt.state[p], statistics_done=side_job is not None)
             kept = entry.setdefault('directions', {})
             if id(p) not in kept or kept[id(p)].shape != d.shape or kept[id(p)].dtype != d.dtype:
                 kept[id(p)] = torch.empty_like(d, memory_format=torch.contiguous_format)

@@ -287,6 +287,39 @@ def test_fused_shampoo2_optimizer_runs_and_resumes_from_a_checkpoint(mods, which
         assert torch.equal(a.detach(), b.detach())
 
 
+def test_statistics_of_unbatched_parameters_on_a_side_thread_change_nothing(mods, tmp_path, monkeypatch):
+    """The statistics update of a parameter the bank cannot take runs on a thread and stream of its own while
+    the bank works; states and parameters must be bit-identical to the run that does it in line."""
+    S2, _ = mods
+    import optimizers.matrix_functions as MF
+    monkeypatch.chdir(tmp_path)
+    real_rand = torch.rand
+    monkeypatch.setattr(MF.torch, "rand", lambda *size, **kw: torch.full(size, 0.75, **kw))
+    g = torch.Generator().manual_seed(11)
+    shapes = SHAPES + [(128, 100), (192, 72)]
+    init = [real_rand(s, generator=g) for s in shapes]
+    gs = [[0.02 * torch.randn(s, generator=g) for s in shapes] for _ in range(4)]
+
+    def run(overlap):
+        monkeypatch.setattr(S2.ShampooAdamW, "overlap_unbatched_statistics", overlap)
+        params = [torch.nn.Parameter(x.clone().cuda()) for x in init]
+        opt = S2.ShampooAdamW(params, lr=1e-2, weight_decay=0.05, start_prec_step=2, stat_compute_steps=1,
+                              prec_compute_steps=2, fused=True, inv_root_mode=1, **KW)
+        for grads in gs:
+            for p, gr in zip(params, grads):
+                p.grad = gr.clone().cuda()
+            opt.step()
+        torch.cuda.synchronize()
+        holders = [h for p in params[len(SHAPES):] for h in opt.state[p]['preconditioner'].statistics]
+        return [p.detach().cpu() for p in params], [(h.var.cpu(), h.absmax.cpu(), h.Svalue.cpu(), h.keep_indices.cpu()) for h in holders]
+
+    with_thread, inline = run(True), run(False)
+    for a, b in zip(with_thread[0], inline[0]):
+        assert torch.equal(a, b)
+    for a, b in zip(with_thread[1], inline[1]):
+        assert all(torch.equal(x, y) for x, y in zip(a, b))
+
+
 @pytest.mark.parametrize("variant,fused", [("shampoo1", True), ("shampoo1", False), ("shampoo2", True)])
 def test_optimizers_reduce_a_small_regression_loss(variant, fused, tmp_path, monkeypatch):
     """End-to-end sanity: a two-layer network fitted to a random teacher with 4-bit Shampoo + AdamW."""
