@@ -279,6 +279,9 @@ def main():
     if args.bank_streams is not None:
         from optimizers.engine import ShampooBank
         ShampooBank.DEFAULT_STREAMS = args.bank_streams
+        if args.bank_streams == 0:           # profiling: nothing may overlap, the side thread of shampoo2 neither
+            from optimizers import shampoo2
+            shampoo2.ShampooAdamW.overlap_unbatched_statistics = False
     if args.section in ("gemm", "step", "step2"):
         if args.section == "gemm":
             part = {"fused_gemm": fused_gemm_gpu(torch, code)}
