@@ -16,6 +16,7 @@ quantize_blockwise_diagreal writes for that matrix.  Parameters with a block the
 cannot take (an order that the blocksize does not divide, or too small to quantize) keep a
 per-parameter `Preconditioner`.
 """
+import threading
 from collections import defaultdict
 
 import torch
@@ -36,6 +37,32 @@ class _Group:
 
     def __len__(self):
         return len(self.param_index)
+
+
+class SideJob:
+    """Runs fn() on a thread and a stream of its own, ordered after what the current stream holds now;
+    join() makes the current stream wait for it and passes an exception on."""
+
+    def __init__(self, device, stream, fn):
+        self.main, self.side, self.error = torch.cuda.current_stream(device), stream, None
+        self.side.wait_stream(self.main)
+
+        def run():
+            try:
+                torch.cuda.set_device(device)
+                with torch.no_grad(), torch.cuda.stream(self.side):       # grad mode and current stream are per thread
+                    fn()
+            except BaseException as exc:                                   # noqa: BLE001 -- handed to join()
+                self.error = exc
+
+        self.thread = threading.Thread(target=run, name="shampoo-side-job")
+        self.thread.start()
+
+    def join(self):
+        self.thread.join()
+        self.main.wait_stream(self.side)
+        if self.error is not None:
+            raise self.error
 
 
 class ShampooBank:

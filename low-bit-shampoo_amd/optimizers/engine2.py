@@ -22,7 +22,7 @@ finish are redone with torch.linalg.qr.
 """
 import torch
 
-from optimizers.engine import ShampooBank
+from optimizers.engine import ShampooBank, SideJob
 from optimizers.matrix_functions import ComputePowerBatched
 from qtensor import fused as X
 
@@ -36,6 +36,11 @@ class ShampooBank2(ShampooBank):
         self.qr_fallbacks = 0                     # matrices that went through torch.linalg.qr so far
         self.qr_rounds = 0                        # Cholesky QR rounds so far, summed over the stacks
         super().__init__(params, name2qmap, code, **kwargs)
+
+    def _early_stream(self):
+        if getattr(self, "_early", None) is None:
+            self._early = torch.cuda.Stream(device=self.device)
+        return self._early
 
     def _init_statistics(self):
         """Basis = quantized identity, every kept quotient and the largest one = matrix_eps
@@ -112,9 +117,7 @@ class ShampooBank2(ShampooBank):
         def iterate(order):
             def run():
                 L = stat[order]
-                Q, redone = solver[order].result()
-                self.qr_fallbacks += redone
-                self.qr_rounds += solver[order].rounds
+                Q, redone[order] = solver[order].result()
                 quotients = (Q * X.gemm(L, Q)).sum(dim=1)                      # diag(Q^T L Q)
                 ascending, where = torch.sort(quotients, dim=1)
                 half = self.keep[order].shape[1]
@@ -128,13 +131,27 @@ class ShampooBank2(ShampooBank):
         self._fan_out([accumulate(g, side) for g in self.groups for side in (0, 1)])
         # The Cholesky QR of every order advances on its own stream; the host waits once per round.
         # (_fan_out gives job i the stream i % streams, so an order keeps its stream from call to call.)
-        solver = {}
+        solver, redone = {}, {}
         self._fan_out([project(o) for o in orders])
+        # The stacks whose factorisation is complete go on (Rayleigh quotients, requantize) on a thread and a
+        # stream of their own while the others still iterate: the later rounds of a few ill-conditioned
+        # matrices are chains of small launches that leave most of the device, and this thread, waiting.
+        early, waiting = None, list(orders)
         while not all(solver[o].finished for o in orders):
             self._fan_out([check(o) for o in orders])
             self._fan_out([poll(o) for o in orders])
             self._fan_out([advance(o) for o in orders])
-        self._fan_out([iterate(o) for o in orders])
+            ready = [o for o in waiting if solver[o].finished]
+            if self.streams and early is None and ready and len(ready) < len(waiting):
+                waiting = [o for o in waiting if o not in ready]
+                early = SideJob(self.device, self._early_stream(), lambda: [iterate(o)() for o in ready])
+        try:
+            self._fan_out([iterate(o) for o in waiting])
+        finally:
+            if early is not None:
+                early.join()
+        self.qr_fallbacks += sum(redone.values())
+        self.qr_rounds += sum(solver[o].rounds for o in orders)
 
     @torch.no_grad()
     def compute_preconditioners(self, v0=None):

@@ -1,37 +1,10 @@
 """One optimizer step with the preconditioner work of all eligible parameters batched in a
 ShampooBank (no counterpart in the reference, whose step() walks the parameters one by one:
 optimizers/shampoo1.py:371-427, shampoo2.py:412-468), and the checkpointing of that bank."""
-import threading
-
 import torch
 
+from optimizers.engine import SideJob as _SideJob
 from optimizers.shampoo_common import CODE
-
-
-class _SideJob:
-    """Runs fn() on a thread and a stream of its own, ordered after what the current stream holds now;
-    join() makes the current stream wait for it and passes an exception on."""
-
-    def __init__(self, device, stream, fn):
-        self.main, self.side, self.error = torch.cuda.current_stream(device), stream, None
-        self.side.wait_stream(self.main)
-
-        def run():
-            try:
-                torch.cuda.set_device(device)
-                with torch.no_grad(), torch.cuda.stream(self.side):       # grad mode and current stream are per thread
-                    fn()
-            except BaseException as exc:                                   # noqa: BLE001 -- handed to join()
-                self.error = exc
-
-        self.thread = threading.Thread(target=run, name="unbatched-statistics")
-        self.thread.start()
-
-    def join(self):
-        self.thread.join()
-        self.main.wait_stream(self.side)
-        if self.error is not None:
-            raise self.error
 
 
 class _FusedStep:
