@@ -27,6 +27,10 @@ class _FusedStep:
     # True: the statistics update of the parameters the bank does not take runs on a thread of its own while
     # the bank updates its statistics (worth it where that update waits for the device again and again)
     overlap_unbatched_statistics = False
+    # True: the inverse roots of those parameters (a Newton iteration that waits for the device twice per round)
+    # are computed on a thread of their own while the bank's batched iteration runs; their power-iteration start
+    # vectors are then drawn first, on the calling thread, so that the generator is used in a fixed order
+    overlap_unbatched_inverse_roots = True
 
     @staticmethod
     def bank_class():
@@ -113,7 +117,7 @@ def fused_step(opt, group, update, group_index=0):
                            "every one of them needs a gradient at every later step")
     directions, grafted = {}, set()
     unbatched = [p for p in params if id(p) not in entry['ids']]
-    side_job = None
+    side_job, roots_done, statistics_done = None, False, False
     if (bank is not None and unbatched and opt.overlap_unbatched_statistics and step % group['stat_compute_steps'] == 0
             and all('preconditioner' in opt.state[p] for p in unbatched)):
         if entry.get('side_stream') is None:
@@ -132,8 +136,33 @@ def fused_step(opt, group, update, group_index=0):
             finally:
                 if side_job is not None:
                     side_job.join()
+                    statistics_done = True
         if step % group['prec_compute_steps'] == 0:
-            bank.compute_preconditioners()
+            roots_job = None
+            if (unbatched and opt.overlap_unbatched_inverse_roots
+                    and all('preconditioner' in opt.state[p] for p in unbatched)):
+                if entry.get('side_stream') is None:
+                    entry['side_stream'] = torch.cuda.Stream(device=unbatched[0].device)
+                if side_job is None and step % group['stat_compute_steps'] == 0:
+                    for q in unbatched:                               # this step's statistics come before its roots
+                        opt.state[q]['preconditioner'].add_statistics(grads[id(q)])
+                    statistics_done = True
+                draw = group.get('inv_root_mode', 1) != 0              # the eigenpair route uses no start vectors
+                starts = {id(q): [torch.rand(h.var_order, device=q.device) * 2 - 1
+                                  for h in opt.state[q]['preconditioner'].statistics] if draw else None
+                          for q in unbatched}
+
+                def roots_of_unbatched():
+                    for q in unbatched:
+                        opt.state[q]['preconditioner'].compute_preconditioners(v0=starts[id(q)])
+
+                roots_job = _SideJob(unbatched[0].device, entry['side_stream'], roots_of_unbatched)
+            try:
+                bank.compute_preconditioners()
+            finally:
+                if roots_job is not None:
+                    roots_job.join()
+                    roots_done = True
         if step >= group['start_prec_step'] and bank.is_active():
             # the rescaling to each gradient's norm happens inside the fused update
             directions = {id(p): o for p, o in zip(banked, bank.preconditioned_grads(bgrads))}
@@ -141,7 +170,8 @@ def fused_step(opt, group, update, group_index=0):
     for p in params:
         if id(p) not in entry['ids']:
             # into a buffer that stays where it is: the fused update keeps a device table of addresses
-            d = opt._shampoo_direction(p, grads[id(p)], group, opt.state[p], statistics_done=side_job is not None)
+            d = opt._shampoo_direction(p, grads[id(p)], group, opt.state[p], statistics_done=statistics_done,
+                                       roots_done=roots_done)
             kept = entry.setdefault('directions', {})
             if id(p) not in kept or kept[id(p)].shape != d.shape or kept[id(p)].dtype != d.dtype:
                 kept[id(p)] = torch.empty_like(d, memory_format=torch.contiguous_format)

@@ -222,13 +222,14 @@ class _ShampooOptimizer(optim.Optimizer):
         kwargs = {k: group[k] for k in _PREC_KEYS + tuple(self.extra_keys)}
         return self.preconditioner_class(p, self.name2qmap, **kwargs)
 
-    def _shampoo_direction(self, p, grad, group, state, statistics_done=False):
+    def _shampoo_direction(self, p, grad, group, state, statistics_done=False, roots_done=False):
         """Statistics / inverse-root bookkeeping for this step and the grafted direction
-        (statistics_done: the caller has already run this step's add_statistics)."""
+        (statistics_done / roots_done: the caller has already run this step's add_statistics /
+        compute_preconditioners)."""
         prec = state['preconditioner']
         if state['step'] % group['stat_compute_steps'] == 0 and not statistics_done:
             prec.add_statistics(grad)
-        if state['step'] % group['prec_compute_steps'] == 0:
+        if state['step'] % group['prec_compute_steps'] == 0 and not roots_done:
             prec.compute_preconditioners()
         direction = grad
         if state['step'] >= group['start_prec_step'] and prec.is_active():

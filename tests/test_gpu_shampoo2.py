@@ -288,8 +288,8 @@ def test_fused_shampoo2_optimizer_runs_and_resumes_from_a_checkpoint(mods, which
 
 
 def test_statistics_of_unbatched_parameters_on_a_side_thread_change_nothing(mods, tmp_path, monkeypatch):
-    """The statistics update of a parameter the bank cannot take runs on a thread and stream of its own while
-    the bank works; states and parameters must be bit-identical to the run that does it in line."""
+    """The statistics update and the inverse roots of a parameter the bank cannot take run on a thread and stream
+    of their own while the bank works; states and parameters must be bit-identical to the run that does them in line."""
     S2, _ = mods
     import optimizers.matrix_functions as MF
     monkeypatch.chdir(tmp_path)
@@ -302,6 +302,7 @@ def test_statistics_of_unbatched_parameters_on_a_side_thread_change_nothing(mods
 
     def run(overlap):
         monkeypatch.setattr(S2.ShampooAdamW, "overlap_unbatched_statistics", overlap)
+        monkeypatch.setattr(S2.ShampooAdamW, "overlap_unbatched_inverse_roots", overlap)
         params = [torch.nn.Parameter(x.clone().cuda()) for x in init]
         opt = S2.ShampooAdamW(params, lr=1e-2, weight_decay=0.05, start_prec_step=2, stat_compute_steps=1,
                               prec_compute_steps=2, fused=True, inv_root_mode=1, **KW)
