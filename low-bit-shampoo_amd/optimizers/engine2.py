@@ -144,7 +144,7 @@ class ShampooBank2(ShampooBank):
             ready = [o for o in waiting if solver[o].finished]
             if self.streams and early is None and ready and len(ready) < len(waiting):
                 waiting = [o for o in waiting if o not in ready]
-                early = SideJob(self.device, self._early_stream(), lambda: [iterate(o)() for o in ready])
+                early = SideJob(self.device, self._early_stream(), lambda done=tuple(ready): [iterate(o)() for o in done])
         try:
             self._fan_out([iterate(o) for o in waiting])
         finally:
