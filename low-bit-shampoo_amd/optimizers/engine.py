@@ -6,7 +6,8 @@ kernels for each of them (optimizers/shampoo1.py:148-241, called per parameter f
 same arithmetic is done here with one launch per group of equally shaped blocks:
 
   statistics   L <- b L + (1-b) G G^T : one fused product per (block shape, side) that reads the
-               quantized L inside its epilogue, then one stack quantize
+               quantized L inside its epilogue and writes the result back re-encoded (blocksize 64;
+               other blocksizes: fp32 result, then one stack quantize)
   inverse root one stack dequantize, one batched sync-free Newton run, one stack quantize per order
   P_L G P_R    two fused products per block shape, the quantized factors expanded on the fly
 
