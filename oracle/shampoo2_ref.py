@@ -67,6 +67,7 @@ class RefEigenSlot:
     def __init__(self, order, eps, bits, code, blocksize, min_lowbit_size, rect_t1=1, rect_t2=4, loop=False,
                  positive_r=False):
         self.order, self.rect_t1, self.rect_t2 = order, rect_t1, rect_t2
+        self.read_dtype = torch.float32      # float64: Bjorck steps and rebuilt statistic in double (a yardstick, see below)
         self.low = bits in (4, 8) and order * order >= min_lowbit_size
         self.bits, self.code, self.bs, self.loop, self.positive_r = bits, code, blocksize, loop, positive_r
         keep = max(1, order // 2)
@@ -109,9 +110,9 @@ class RefEigenSlot:
 
     # ---- utils.py:192-203 ----------------------------------------------------------------------
     def dequantize(self):
-        vt = bjorck(self.basis(), self.rect_t1) if self.low else self.dense
+        vt = bjorck(self.basis().to(self.read_dtype), self.rect_t1) if self.low else self.dense
         rows = vt[self.keep]
-        return rows.T @ self.svalue.diag() @ rows, vt
+        return rows.T @ self.svalue.to(vt.dtype).diag() @ rows, vt
 
     # ---- utils.py:156-171 ----------------------------------------------------------------------
     def quantize(self, stat, vt):
@@ -130,9 +131,9 @@ class RefEigenSlot:
     def computepower(self, p, ridge_epsilon, steps=None):
         if steps is None:
             steps = self.rect_t2 if self.low else 0
-        rows = bjorck(self.basis()[self.keep], steps)
+        rows = bjorck(self.basis()[self.keep].to(self.read_dtype), steps)
         rho = ridge_epsilon * self.max_eig
-        weights = 1 / (self.svalue + rho).pow(1 / p)
+        weights = (1 / (self.svalue + rho).pow(1 / p)).to(rows.dtype)
         return rows.T @ weights.diag() @ rows
 
 
@@ -140,6 +141,10 @@ class RefPreconditioner2:
     def __init__(self, shape, code, stat_decay=0.95, matrix_eps=1e-6, prec_maxorder=1200, prec_bits=4,
                  min_lowbit_size=4096, quan_blocksize=64, rect_t1=1, rect_t2=4, inv_root_mode=0, loop=False,
                  positive_r=False):
+        # (root_dtype, set by tests to torch.float64 before compute_preconditioners: the inverse roots -- Bjorck
+        # steps, rebuilt statistic, Newton iteration -- in double on the same stored state; not the reference's
+        # arithmetic, but the yardstick for how far fp32 rounding alone moves an inverse root)
+        self.root_dtype = torch.float32
         dims = [d for d in shape if d != 1]
         self.shape = tuple(shape)
         self.rank2 = len(dims) > 1
@@ -186,12 +191,14 @@ class RefPreconditioner2:
     def compute_preconditioners(self, v0s=None):
         """v0s (mode 1 only): one power-iteration start vector per statistic, in storage order."""
         for i, (slot, prec) in enumerate(zip(self.stats, self.precs)):
+            slot.read_dtype = self.root_dtype
             if self.mode == 0:
                 root = slot.computepower(4, self.eps)
             else:
                 stat, _ = slot.dequantize()
-                root = newton_root(stat.float().clone(), 4, self.eps, v0s[i])
-            prec.put(root)
+                root = newton_root(stat.clone(), 4, self.eps, v0s[i])
+            slot.read_dtype = torch.float32
+            prec.put(root.float())
         self.active = True
 
     def preconditioned_grad(self, grad):

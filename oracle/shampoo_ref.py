@@ -36,7 +36,7 @@ def pieces(extent: int, block: int):
 
 
 def power_iteration(mat, v0, tol=1e-6, iters=10):
-    v, value, change, used = v0.clone(), 0.0, 1.0, 0
+    v, value, change, used = v0.to(mat.dtype).clone(), 0.0, 1.0, 0
     while change > tol and used < iters:
         v = v / torch.norm(v)
         w = torch.mv(mat, v)
@@ -50,7 +50,7 @@ def power_iteration(mat, v0, tol=1e-6, iters=10):
 def newton_root(mat, p, eps, v0, iters=10, tol=1e-6):
     """(mat + eps*lambda_max*I)^(-1/p); mat is modified like in the reference."""
     n = mat.shape[0]
-    eye = torch.eye(n)
+    eye = torch.eye(n, dtype=mat.dtype)          # (float64 input: the same iteration in double, used as a yardstick)
     if n == 1:
         return eye
     w = -1.0 / p
@@ -109,10 +109,13 @@ class _Slot:
 
 class RefPreconditioner:
     def __init__(self, shape, code, stat_decay=0.95, matrix_eps=1e-6, prec_maxorder=1200, prec_bits=4,
-                 min_lowbit_size=4096, quan_blocksize=64, loop=False):
+                 min_lowbit_size=4096, quan_blocksize=64, loop=False, root_dtype=torch.float32):
+        # root_dtype=torch.float64 runs the Newton iteration in double on the same stored statistics: not the
+        # reference's arithmetic, but the yardstick for how far fp32 rounding alone moves an inverse root
         dims = [d for d in shape if d != 1]
         self.shape = tuple(shape)
         self.rank2 = len(dims) > 1
+        self.root_dtype = root_dtype
         self.beta, self.eps = stat_decay, matrix_eps
         self.active = False
         self.stats, self.precs = [], []
@@ -155,10 +158,10 @@ class RefPreconditioner:
     def compute_preconditioners(self, v0s):
         """v0s: one start vector per statistic, in storage order."""
         for slot, prec, v0 in zip(self.stats, self.precs, v0s):
-            stat = slot.get()
-            root = newton_root(stat, 4, self.eps, v0)
+            stat = slot.get().to(self.root_dtype)
+            root = newton_root(stat, 4, self.eps, v0).float()
             if not slot.low:
-                slot.dense = stat          # the reference's in-place ridge on a dense statistic
+                slot.dense = stat.float()  # the reference's in-place ridge on a dense statistic
             prec.put(root)
         self.active = True
 

@@ -82,6 +82,45 @@ def test_svdfast_low_bit_tracks_dense_eigenbasis(U, code_maps, tmp_path, monkeyp
     assert float((p_low - p_dense).norm() / p_dense.norm()) < 0.7
 
 
+def test_svdfast_low_bit_follows_the_oracle_holder(U, code_maps, tmp_path, monkeypatch):
+    """QTensorSVDFast in 4 bits against the CPU restatement of the reference holder (oracle/shampoo2_ref.py,
+    R made positive on its diagonal), update by update from the same stored bits: codes, segment maxima,
+    kept quotients and rows, largest quotient, rebuilt statistic and the inverse root from the eigenpairs."""
+    from oracle.shampoo2_ref import RefEigenSlot
+    monkeypatch.chdir(tmp_path)
+    code = code_maps[("linear-2", 4)]
+    g = torch.Generator().manual_seed(1)
+    n = 128
+    low = U.QTensorSVDFast(1e-6 * torch.eye(n, device="cuda"), bits=4, name2qmap=qmap(code_maps), code="linear-2",
+                           blocksize=64, min_lowbit_size=4096)
+    ref = RefEigenSlot(n, 1e-6, 4, code, 64, 4096, positive_r=True)
+    flips = 0
+    for _ in range(3):
+        X_ = torch.randn(n, 4 * n, generator=g)
+        L = X_ @ X_.T / (4 * n)
+        codes, absmax = ref.codes()
+        low.var.copy_(torch.from_numpy(codes)), low.absmax.copy_(torch.from_numpy(absmax))
+        low.Svalue, low.keep_indices, low.max_eigenvalue = ref.svalue.cuda(), ref.keep.cuda(), ref.max_eig.cuda()
+        a_ref, vt_ref = ref.dequantize()
+        a_low, vt_low = low.dequantize()
+        assert float((a_low.cpu() - a_ref).norm()) <= 1e-5 * max(float(a_ref.norm()), 1e-6)     # same bits in: rounding only
+        assert float((vt_low.cpu() - vt_ref).abs().max()) <= 1e-5
+        ref.quantize(0.9 * a_ref + 0.1 * L, vt_ref)
+        low.quantize(0.9 * a_low + 0.1 * L.cuda(), vt_low)
+        codes, absmax = ref.codes()
+        got = low.var.cpu().numpy()
+        flips += int(np.count_nonzero((got >> 4) != (codes >> 4)) + np.count_nonzero((got & 15) != (codes & 15)))
+        assert float((low.absmax.cpu() - torch.from_numpy(absmax)).abs().max()) <= 1e-5 * float(absmax.max())
+        assert torch.equal(low.keep_indices.cpu(), ref.keep)
+        top = float(ref.max_eig)
+        assert float((low.Svalue.cpu() - ref.svalue).abs().max()) <= 1e-5 * top
+        assert abs(float(low.max_eigenvalue) - top) <= 1e-5 * top
+        p_ref, p_low = ref.computepower(4, 1e-6), low.computepower(4, 1e-6).cpu()
+        assert float((p_low - p_ref).norm() / p_ref.norm()) <= 5e-3                 # (a differing code or two)
+    print("QTensorSVDFast: differing codes over three updates", flips, "of", 3 * n * n)
+    assert flips <= 1e-3 * 3 * n * n
+
+
 def test_shampoo2_low_bit_preconditioner_matches_host_recomputation_from_its_own_state(code_maps, tmp_path, monkeypatch):
     """4-bit eigenbasis storage is lossy by design, so the low-bit preconditioner is not compared with
     the 32-bit one; every stage is recomputed on the host from the state the holders actually store."""
