@@ -195,6 +195,21 @@ typedef struct {
  * (DENSE, DENSE_T) or (DENSE_T, DENSE); anything else is an error. */
 void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
 
+/* qtensor_hip_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc); it has no counterpart in the reference.  The partial
+ * products of a product that is cut along k go to a static device array of the library image,
+ * QTENSOR_STATIC_SCRATCH_FLOATS floats (64 MiB) per GPU, held until the process ends; desc->args.workspace
+ * is ignored and nothing is allocated or freed, here or in any routine it calls.  Takes the plain-store
+ * epilogue without the symmetric / triangular / two-level batch options (the only products that are ever cut);
+ * anything else, and any product with 2 * batch * M * N > QTENSOR_STATIC_SCRATCH_FLOATS, is refused with an
+ * error and nothing is launched.  Results are bit-identical to qtensor_hip_gemm with a caller workspace of
+ * that size.  All calls on one GPU share the array: calls that overlap in time on one GPU (several streams or
+ * threads) race; nothing in the array needs clearing between calls (every partial product is written in full
+ * before it is read).  The first call on a GPU looks the array's address up (hipGetSymbolAddress): make it
+ * before a graph capture begins. */
+#define QTENSOR_STATIC_SCRATCH_FLOATS (1 << 24)
+void qtensor_hip_gemm_static(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
+
 /* ---- batched Cholesky factorisation and triangular solve (Cholesky QR) ---------------------------
  * Replace, for a whole stack of statistics at once, the QR factorisation the reference calls per
  * matrix in QTensorSVDFast.quantize (torch.linalg.qr, qtensor/utils.py:157): one round of

@@ -25,6 +25,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
 
 namespace qt {
@@ -845,10 +846,76 @@ struct qtensor_gemm_desc {
     qt::GemmArgs args;
 };
 
+// Scratch that is part of the library image, for callers that cannot allocate (qtensor_hip_gemm_static):
+// one copy per GPU, held until the process ends.  In host code the name is only a handle for
+// hipGetSymbolAddress; kernels get the address that call returns.
+#ifndef QTENSOR_STATIC_SCRATCH_FLOATS
+#define QTENSOR_STATIC_SCRATCH_FLOATS (1 << 24)
+#endif
+static __device__ __align__(256) float scratch[QTENSOR_STATIC_SCRATCH_FLOATS];
+
+namespace {
+// Device address of `scratch` on the current device, looked up once per device.
+float *static_scratch() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex guard;
+    static float *address[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        qt::set_error(qt::kBadArgument, "gemm_static: no current device");
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(guard);
+    if (address[dev] == nullptr) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr) {
+            qt::set_error(qt::kLaunchFailed, "gemm_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        address[dev] = static_cast<float *>(p);
+    }
+    return address[dev];
+}
+
+void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream);
+}  // namespace
+
 extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
+    qt::clear_error();
+    gemm_dispatch(d, (hipStream_t)stream_v);
+}
+
+extern "C" void qtensor_hip_gemm_static(const qtensor_gemm_desc *d, void *stream_v) {
     using namespace qt;
     clear_error();
-    hipStream_t stream = (hipStream_t)stream_v;
+    if (!d) { set_error(kNullPointer, "gemm_static: null descriptor"); return; }
+    if (d->M < 1 || d->N < 1 || d->K < 1 || d->batch < 1 || d->batch > 65535) {
+        set_error(kBadArgument, "gemm_static: need M, N, K >= 1 and 1 <= batch <= 65535 (got %d %d %d, batch %d)", d->M, d->N, d->K, d->batch);
+        return;
+    }
+    if (d->epilogue != kStore || d->args.symmetric != 0 || d->args.batch_inner > 1 || d->args.triangular != 0) {
+        set_error(kBadArgument, "gemm_static: only plain-store products without the symmetric / triangular / two-level batch "
+                                "options are cut along k; the others need no scratch: use qtensor_hip_gemm");
+        return;
+    }
+    const long long need = 2LL * d->batch * d->M * d->N;       // two partial products: the least a cut needs
+    if (need > QTENSOR_STATIC_SCRATCH_FLOATS) {
+        set_error(kBadArgument, "gemm_static: 2 * batch * M * N = %lld floats exceed the static scratch of %d floats",
+                  need, QTENSOR_STATIC_SCRATCH_FLOATS);
+        return;
+    }
+    float *ptr = static_scratch();
+    if (ptr == nullptr) return;
+    qtensor_gemm_desc with_scratch = *d;
+    with_scratch.args.workspace = ptr;
+    with_scratch.args.workspace_floats = QTENSOR_STATIC_SCRATCH_FLOATS;
+    gemm_dispatch(&with_scratch, (hipStream_t)stream_v);
+}
+
+namespace {
+void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
+    using namespace qt;
     if (!d) { set_error(kNullPointer, "gemm: null descriptor"); return; }
     GemmArgs a = d->args;
     a.M = d->M; a.N = d->N; a.K = d->K;
@@ -987,3 +1054,4 @@ extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
 #undef QT_GEMM_CASE
     launch_ok("gemm");
 }
+}  // namespace
