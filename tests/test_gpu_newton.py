@@ -53,3 +53,26 @@ def test_batched_power_iteration_and_stopping_rules():
         assert float((out[b] - want).norm() / want.norm()) <= 1e-5
     one = ComputePowerBatched(torch.full((3, 1, 1), 5.0, device="cuda"), 4)
     assert torch.equal(one.cpu(), torch.ones(3, 1, 1))
+
+
+@pytest.mark.parametrize("n,cond", [(768, 4.0), (768, 6.0), (1024, 4.0), (1024, 6.0), (256, 6.0)])
+def test_ill_conditioned_inverse_roots_are_as_good_as_the_cpu_iteration(n, cond):
+    """Eigenvalues log-uniform in [10^-cond, 1] (the spread of the statistics in the fused-product and ViT-B/32
+    workloads).  Ten Newton rounds in fp32 do not reach the definition (G + r I)^(-1/4) to 1e-5 there, on any
+    machine; the claim is that the matrix-core path is as close to it as the reference's own fp32 arithmetic on
+    the CPU: error(GPU) <= 2 * error(CPU fp32 iteration) + 1e-5, both measured against float64 eigh, and the
+    two fp32 results agree with each other to a small multiple of the CPU's own error."""
+    batch = 2
+    mats, v0 = psd_stack(batch, n, cond, seed=int(n + cond))
+    got = ComputePowerBatched(mats.clone().cuda(), 4, ridge_epsilon=1e-6, v0=v0).cpu()
+    for b in range(batch):
+        cpu = ComputePower(mats[b].clone(), 4, ridge_epsilon=1e-6, v0=v0[b])
+        lam, vec = torch.linalg.eigh(mats[b].double())
+        top, _, _ = PowerIter(mats[b], v0=v0[b])
+        exact = (vec * (lam + 1e-6 * float(top)) ** -0.25) @ vec.T
+        e_cpu = float((cpu.double() - exact).norm() / exact.norm())
+        e_gpu = float((got[b].double() - exact).norm() / exact.norm())
+        apart = float((got[b] - cpu).norm() / cpu.norm())
+        print(f"n {n} cond 1e{cond:.0f}: error of the CPU fp32 iteration {e_cpu:.2e}, of the GPU {e_gpu:.2e}, apart {apart:.2e}")
+        assert e_gpu <= 2 * e_cpu + 1e-5, (n, cond, b, e_cpu, e_gpu)
+        assert apart <= 5e-5, (n, cond, b, apart)
