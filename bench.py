@@ -6,10 +6,12 @@ on one MI355X, reported as achieved HBM GB/s over the algorithmic bytes.
 
 One "step" = one quantize launch + one dequantize launch over the whole tensor, inputs
 resident in HBM.  The same JSON line also carries, under "precond_step", the second half of the
-metric: ms per 4-bit Shampoo preconditioner step over the ViT-B/32 weight shapes, with the CPU
-restatement timed on a bounded sample beside it; under "fused_gemm" the fused dequantize -> MFMA
-products deq(L) G deq(R) against the fp32 matrix peak; under "other_formats" the 8-bit and
-blocksize-256 variants of the headline tensor.  Prints one JSON line.
+metric: ms per full 4-bit Shampoo2 step (eigenbasis variant, coupled-Newton inverse roots) over the
+ViT-B/32 weight shapes, with its own roofline entry (the batched fp32 MFMA product that dominates
+it) and the CPU restatement timed on a bounded sample beside it; under "precond_step_naive" the
+same for the variant that stores the statistics themselves; under "fused_gemm" the fused
+dequantize -> MFMA products deq(L) G deq(R) against the fp32 matrix peak; under "other_formats"
+the 8-bit and blocksize-256 variants of the headline tensor.  Prints one JSON line.
 """
 import argparse
 import json
@@ -31,6 +33,9 @@ BYTES_PER_ELEMENT = 4 + BITS / 8 + 4 / BLOCK      # fp32 in/out + packed code + 
 # HBM bytes per launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE on this workload, scaled by
 # the library's plain copy kernel (summary: profiles/quantize_dequantize_16384sq_4bit_bs64_hbm_traffic.txt)
 MEASURED_TRAFFIC = {"quantize": 1225662500, "dequantize": 1225738000}
+TRAFFIC_SOURCE = ("profiles/quantize_dequantize_16384sq_4bit_bs64_hbm_traffic.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
+                  "this workload, scaled by the same counters over the library's plain copy kernel; a kept profile, "
+                  "not re-measured by this run")
 
 
 def stress_tensor(torch, order, seed=0):
@@ -223,31 +228,80 @@ def other_formats_gpu(torch, F, x):
     return out
 
 
-def precond_step_cpu(torch, code_host):
-    """The same regular step (statistics update + preconditioned gradient) for ONE transformer layer
-    (qkv, proj, fc1, fc2: 10 of the 124 blocks) through the CPU restatement whose quantizer is the
-    reference's per-segment torch loop; the inverse roots are timed separately on the same layer."""
-    from oracle.shampoo_ref import RefPreconditioner
+LAYER_SHAPES = [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
 
+
+def block_cost(shapes):
+    """Sum over the blocks (at most 1024 per side) of m^2 n + m n^2: what the cost of a step is proportional to
+    (Gram matrices and applications 2 (m^2 n + m n^2) flop each; the per-statistic work n^3 follows it closely)."""
+    total = 0
+    for m, n in shapes:
+        rows = [1024] * ((m - 1) // 1024) + [m - 1024 * ((m - 1) // 1024)]
+        cols = [1024] * ((n - 1) // 1024) + [n - 1024 * ((n - 1) // 1024)]
+        total += sum(a * a * b + a * b * b for a in rows for b in cols)
+    return total
+
+
+def precond_step_cpu(torch, code_host, variant):
+    """The same regular step (statistics update + preconditioned gradient + norm graft) for ONE transformer
+    layer (qkv, proj, fc1, fc2: 10 of the 124 blocks) through the CPU restatement of the reference flow with the
+    bit width forced to 4, whose quantizer is the reference's per-segment torch loop."""
+    if variant == "shampoo2":
+        from oracle.shampoo2_ref import RefPreconditioner2
+        make = lambda s: RefPreconditioner2(s, code_host.numpy(), loop=True, inv_root_mode=1, **STEP_KW)   # noqa: E731
+    else:
+        from oracle.shampoo_ref import RefPreconditioner
+        make = lambda s: RefPreconditioner(s, code_host.numpy(), loop=True, **STEP_KW)                     # noqa: E731
     g = torch.Generator().manual_seed(1)
-    shapes = [(768, 2304), (768, 768), (768, 3072), (3072, 768)]
-    grads = [0.02 * torch.randn(s, generator=g) for s in shapes]
-    pres = [RefPreconditioner(s, code_host.numpy(), loop=True, **STEP_KW) for s in shapes]
+    grads = [0.02 * torch.randn(s, generator=g) for s in LAYER_SHAPES]
+    pres = [make(s) for s in LAYER_SHAPES]
     t0 = time.perf_counter()
     for pre, gr in zip(pres, grads):
         pre.add_statistics(gr)
         out = pre.preconditioned_grad(gr)
         out.mul_(gr.norm() / (out.norm() + 1e-12))
     regular = time.perf_counter() - t0
+    factor = block_cost(vit_b32_shapes()) / block_cost(LAYER_SHAPES)
     return {
+        "value": round(regular * 1e3 * factor, 1),
+        "unit": "ms per regular step, EXTRAPOLATED from the sample by the ratio %.2f of sum(m^2 n + m n^2) over the blocks" % factor,
         "kind": "port",
         "cores": torch.get_num_threads(),
         "sample": "one transformer layer (4 of 50 parameters, 10 of 124 blocks, 20 of 248 statistics): statistics "
-                  "update + preconditioned gradient + norm graft; quantizer = per-segment torch loop (1 core), "
-                  "products = torch.matmul on %d threads" % torch.get_num_threads(),
+                  "update + preconditioned gradient + norm graft through oracle/%s; quantizer = per-segment torch "
+                  "loop (1 core), products%s = torch on %d threads"
+                  % ("shampoo2_ref.py" if variant == "shampoo2" else "shampoo_ref.py",
+                     " and QR" if variant == "shampoo2" else "", torch.get_num_threads()),
         "seconds_for_sample": round(regular, 3),
-        "ms_per_full_step_extrapolated": round(regular * 1e3 * 124 / 10, 1),
     }
+
+
+def dominant_product_gpu(torch):
+    """The kernel most of a step's time goes to -- gemm_kernel<128,128,dense,dense,store>, the batched plain fp32
+    product (L Q, the Newton products, the solve panels) -- on the step's biggest stack (99 statistics of order
+    1024), timed per launch with events on the launch stream."""
+    import qtensor.fused as X
+    g = torch.Generator(device="cuda").manual_seed(5)
+    batch, n = 99, 1024
+    A = torch.randn(batch, n, n, device="cuda", generator=g)
+    B = torch.randn(batch, n, n, device="cuda", generator=g)
+    C = torch.empty(batch, n, n, device="cuda")
+    for _ in range(3):
+        X.gemm(A, B, out=C)
+    reps = 10
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+    ev[0].record()
+    for i in range(reps):
+        X.gemm(A, B, out=C)
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    ms = sum(ev[i].elapsed_time(ev[i + 1]) for i in range(reps)) / reps
+    flop = 2.0 * batch * n ** 3
+    tf = flop / (ms * 1e-3) / 1e12
+    return {"bound": "mfma", "kernel": "gemm_kernel<128,128,dense,dense,store> on 99 x (1024 x 1024 x 1024)",
+            "achieved": round(tf, 1), "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(tf / FP32_MATRIX_PEAK_TFLOPS, 4), "traffic": None, "avg_launch_ms": round(ms, 4),
+            "algorithmic_flop_per_launch": flop}
 
 
 def main():
@@ -256,7 +310,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--section", choices=["all", "quant", "gemm", "step", "step2"], default="all",
+    ap.add_argument("--section", choices=["all", "quant", "gemm", "step", "step2", "product"], default="all",
                     help="run only one part (for profiling one kernel family); the JSON line then lacks the others")
     ap.add_argument("--bank-streams", type=int, default=None,
                     help="side streams of the batched preconditioner engine (0 serialises its launches, which "
@@ -282,13 +336,15 @@ def main():
         if args.bank_streams == 0:           # profiling: nothing may overlap, the side thread of shampoo2 neither
             from optimizers import shampoo2
             shampoo2.ShampooAdamW.overlap_unbatched_statistics = False
-    if args.section in ("gemm", "step", "step2"):
+    if args.section in ("gemm", "step", "step2", "product"):
         if args.section == "gemm":
             part = {"fused_gemm": fused_gemm_gpu(torch, code)}
         elif args.section == "step":
-            part = {"precond_step": precond_step_gpu(torch)}
+            part = {"precond_step_naive": precond_step_gpu(torch)}
+        elif args.section == "product":
+            part = {"roofline": dominant_product_gpu(torch)}
         else:
-            part = {"precond_step_shampoo2": precond_step_gpu(torch, "shampoo2")}
+            part = {"precond_step": precond_step_gpu(torch, "shampoo2")}
         print(json.dumps({"section": args.section, "n_gpus": 1, **part}))
         return
     if args.section == "quant":
@@ -365,6 +421,7 @@ def main():
             "unit": "GB/s",
             "frac": round(q_gbs / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC["quantize"],
+            "traffic_source": TRAFFIC_SOURCE,
             "avg_launch_ms": round(q_ms, 4),
             "algorithmic_bytes_per_launch": int(algo),
         },
@@ -384,15 +441,18 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_step:
         result["fused_gemm"] = fused_gemm_gpu(torch, code)
-        result["precond_step"] = precond_step_gpu(torch)
-        result["precond_step_shampoo2"] = precond_step_gpu(torch, "shampoo2")
+        # the step BASELINE's configuration names: eigenbasis variant with coupled-Newton inverse roots
+        result["precond_step"] = precond_step_gpu(torch, "shampoo2")
+        result["precond_step"]["roofline"] = dominant_product_gpu(torch)
+        result["precond_step_naive"] = precond_step_gpu(torch, "shampoo1")
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(torch, x_slice, code_host)
         if not args.no_step:
-            cpu = precond_step_cpu(torch, code_host)
-            result["precond_step"]["cpu_baseline"] = cpu
-            result["precond_step"]["speedup_vs_cpu_regular_step"] = round(
-                cpu["ms_per_full_step_extrapolated"] / result["precond_step"]["ms_per_step_regular"], 1)
+            for key, variant in (("precond_step", "shampoo2"), ("precond_step_naive", "shampoo1")):
+                cpu = precond_step_cpu(torch, code_host, variant)
+                result[key]["cpu_baseline"] = cpu
+                result[key]["speedup_vs_extrapolated_cpu_regular_step"] = round(
+                    cpu["value"] / result[key]["ms_per_step_regular"], 1)
     print(json.dumps(result))
 
 
