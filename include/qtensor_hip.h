@@ -218,10 +218,17 @@ void qtensor_hip_gemm_static(const qtensor_gemm_desc *desc, qtensor_stream_t str
  * Stacks are contiguous [batch, n, n] fp32 with n a multiple of 64; everything runs on `stream`.
  *
  * cholesky_upper: gram (upper triangle read, contents destroyed) = U^T U.  u receives the block
- *   rows of U on and above the diagonal (the part below the diagonal blocks is not written); the
+ *   rows of U on and above the diagonal (of the part below the diagonal blocks only the 64 x 64 block under
+ *   each diagonal block is written: scratch); the
  *   64 x 64 diagonal blocks of x [batch, n, n] receive the inverses of U's diagonal blocks (nothing
- *   else of x is touched).  info[b] (zeroed by the caller) is set to 1 when matrix b has a
- *   non-positive pivot (its factor is then meaningless).
+ *   else of x is touched).  info[b] (zeroed by the caller) gets bit 0 set when matrix b has a
+ *   non-positive or NaN pivot (its factor is then meaningless).
+ * cholesky_upper_floor: the same with a floor under the pivots (the squared lengths of what is left of a
+ *   column after the columns before it are taken out): a pivot that is not above pivot_floor -- a column that
+ *   depends on the earlier ones up to the rounding noise of the Gram matrix -- is taken out of the factorisation
+ *   (pivot = the floor, rest of its row of U zero) and bit 1 of info[b] is set; q U^-1 then leaves that column
+ *   lifted by 1 / sqrt(pivot_floor) instead of failing, and a repeated round completes the basis.  Bit 0 is
+ *   then only set by a NaN.  pivot_floor = 0 is cholesky_upper.
  * solve_upper_right: out = q U^-1 for q, out [batch, rows, n] with u, x from cholesky_upper.  x must
  *   be zero below its diagonal blocks (zero it once before the first factorisation; no call writes
  *   there).  Its inverted diagonal blocks are doubled level by level (two launches per level for all
@@ -229,6 +236,22 @@ void qtensor_hip_gemm_static(const qtensor_gemm_desc *desc, qtensor_stream_t str
  *   out_j = (q_j - out_<j U_<j,j) x_jj.  work is scratch of batch * max(rows, n) * n floats (gram may
  *   be passed when rows <= n).  out must not alias q. */
 void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float *x, int *info, int n, int batch, qtensor_stream_t stream);
+void qtensor_hip_cholesky_upper_floor_batched(float *gram, float *u, float *x, int *info, int n, int batch, float pivot_floor,
+                                              qtensor_stream_t stream);
+/* Block Gram-Schmidt with reorthogonalisation, in place: the columns of every q[b] (n x n, unit columns on entry) are
+ * made orthonormal left to right in panels -- a panel has the finished columns taken out of it (W = Q_<^T Y_p,
+ * Y_p -= Q_< W), its columns rescaled to unit length, is orthonormalised inside, and all of that once more; on
+ * the outer level a panel is qtensor_hip_block_gram_schmidt_width() columns wide and "inside" is the same scheme
+ * over its 64-column panels, where "inside" is Cholesky QR (pivot_floor as in cholesky_upper_floor).  Keeps span(q[:, :k]) for every k like the Cholesky
+ * QR rounds above, but loses orthogonality only in proportion to fp32 rounding, not to the squared condition
+ * number, so one sweep replaces their repetition; it replaces torch.linalg.qr of qtensor/utils.py:157 for a whole
+ * stack.  fill (optional, [n, n], unit columns): a column that the first projection leaves shorter than
+ * sqrt(null_norm2) -- rounding noise: it depends on the columns before it -- is replaced by the same column of
+ * fill (bit 2 of info[b]) and then treated like any other.  w: scratch [batch, n, width]; gram, u, x: scratch
+ * [batch, 64, 64] each; info as in cholesky_upper_floor (zeroed by the caller). */
+int qtensor_hip_block_gram_schmidt_width(void);
+void qtensor_hip_block_gram_schmidt_batched(float *q, float *w, float *gram, float *u, float *x, const float *fill, int *info,
+                                            int n, int batch, float pivot_floor, float null_norm2, qtensor_stream_t stream);
 /* The test that ends the rounds: out[2 b] = max |G_b - I|, out[2 b + 1] = ||G_b - I||_F^2 for the stack
  * gram [batch, n, n], one pass, fixed summation order, NaN if G_b holds one.  partial: scratch of
  * batch * 64 floats.  (No counterpart in the reference: Householder QR needs no such test.) */

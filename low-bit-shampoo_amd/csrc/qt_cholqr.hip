@@ -27,8 +27,16 @@ constexpr int kFactorPanel = 256;      // rows factored between two updates of t
 constexpr int kSolvePanel = 256;       // diagonal blocks of the factor are inverted up to this size, then panels of that width are solved
 
 // One wave per matrix: upper Cholesky factor U (G = U^T U) of a 64 x 64 block and U^-1.
-// Reads the upper triangle of G only.  A non-positive (or NaN) pivot sets info[b] = 1 and is
-// replaced by 1; the factor of that matrix is then meaningless.
+// Reads the upper triangle of G only.  A pivot that is not above `pivot_floor` is a column that depends on
+// the ones before it up to the rounding noise of the Gram matrix.  With pivot_floor > 0 such a column is
+// taken out of the factorisation: its pivot becomes the floor and the rest of its row of U zero (bit 1 of
+// info[b] is set), so nothing of its noise reaches the columns after it; Q U^-1 still takes the earlier
+// columns out of it and lifts what is left by 1 / sqrt(floor), and the next round treats it like any other
+// column.  (Raising the pivot alone lets the noise grow geometrically through the trailing updates.)
+// `inv` receives U^-1; `panel_inv`, if not null, the same with the dropped columns' rows of U^-T zeroed: the
+// factor that turns G_j,> into the block row U_j,> with zero rows for the dropped columns.
+// With pivot_floor == 0, and for a NaN pivot always, bit 0 of info[b] is set, the pivot is replaced by 1 and
+// the factor of that matrix is meaningless.
 //
 // Lane i keeps row i of the (full, symmetric) trailing matrix in registers.  Step k scales column k
 // (one value per lane) into column k of L = U^T, parks it in LDS, and every lane reads it back as
@@ -44,7 +52,7 @@ __device__ __forceinline__ float lane_value(float x, int lane) {
 
 __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long long g_stride, int ldg, float *u,
                                                         long long u_stride, int ldu, float *inv, long long inv_stride,
-                                                        int ldi, int *info) {
+                                                        int ldi, float *panel_inv, int *info, float pivot_floor) {
     __shared__ __attribute__((aligned(16))) float cols[NB][LDC];
     const int b = blockIdx.x, lane = threadIdx.x;
     const float *G = gram + (long long)b * g_stride;
@@ -59,6 +67,7 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
     }
     __syncthreads();
     bool ok = true;
+    unsigned long long dropped = 0;              // columns taken out of the factorisation (uniform over the wave)
     // Step k: pivot, column k of L, then the two next columns at once through v_readlane (they carry the
     // chain from one pivot to the next); all further columns get the update of step k one step later, from
     // the copy of column k parked in LDS, so that no pivot ever waits for an LDS round trip.
@@ -71,10 +80,15 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
             for (int j = (k + 2) & ~3; j < NB; j += 4) far[j / 4] = *reinterpret_cast<const float4 *>(&cols[k - 1][j]);
         }
         float d = lane_value(row[k], k);
-        if (!(d > 0.0f)) { ok = false; d = 1.0f; }
+        bool drop = false;
+        if (!(d > pivot_floor)) {
+            if (pivot_floor > 0.0f && d == d) { drop = true; dropped |= 1ull << k; d = pivot_floor; }
+            else { ok = false; d = 1.0f; }
+        }
         float r = __builtin_amdgcn_rsqf(d);
         r = r * __builtin_fmaf(-0.5f * d * r, r, 1.5f);
-        const float l = row[k] * r;              // L[lane][k] (lanes above k: unused values)
+        float l = row[k] * r;                    // L[lane][k] (lanes above k: unused values)
+        if (drop) l = lane == k ? d * r : 0.0f;  // sqrt(floor) on the diagonal, nothing below it
         row[k] = l;
         s[k] *= r;                               // x[k] = s[k] / L[k][k]
         const float xk = s[k];
@@ -108,7 +122,17 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
 #pragma unroll
     for (int c = 0; c < NB; c += 4)              // U^-1[lane][c] = L^-1[c][lane] = s[c] of this lane (zero for c < lane)
         *reinterpret_cast<float4 *>(I + c) = make_float4(s[c], s[c + 1], s[c + 2], s[c + 3]);
-    if (!ok && lane == 0) info[b] = 1;
+    if (panel_inv != nullptr) {
+        float *P = panel_inv + (long long)b * inv_stride + (long long)lane * ldi;
+#pragma unroll
+        for (int c = 0; c < NB; c += 4) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = (dropped >> (c + e)) & 1ull ? 0.0f : s[c + e];
+            *reinterpret_cast<float4 *>(P + c) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+    }
+    if ((!ok || dropped != 0) && lane == 0) info[b] |= (ok ? 0 : 1) | (dropped != 0 ? 2 : 0);
 }
 
 // How far a stack of Gram matrices is from the identity: per matrix max |G - I| and ||G - I||_F^2, in
@@ -174,6 +198,48 @@ __global__ __launch_bounds__(256) void copy_flagged_kernel(float *dst, const flo
     for (long long q = blockIdx.x * 256ll + threadIdx.x; q < quads; q += (long long)gridDim.x * 256) d[q] = s[q];
 }
 
+// One 64-column panel of every matrix of a stack: each column is scaled to unit length; with `fill` given, a
+// column whose squared length is below null_norm2 (what projecting out the earlier columns has left of a
+// unit column: rounding noise) is replaced by the same column of `fill` (unit columns in general position)
+// and bit 2 of info[b] is set.  The panel is n x 64 with leading dimension ld.  Two launches over
+// (kNormChunks row chunks, batch): squared lengths per chunk into partial [batch][kNormChunks][64], then
+// every chunk adds them up in the same order and rescales (or replaces) its rows.
+constexpr int kNormChunks = 8;
+
+__global__ __launch_bounds__(256) void panel_norms_kernel(const float *panel, long long stride, int ld, int n, float *partial) {
+    const int chunk = blockIdx.x, b = blockIdx.y, c = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const float *P = panel + (long long)b * stride;
+    const int rows = (n + kNormChunks - 1) / kNormChunks, r0 = chunk * rows, r1 = min(r0 + rows, n);
+    float sum = 0.0f;
+    for (int r = r0 + g; r < r1; r += 4) {
+        const float v = P[(long long)r * ld + c];
+        sum = __builtin_fmaf(v, v, sum);
+    }
+    __shared__ float part[4][64];
+    part[g][c] = sum;
+    __syncthreads();
+    if (g == 0) partial[((long long)b * kNormChunks + chunk) * 64 + c] = (part[0][c] + part[1][c]) + (part[2][c] + part[3][c]);
+}
+
+__global__ __launch_bounds__(256) void panel_rescale_kernel(float *panel, long long stride, int ld, int n, const float *partial,
+                                                            const float *fill, int fill_ld, float null_norm2, int *info) {
+    const int chunk = blockIdx.x, b = blockIdx.y, c = threadIdx.x & 63, g = threadIdx.x >> 6;
+    float *P = panel + (long long)b * stride;
+    float norm2 = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kNormChunks; ++k) norm2 += partial[((long long)b * kNormChunks + k) * 64 + c];
+    const int rows = (n + kNormChunks - 1) / kNormChunks, r0 = chunk * rows, r1 = min(r0 + rows, n);
+    const bool replace = fill != nullptr && !(norm2 >= null_norm2);          // (a NaN column is replaced as well)
+    if (replace) {
+        for (int r = r0 + g; r < r1; r += 4) P[(long long)r * ld + c] = fill[(long long)r * fill_ld + c];
+        if (g == 0 && chunk == 0) atomicOr(info + b, 4);
+    } else if (norm2 > 0.0f) {
+        float scale = __builtin_amdgcn_rsqf(norm2);
+        scale = scale * __builtin_fmaf(-0.5f * norm2 * scale, scale, 1.5f);
+        for (int r = r0 + g; r < r1; r += 4) P[(long long)r * ld + c] *= scale;
+    }
+}
+
 qtensor_batch_ptr strided(const float *base, long long stride) {
     qtensor_batch_ptr p;
     p.base = base;
@@ -201,9 +267,15 @@ bool stack_args_ok(const char *what, int n, int batch, std::initializer_list<con
 }  // namespace qt
 
 extern "C" void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float *x, int *info, int n, int batch, void *stream_v) {
+    qtensor_hip_cholesky_upper_floor_batched(gram, u, x, info, n, batch, 0.0f, stream_v);
+}
+
+extern "C" void qtensor_hip_cholesky_upper_floor_batched(float *gram, float *u, float *x, int *info, int n, int batch,
+                                                         float pivot_floor, void *stream_v) {
     using namespace qt;
     clear_error();
     if (!stack_args_ok("cholesky_upper_batched", n, batch, {gram, u, x, info})) return;
+    if (!(pivot_floor >= 0.0f)) { set_error(kBadArgument, "cholesky_upper_batched: the pivot floor must not be negative"); return; }
     hipStream_t stream = (hipStream_t)stream_v;
     const long long mat = (long long)n * n;
     // Two levels of blocking: inside a panel of kFactorPanel rows the 64-row steps update only the rest of
@@ -214,16 +286,18 @@ extern "C" void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float 
         for (int j0 = p0; j0 < p1; j0 += NB) {
             const int j1 = j0 + NB, rest = n - j1;
             const long long corner = (long long)j0 * n + j0;
+            // (the block of u right below the diagonal block is free: it takes the factor for the block row)
+            float *panel_inv = rest > 0 ? u + (long long)j1 * n + j0 : nullptr;
             hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram + corner, mat, n, u + corner, mat, n,
-                               x + corner, mat, n, info);
+                               x + corner, mat, n, panel_inv, info, pivot_floor);
             if (!launch_ok("cholesky_upper_batched (diagonal block)")) return;
             if (rest == 0) break;
             const long long row = (long long)j0 * n + j1;
             qtensor_gemm_desc d = {};
-            // U_j,> = U_jj^-T G_j,>
+            // U_j,> = U_jj^-T G_j,>  (zero rows for columns taken out of the factorisation)
             d.M = NB; d.N = rest; d.K = NB; d.batch = batch;
             d.kind_a = QTENSOR_DENSE_T; d.kind_b = QTENSOR_DENSE; d.epilogue = QTENSOR_EPI_STORE;
-            d.args.A = strided(x + corner, mat); d.args.lda = n;
+            d.args.A = strided(panel_inv, mat); d.args.lda = n;
             d.args.B = strided(gram + row, mat); d.args.ldb = n;
             d.args.C = strided(u + row, mat); d.args.ldc = n;
             if (!run(d, stream)) return;
@@ -255,6 +329,122 @@ extern "C" void qtensor_hip_cholesky_upper_batched(float *gram, float *u, float 
             t.args.alpha = -1.0f; t.args.beta = 1.0f;
             t.args.symmetric = 1;
             if (!run(t, stream)) return;
+        }
+    }
+}
+
+namespace qt {
+namespace {
+
+// State of one block Gram-Schmidt sweep over a stack (see qtensor_hip_block_gram_schmidt_batched).
+struct Sweep {
+    float *q, *w, *gram, *u, *x;
+    const float *fill;
+    int *info;
+    int n, batch, w_cols;
+    float pivot_floor, null_norm2;
+    hipStream_t stream;
+    long long mat() const { return (long long)n * n; }
+
+    // columns [c0, c0 + width) -= Q[:, a0:c0] (Q[:, a0:c0]^T columns): the columns a0..c0 are orthonormal
+    bool project(int a0, int c0, int width) {
+        const int k = c0 - a0;
+        if (k <= 0) return true;
+        const long long w_stride = (long long)n * w_cols;
+        qtensor_gemm_desc p = {};                             // W = Q_a^T Y
+        p.M = k; p.N = width; p.K = n; p.batch = batch;
+        p.kind_a = QTENSOR_DENSE_T; p.kind_b = QTENSOR_DENSE; p.epilogue = QTENSOR_EPI_STORE;
+        p.args.A = strided(q + a0, mat()); p.args.lda = n;
+        p.args.B = strided(q + c0, mat()); p.args.ldb = n;
+        p.args.C = strided(w, w_stride); p.args.ldc = width;
+        if (!run(p, stream)) return false;
+        qtensor_gemm_desc r = {};                             // Y -= Q_a W
+        r.M = n; r.N = width; r.K = k; r.batch = batch;
+        r.kind_a = QTENSOR_DENSE; r.kind_b = QTENSOR_DENSE; r.epilogue = QTENSOR_EPI_AXPBY_DENSE;
+        r.args.A = strided(q + a0, mat()); r.args.lda = n;
+        r.args.B = strided(w, w_stride); r.args.ldb = width;
+        r.args.C = strided(q + c0, mat()); r.args.ldc = n;
+        r.args.E = strided(q + c0, mat()); r.args.lde = n;
+        r.args.alpha = -1.0f; r.args.beta = 1.0f;
+        return run(r, stream);
+    }
+
+    // The 64 columns from c0 on: `passes` times { take the columns a0..c0 out, unit columns, Cholesky QR rounds
+    // inside (two the first time, one afterwards) }.
+    bool panel(int a0, int c0, int passes, int first_rounds, bool may_fill) {
+        float *panel_ptr = q + c0;
+        const long long small = (long long)NB * NB;
+        float *norms = u;                                     // [batch][kNormChunks][64]: u is free between factorisations
+        for (int pass = 0; pass < passes; ++pass) {
+            if (!project(a0, c0, NB)) return false;
+            hipLaunchKernelGGL(panel_norms_kernel, dim3(kNormChunks, batch), dim3(256), 0, stream, panel_ptr, mat(), n, n, norms);
+            hipLaunchKernelGGL(panel_rescale_kernel, dim3(kNormChunks, batch), dim3(256), 0, stream, panel_ptr, mat(), n, n, norms,
+                               may_fill && pass == 0 && fill != nullptr ? fill + c0 : nullptr, n, null_norm2, info);
+            if (!launch_ok("block_gram_schmidt_batched (normalize)")) return false;
+            const int rounds = pass == 0 ? first_rounds : 1;
+            for (int round = 0; round < rounds; ++round) {
+                qtensor_gemm_desc g = {};                     // S = Y_p^T Y_p
+                g.M = NB; g.N = NB; g.K = n; g.batch = batch;
+                g.kind_a = QTENSOR_DENSE_T; g.kind_b = QTENSOR_DENSE; g.epilogue = QTENSOR_EPI_STORE;
+                g.args.A = strided(panel_ptr, mat()); g.args.lda = n;
+                g.args.B = strided(panel_ptr, mat()); g.args.ldb = n;
+                g.args.C = strided(gram, small); g.args.ldc = NB;
+                g.args.workspace = w;                         // one tile per matrix and a long k range: cut along k
+                g.args.workspace_floats = (long long)batch * n * w_cols;
+                if (!run(g, stream)) return false;
+                hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram, small, NB, u, small, NB, x, small, NB,
+                                   (float *)nullptr, info, pivot_floor);
+                if (!launch_ok("block_gram_schmidt_batched (panel factor)")) return false;
+                qtensor_gemm_desc t = {};                     // Y_p <- Y_p U^-1 (one tile column: in place is safe)
+                t.M = n; t.N = NB; t.K = NB; t.batch = batch;
+                t.kind_a = QTENSOR_DENSE; t.kind_b = QTENSOR_DENSE; t.epilogue = QTENSOR_EPI_STORE;
+                t.args.A = strided(panel_ptr, mat()); t.args.lda = n;
+                t.args.B = strided(x, small); t.args.ldb = NB;
+                t.args.C = strided(panel_ptr, mat()); t.args.ldc = n;
+                t.args.triangular = 2;
+                if (!run(t, stream)) return false;
+            }
+        }
+        return true;
+    }
+};
+
+}  // namespace
+}  // namespace qt
+
+extern "C" int qtensor_hip_block_gram_schmidt_width(void) {
+    // QT_BGS_PANEL (a tuning knob): another width of the outer panels, a multiple of 64
+    static const int width = [] {
+        const char *env = getenv("QT_BGS_PANEL");
+        const int asked = env != nullptr ? atoi(env) : 0;
+        return asked >= qt::NB && asked % qt::NB == 0 && asked <= 1024 ? asked : 128;
+    }();
+    return width;
+}
+
+extern "C" void qtensor_hip_block_gram_schmidt_batched(float *q, float *w, float *gram, float *u, float *x, const float *fill,
+                                                       int *info, int n, int batch, float pivot_floor, float null_norm2,
+                                                       void *stream_v) {
+    using namespace qt;
+    clear_error();
+    if (!stack_args_ok("block_gram_schmidt_batched", n, batch, {q, w, gram, u, x, info})) return;
+    if (!(pivot_floor >= 0.0f) || !(null_norm2 >= 0.0f)) { set_error(kBadArgument, "block_gram_schmidt_batched: negative threshold"); return; }
+    const int outer = qtensor_hip_block_gram_schmidt_width();
+    Sweep s = {q, w, gram, u, x, fill, info, n, batch, outer, pivot_floor, null_norm2, (hipStream_t)stream_v};
+    // Two levels.  An outer panel of `outer` columns has the finished columns taken out of it as a whole (the
+    // bulk of the arithmetic, as products with a wide right-hand side) and is then swept inside -- every
+    // 64-column panel: take the earlier panels of the same outer panel out, unit columns, one Cholesky QR
+    // round -- and all of that is done twice.  The second pass acts on a panel that is orthonormal up to what
+    // the rounding of the first one left, so nothing amplifies its own rounding: the panel ends orthonormal,
+    // and orthogonal to the earlier columns, to fp32 rounding whatever the conditioning of the matrix (block
+    // classical Gram-Schmidt with reorthogonalisation; the Cholesky QR inside a 64-column panel sees at most
+    // that panel's own conditioning, and its pivot floor takes care of columns that depend on each other).
+    for (int o0 = 0; o0 < n; o0 += outer) {
+        const int width = n - o0 < outer ? n - o0 : outer;
+        for (int pass = 0; pass < 2; ++pass) {
+            if (!s.project(0, o0, width)) return;
+            for (int c0 = o0; c0 < o0 + width; c0 += NB)
+                if (!s.panel(o0, c0, 1, 1, pass == 0)) return;
         }
     }
 }

@@ -14,11 +14,12 @@ of subspace iteration per matrix (shampoo2.py:185-200, utils.py:156-203):
 Here all statistics of one order form a stack and every line above is one or two launches for
 the whole stack: the products run on the matrix cores through qtensor.fused.gemm (symmetric
 ones compute half and mirror), and the QR factorisation -- 20 ms per 1024 x 1024 matrix through
-the vendor's Householder routine, 5 s per step for a ViT-B/32 -- is replaced by a shifted
-Cholesky QR (rounds of  G = Q^T Q,  U = chol(G + s I),  Q <- Q U^-1  on the column-scaled
-matrix until Q is orthonormal; the factorisation and the solve are blocked, batched launches of
-libqtensor_hip.so), which yields the same factor Q up to column signs.  Matrices it cannot
-finish are redone with torch.linalg.qr.
+the vendor's Householder routine, 5 s per step for a ViT-B/32 -- is replaced by one sweep of
+block Gram-Schmidt with reorthogonalisation per stack (panels of the column-scaled matrix left to
+right; the products run on the matrix cores, the 64-column panels are orthonormalised by Cholesky
+QR; batched launches of libqtensor_hip.so), checked afterwards and polished by a Cholesky QR round
+where needed, which yields the same factor Q up to column signs.  Matrices that cannot be
+finished this way are redone with torch.linalg.qr.
 """
 import torch
 

@@ -324,9 +324,13 @@ def dequantize_stack(q: Quantized, out: Optional[Tensor] = None, outdtype=torch.
 
 # --------------------------------------------------------------------------- Cholesky QR pieces
 if F.lib is not None:
-    F.lib.qtensor_hip_cholesky_upper_batched.restype = None
-    F.lib.qtensor_hip_cholesky_upper_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int,
-                                                         ct.c_void_p]
+    F.lib.qtensor_hip_cholesky_upper_floor_batched.restype = None
+    F.lib.qtensor_hip_cholesky_upper_floor_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int,
+                                                               ct.c_int, ct.c_float, ct.c_void_p]
+    F.lib.qtensor_hip_block_gram_schmidt_width.restype = ct.c_int
+    F.lib.qtensor_hip_block_gram_schmidt_width.argtypes = []
+    F.lib.qtensor_hip_block_gram_schmidt_batched.restype = None
+    F.lib.qtensor_hip_block_gram_schmidt_batched.argtypes = [ct.c_void_p] * 7 + [ct.c_int, ct.c_int, ct.c_float, ct.c_float, ct.c_void_p]
     F.lib.qtensor_hip_gram_deviation_batched.restype = None
     F.lib.qtensor_hip_gram_deviation_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
     F.lib.qtensor_hip_copy_flagged_batched.restype = None
@@ -342,15 +346,52 @@ def _stack(t: Tensor, name: str, shape=None) -> Tensor:
     return t
 
 
-def cholesky_upper(gram: Tensor, u: Tensor, x: Tensor, info: Tensor) -> None:
+def cholesky_upper(gram: Tensor, u: Tensor, x: Tensor, info: Tensor, pivot_floor: float = 0.0) -> None:
     """gram [B, n, n] (destroyed) = U^T U: block rows of U into u, inverses of its 64 x 64 diagonal blocks
     into the diagonal blocks of x [B, n, n] (nothing else of x is written); info int32 [B] (zeroed by the
-    caller) flags non-positive pivots."""
+    caller): bit 0 = a non-positive or NaN pivot (factor meaningless), bit 1 = a pivot at or below
+    pivot_floor > 0 was raised to it (with pivot_floor = 0 such a pivot sets bit 0)."""
     B, n, _ = gram.shape
     _stack(gram, "gram", (B, n, n)), _stack(u, "u", (B, n, n)), _stack(x, "x", (B, n, n))
     if info.dtype != torch.int32 or info.numel() != B or not info.is_cuda:
         raise ValueError("info must be an int32 GPU vector with one entry per matrix")
-    F._call(F.lib.qtensor_hip_cholesky_upper_batched, gram.device, gram.data_ptr(), u.data_ptr(), x.data_ptr(), info.data_ptr(), n, B)
+    F._call(F.lib.qtensor_hip_cholesky_upper_floor_batched, gram.device, gram.data_ptr(), u.data_ptr(), x.data_ptr(), info.data_ptr(),
+            n, B, float(pivot_floor))
+
+
+_COMPLETION = {}                 # (device index, order) -> fixed matrix of unit columns that stand in for null directions
+NULL_COLUMN_NORM2 = 1e-11        # what a projection leaves of a unit column that depends on the earlier ones: rounding noise
+
+
+def completion_columns(device: torch.device, n: int) -> Tensor:
+    """[n, n] fixed pseudo-random unit columns (the same for every call): stand-ins for the columns of a
+    rank-deficient matrix that are rounding noise once the columns before them are taken out."""
+    key = (device.index, n)
+    if key not in _COMPLETION:
+        gen = torch.Generator(device=device).manual_seed(0x5eed + n)
+        r = torch.randn(n, n, device=device, generator=gen)
+        _COMPLETION[key] = (r / torch.linalg.vector_norm(r, dim=0, keepdim=True)).contiguous()
+    return _COMPLETION[key]
+
+
+def block_gram_schmidt(q: Tensor, info: Tensor, pivot_floor: float = 2e-4, null_norm2: float = NULL_COLUMN_NORM2,
+                       complete: bool = True) -> Tensor:
+    """Orthonormalise the columns of every matrix of the stack q [B, n, n] (unit columns, n a multiple of 64)
+    in place, left to right in panels of 64 columns: block Gram-Schmidt with reorthogonalisation, Cholesky QR
+    inside a panel.  span(q[:, :, :k]) is kept for every k.  complete: columns that depend on the earlier ones
+    up to rounding noise are replaced by fixed unit columns in general position (bit 2 of info[b]); info int32
+    [B], zeroed by the caller, bits as in cholesky_upper."""
+    B, n, _ = q.shape
+    _stack(q, "q", (B, n, n))
+    if info.dtype != torch.int32 or info.numel() != B or not info.is_cuda:
+        raise ValueError("info must be an int32 GPU vector with one entry per matrix")
+    w = torch.empty(B, n, F.lib.qtensor_hip_block_gram_schmidt_width(), device=q.device)
+    small = torch.empty(3, B, 64, 64, device=q.device)
+    fill = completion_columns(q.device, n) if complete else None
+    F._call(F.lib.qtensor_hip_block_gram_schmidt_batched, q.device, q.data_ptr(), w.data_ptr(), small[0].data_ptr(),
+            small[1].data_ptr(), small[2].data_ptr(), None if fill is None else fill.data_ptr(), info.data_ptr(), n, B,
+            float(pivot_floor), float(null_norm2))
+    return q
 
 
 def gram_deviation(gram: Tensor) -> Tensor:
@@ -390,20 +431,33 @@ def solve_upper_right(q: Tensor, u: Tensor, x: Tensor, work: Tensor, out: Tensor
 
 
 _householder_qr = torch.linalg.qr
+PIVOT_FLOOR = 2e-4               # a hundred times the rounding error of an fp32 Gram matrix of unit columns
 
 
 class CholeskyQR:
     """Orthonormal Q [B, n, n] with span(Q[:, :, :k]) == span(Y[:, :, :k]) for every k (the Q factor
-    of a QR factorisation with positive diagonal of R), by rounds of  G = Q^T Q,  U = chol(G + s I),
-    Q <- Q U^-1  on the column-scaled matrix; every U is upper triangular, so the nested spans
-    survive each round.  A matrix far from orthonormal (||G - I||_F >= 0.5) gets the shift s (a few
-    times the rounding error of an fp32 Gram matrix of unit columns, so that G + s I stays positive
-    definite), which lifts its small singular values by 1 / sqrt(s) per round -- a numerically singular Y ends, like
-    with Householder reflections, in a completion fixed by rounding noise.  Once ||G - I||_F < 0.5
-    (all singular values of Q within [0.7, 1.23]) one unshifted round makes Q orthonormal to fp32
-    rounding and the matrix leaves the working set; matrices that still are far after max_rounds, or
-    whose factorisation hits a non-positive pivot, go through torch.linalg.qr.  Orders that are not
-    a multiple of 64 are padded with an identity block (QR of diag(Y, I) is diag(Q, I)).
+    of a QR factorisation with positive diagonal of R) for a whole stack.
+
+    The work is done by one sweep of block Gram-Schmidt with reorthogonalisation over the column-scaled
+    matrix (block_gram_schmidt: panels left to right, every panel has the finished columns taken out of it
+    twice and is orthonormalised inside by Cholesky QR), which loses orthogonality only in proportion to
+    fp32 rounding whatever the conditioning of Y.  What follows is a safety net of Cholesky QR rounds on the
+    whole matrix --  G = Q^T Q,  U = chol(G),  Q <- Q U^-1,  every U upper triangular, so the nested spans
+    survive -- for the few matrices the test after the sweep does not find orthonormal (typically a
+    rank-deficient one whose last panel of stand-in columns is a little off): one round each.
+
+    Rank-deficient Y (a statistic of order 768 fed by a 768 x 256 gradient block has rank 256 plus whatever
+    its kept eigenpairs add): a column that depends on the ones before it is rounding noise once those are
+    taken out, and the Q column it leads to is noise in any QR algorithm (Householder's included).  The
+    sweep replaces such a column (shorter than sqrt(1e-11) after the first projection of a unit column) by a
+    fixed unit column in general position, which is then orthogonalised like any other; columns with a real
+    independent part, however small, are kept.  Inside the factorisations a pivot that is not above
+    PIVOT_FLOOR takes its column out of that factorisation (cholesky_upper) instead of failing it.
+
+    Once ||G - I||_F < 0.5 one Cholesky QR round makes Q orthonormal to fp32 rounding and the matrix leaves
+    the working set without a further test; matrices that still are far after max_rounds, or whose
+    factorisation meets a NaN, go through torch.linalg.qr.  Orders that are not a multiple of 64 are padded
+    with an identity block (QR of diag(Y, I) is diag(Q, I)).
 
     The object is a small state machine so that several stacks can advance on their own streams while
     the host waits only once per round for all of them:  check() enqueues the orthonormality test,
@@ -411,7 +465,7 @@ class CholeskyQR:
     matrices still in the working set, result() returns (Q, number of matrices redone by the
     library).  All calls for one object must be made with the same current stream."""
 
-    def __init__(self, Y, max_rounds=12, shift=2e-4, tolerance=2e-5):
+    def __init__(self, Y, max_rounds=12, pivot_floor=PIVOT_FLOOR, tolerance=2e-5, sweep=True):
         if Y.dim() != 3 or Y.shape[1] != Y.shape[2] or Y.dtype != torch.float32 or not Y.is_cuda:
             raise ValueError("CholeskyQR takes an fp32 GPU stack [B, n, n]")
         B, self.true_n, _ = Y.shape
@@ -421,7 +475,7 @@ class CholeskyQR:
             padded[:, :self.true_n, :self.true_n] = Y
             padded.diagonal(dim1=1, dim2=2)[:, self.true_n:] = 1.0
             Y = padded
-        self.Y, self.shift, self.tolerance, self.rounds_left = Y, shift, tolerance, max_rounds
+        self.Y, self.pivot_floor, self.tolerance, self.rounds_left = Y, pivot_floor, tolerance, max_rounds
         scale = torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)
         self.Q = (Y / scale).contiguous()             # working set; unit columns: the Gram matrix has a unit diagonal
         self.U = torch.empty_like(self.Q)
@@ -433,12 +487,15 @@ class CholeskyQR:
         self.rounds = 0                               # factorisation rounds enqueued so far
         self.gram = self.far = None
         # The bookkeeping lives on the host (it waits once per round anyway), per working-set entry:
-        # which matrix of the stack it is, whether it is within ||G - I||_F < 0.5, and whether a factorisation
-        # WITHOUT the shift hit a non-positive pivot (it kept its Q and gets the shift from now on).
+        # which matrix of the stack it is and whether it is within ||G - I||_F < 0.5.
         self.ids = np.arange(B)
         self.near = np.zeros(B, dtype=bool)
-        self.needs_shift = np.zeros(B, dtype=bool)
-        self.last = None                              # (pivot flags, shifted, near, ids) of the round not yet looked at
+        self.last = None                              # (pivot flags, near, ids) of the round not yet looked at
+        if sweep:
+            # one sweep of block Gram-Schmidt with reorthogonalisation leaves all but pathological matrices
+            # orthonormal to rounding: the rounds below then only confirm it (one test, no factorisation)
+            block_gram_schmidt(self.Q, self.info, pivot_floor)
+            self.info.zero_()
 
     def _index(self, positions):
         return torch.as_tensor(np.ascontiguousarray(positions), dtype=torch.int64).to(self.Q.device)
@@ -463,26 +520,25 @@ class CholeskyQR:
         self.Q = self.Q.index_select(0, index)
         if self.gram is not None:
             self.gram = self.gram.index_select(0, index)
-        self.ids, self.near, self.needs_shift = self.ids[keep], self.near[keep], self.needs_shift[keep]
+        self.ids, self.near = self.ids[keep], self.near[keep]
 
     def check(self):
         self.gram = gemm(self.Q, self.Q, trans_a=True, symmetric=True)
         self.far = gram_deviation(self.gram)                                    # max |G - I|, ||G - I||_F^2
 
+    def _failures(self):
+        """Host mask over the entries of the last round: the factorisation met a NaN."""
+        info, near, ids = self.last
+        self.last = None
+        return (info.cpu().numpy()[:ids.size] & 1) != 0, near, ids
+
     def poll(self):
         far = self.far.cpu().numpy()                                            # the host synchronisation
-        k = self.ids.size
-        failed = np.zeros(k, dtype=bool)
+        failed = np.zeros(self.ids.size, dtype=bool)
         if self.last is not None:
-            # pivot flags of the previous round: a failure with the shift (or of a matrix that was already close:
-            # it has been finalised, wrongly) is hopeless and goes to the library; one without the shift keeps its Q
-            info, shifted, near, ids = self.last
-            bad = info.cpu().numpy()[:shifted.size] != 0
-            self.redo += ids[bad & near].tolist()
-            bad, shifted = bad[~near], shifted[~near]                           # the entries still in the working set
-            failed |= bad & shifted
-            self.needs_shift |= bad
-            self.last = None
+            bad, near, ids = self._failures()
+            self.redo += ids[bad & near].tolist()                               # (already finalised, wrongly)
+            failed |= bad[~near]                                                # the entries still in the working set
         with np.errstate(invalid="ignore"):
             done = far[:, 0] < self.tolerance                                   # False for NaN as well
             self.near = far[:, 1] < 0.25
@@ -497,35 +553,26 @@ class CholeskyQR:
 
     def advance(self):
         k = self.ids.size
-        # The first round is tried without the shift: for condition numbers up to about 1e3 that saves a
-        # round, and a matrix for which it fails (non-positive pivot) simply keeps its Q and joins the
-        # shifted rounds.
-        shifted = ~self.near & (self.needs_shift if self.rounds == 0 else True)
-        if shifted.any():
-            add = torch.as_tensor(np.where(shifted, self.shift, 0.0).astype(np.float32)).to(self.Q.device)
-            self.gram.diagonal(dim1=1, dim2=2).add_(add.unsqueeze(1))
         info = self.info[:k]
         info.zero_()
-        cholesky_upper(self.gram, self.U[:k], self.X[:k], info)
+        cholesky_upper(self.gram, self.U[:k], self.X[:k], info, self.pivot_floor)
         out = torch.empty_like(self.Q)
         solve_upper_right(self.Q, self.U[:k], self.X[:k], self.gram, out)      # the Gram matrix is used up: scratch
-        copy_flagged(out, self.Q, info)                                         # a failed matrix keeps its iterate
         self.Q, self.gram = out, None
-        self.last = (info, shifted, self.near.copy(), self.ids.copy())
+        self.last = (info, self.near.copy(), self.ids.copy())
         self.rounds_left -= 1
         self.rounds += 1
         if self.near.any():
-            # ||G - I||_F < 0.5 before an unshifted round: G was positive definite with eigenvalues in
-            # (0.5, 1.5), the round leaves Q orthonormal to rounding
+            # ||G - I||_F < 0.5 before the round: G was positive definite with eigenvalues in (0.5, 1.5),
+            # no pivot came near the floor and the round leaves Q orthonormal to rounding
             self._finish(np.nonzero(self.near)[0], self.Q)
             self._keep(~self.near)
             self.finished = self.ids.size == 0
 
     def result(self):
         if self.last is not None:                     # pivot flags of the last round
-            info, shifted, near, ids = self.last
-            self.redo += ids[(info.cpu().numpy()[:shifted.size] != 0) & near].tolist()
-            self.last = None
+            bad, near, ids = self._failures()
+            self.redo += ids[bad & near].tolist()
         if self.final is None:
             self.final = torch.empty_like(self.Y)
         if self.redo:
@@ -539,9 +586,9 @@ class CholeskyQR:
         return Q, len(set(self.redo))
 
 
-def cholesky_qr(Y, max_rounds=12, shift=2e-4, tolerance=2e-5):
+def cholesky_qr(Y, max_rounds=12, pivot_floor=PIVOT_FLOOR, tolerance=2e-5):
     """(Q, number of matrices redone by the library) for one stack; see CholeskyQR."""
-    state = CholeskyQR(Y, max_rounds, shift, tolerance)
+    state = CholeskyQR(Y, max_rounds, pivot_floor, tolerance)
     while not state.finished:
         state.check()
         if not state.poll():

@@ -129,11 +129,97 @@ def test_cholesky_qr_gives_the_householder_factor_up_to_signs(mods):
     Qh, Rh = torch.linalg.qr(Y.double().cpu())
     Qh = Qh * torch.sign(torch.diagonal(Rh, dim1=1, dim2=2)).unsqueeze(1)
     assert redone == 0 and Q.shape == (3, 100, 100) and rel(Q, Qh) <= 1e-4
-    # a matrix with a zero column cannot be factorised this way: it is sent to the library routine
+    # a zero column depends on the columns before it in the plainest way: it gets a stand-in, the columns
+    # before it are what Householder reflections give, and the whole is orthonormal
     Y = torch.randn(2, n, n, generator=g).cuda()
     Y[1, :, 5] = 0.0
     Q, redone = E2.cholesky_qr(Y)
-    assert redone == 1 and float((Q.transpose(1, 2) @ Q - torch.eye(n, device="cuda")).abs().max()) < 1e-4
+    assert redone == 0 and float((Q.transpose(1, 2) @ Q - torch.eye(n, device="cuda")).abs().max()) < 1e-4
+    Qh, Rh = torch.linalg.qr(Y[1].double().cpu())
+    Qh = Qh * torch.sign(torch.diagonal(Rh)).unsqueeze(0)
+    assert rel(Q[1][:, :5], Qh[:, :5]) <= 1e-5
+
+
+@pytest.mark.parametrize("n,batch,cond", [(64, 3, 1e2), (192, 4, 1e4), (320, 2, 1e1), (768, 3, 1e5), (1024, 2, 1e3)])
+def test_block_gram_schmidt_sweep_against_float64_householder(mods, n, batch, cond):
+    """One sweep of qtensor_hip_block_gram_schmidt_batched: orthonormal to fp32 rounding whatever the conditioning,
+    nested spans kept (R = Q^T Y upper triangular with a positive diagonal), the Householder factor up to what
+    the pivots allow."""
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(n)
+    U, _ = torch.linalg.qr(torch.randn(batch, n, n, generator=g))
+    V, _ = torch.linalg.qr(torch.randn(batch, n, n, generator=g))
+    lam = torch.logspace(0, -torch.log10(torch.tensor(cond)).item(), n)
+    Y = ((U * lam) @ V.transpose(1, 2))
+    Y = (Y / torch.linalg.vector_norm(Y, dim=1, keepdim=True)).cuda().contiguous()      # unit columns, as the caller provides
+    Q = Y.clone()
+    info = torch.zeros(batch, dtype=torch.int32, device="cuda")
+    X.block_gram_schmidt(Q, info)
+    assert info.tolist() == [0] * batch                        # no pivot near the floor, nothing replaced
+    eye = torch.eye(n, device="cuda")
+    assert float((Q.transpose(1, 2) @ Q - eye).abs().max()) < 2e-5
+    R = (Q.transpose(1, 2).double() @ Y.double()).cpu()
+    assert float(torch.tril(R, -1).abs().max()) < 2e-5 and bool((torch.diagonal(R, dim1=1, dim2=2) > 0).all())
+    Qh, Rh = torch.linalg.qr(Y.double().cpu())
+    Qh = Qh * torch.sign(torch.diagonal(Rh, dim1=1, dim2=2)).unsqueeze(1)
+    # a column is determined to (fp32 rounding / its pivot): Gram-Schmidt with reorthogonalisation reaches that,
+    # where repeated Cholesky QR of the whole matrix only reached (rounding of the Gram matrix / pivot)
+    weighted = (Q.double().cpu() - Qh).norm(dim=1) * torch.diagonal(Rh, dim1=1, dim2=2).abs()
+    assert float(weighted.max()) < 5e-6, float(weighted.max())
+
+
+def test_rank_deficient_stacks_get_a_completed_basis(mods):
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(17)
+    n, r = 256, 96
+    A = torch.randn(2, n, r, generator=g)
+    Y = (A @ torch.randn(2, r, n, generator=g))                 # rank 96: columns 96.. depend on the first 96
+    Y[1] = torch.randn(n, n, generator=g)                       # the second matrix is regular
+    Y = (Y / torch.linalg.vector_norm(Y, dim=1, keepdim=True)).cuda().contiguous()
+    Q, redone = X.cholesky_qr(Y)
+    assert redone == 0
+    assert float((Q.transpose(1, 2) @ Q - torch.eye(n, device="cuda")).abs().max()) < 1e-4
+    Qh, Rh = torch.linalg.qr(Y.double().cpu())
+    Qh = Qh * torch.sign(torch.diagonal(Rh, dim1=1, dim2=2)).unsqueeze(1)
+    assert rel(Q[0][:, :r - 8], Qh[0][:, :r - 8]) <= 1e-4       # (the last few independent columns have small pivots)
+    assert rel(Q[1], Qh[1]) <= 1e-3
+    # the first 96 columns span the range of Y[0]: every column of Y[0] lies in it
+    lead = Q[0][:, :r].double().cpu()
+    resid = Y[0].double().cpu() - lead @ (lead.T @ Y[0].double().cpu())
+    assert float(resid.norm(dim=0).max()) < 1e-5
+    # the sweep alone: bit 2 of info marks the matrix whose noise columns were replaced, and only that one
+    Q2 = Y.clone()
+    info = torch.zeros(2, dtype=torch.int32, device="cuda")
+    X.block_gram_schmidt(Q2, info)
+    assert (info[0].item() & 4) != 0 and (info[1].item() & 4) == 0
+    # without stand-ins the noise columns stay noise: the sweep then leaves the matrix far from orthonormal
+    Q3 = Y.clone()
+    info.zero_()
+    X.block_gram_schmidt(Q3, info, complete=False)
+    assert (info[0].item() & 4) == 0
+    assert float((Q3[1].T @ Q3[1] - torch.eye(n, device="cuda")).abs().max()) < 2e-5
+
+
+def test_pivot_floor_takes_a_dependent_column_out_of_the_factorisation(mods):
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(23)
+    n = 128
+    A = torch.randn(n, n, generator=g, dtype=torch.float64)
+    A[:, 70] = A[:, :70] @ torch.randn(70, generator=g, dtype=torch.float64)           # column 70 depends on the ones before
+    A = A / A.norm(dim=0, keepdim=True)
+    G = (A.T @ A).float().cuda().unsqueeze(0).contiguous()
+    U, inv = torch.zeros(1, n, n, device="cuda"), torch.zeros(1, n, n, device="cuda")
+    info = torch.zeros(1, dtype=torch.int32, device="cuda")
+    X.cholesky_upper(G.clone(), U, inv, info, pivot_floor=2e-4)
+    assert info.item() == 2
+    Ut = torch.triu(U[0]).cpu()
+    assert abs(float(Ut[70, 70]) - 2e-4 ** 0.5) < 1e-6 and float(Ut[70, 71:].abs().max()) == 0.0
+    keep = [j for j in range(n) if j != 70]
+    want = torch.linalg.cholesky((A[:, keep].T @ A[:, keep]), upper=True)              # the factor without that column
+    assert rel(Ut[keep][:, keep], want) <= 1e-4
+    info.zero_()
+    X.cholesky_upper(G.clone(), U, inv, info)                                          # no floor: flagged as failed (or barely positive)
+    assert info.item() in (0, 1)
 
 
 def run_both(S2, E2, code_maps, mode, same_qr, monkeypatch, steps=3):
