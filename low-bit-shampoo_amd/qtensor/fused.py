@@ -478,8 +478,7 @@ class CholeskyQR:
         self.Y, self.pivot_floor, self.tolerance, self.rounds_left = Y, pivot_floor, tolerance, max_rounds
         scale = torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)
         self.Q = (Y / scale).contiguous()             # working set; unit columns: the Gram matrix has a unit diagonal
-        self.U = torch.empty_like(self.Q)
-        self.X = torch.zeros_like(self.Q)             # inverse factors; the part below the diagonal blocks stays zero
+        self.U = self.X = None                        # factors of the polishing rounds: allocated for the working set only
         self.info = torch.zeros(B, dtype=torch.int32, device=Y.device)
         self.final = None                             # allocated when the first matrix is done
         self.redo = []                                # matrices handed to the library at the end
@@ -491,11 +490,12 @@ class CholeskyQR:
         self.ids = np.arange(B)
         self.near = np.zeros(B, dtype=bool)
         self.last = None                              # (pivot flags, near, ids) of the round not yet looked at
+        self.swept = sweep
         if sweep:
-            # one sweep of block Gram-Schmidt with reorthogonalisation leaves all but pathological matrices
-            # orthonormal to rounding: the rounds below then only confirm it (one test, no factorisation)
+            # One sweep of block Gram-Schmidt with reorthogonalisation.  Where no pivot of a panel factorisation
+            # came near the floor and no column had to be replaced (info == 0) the result is orthonormal to
+            # fp32 rounding by construction; the rounds below are for the other matrices only.
             block_gram_schmidt(self.Q, self.info, pivot_floor)
-            self.info.zero_()
 
     def _index(self, positions):
         return torch.as_tensor(np.ascontiguousarray(positions), dtype=torch.int64).to(self.Q.device)
@@ -523,6 +523,14 @@ class CholeskyQR:
         self.ids, self.near = self.ids[keep], self.near[keep]
 
     def check(self):
+        if self.swept:
+            self.swept = False
+            clean = self.info.cpu().numpy() == 0                                # (a host synchronisation)
+            self._finish(np.nonzero(clean)[0], self.Q)
+            self._keep(~clean)
+            self.finished = self.ids.size == 0
+            if self.finished:
+                return
         self.gram = gemm(self.Q, self.Q, trans_a=True, symmetric=True)
         self.far = gram_deviation(self.gram)                                    # max |G - I|, ||G - I||_F^2
 
@@ -533,6 +541,8 @@ class CholeskyQR:
         return (info.cpu().numpy()[:ids.size] & 1) != 0, near, ids
 
     def poll(self):
+        if self.finished:
+            return True
         far = self.far.cpu().numpy()                                            # the host synchronisation
         failed = np.zeros(self.ids.size, dtype=bool)
         if self.last is not None:
@@ -555,6 +565,9 @@ class CholeskyQR:
         k = self.ids.size
         info = self.info[:k]
         info.zero_()
+        if self.U is None:
+            self.U = torch.empty_like(self.Q)
+            self.X = torch.zeros_like(self.Q)         # inverse factors; the part below the diagonal blocks stays zero
         cholesky_upper(self.gram, self.U[:k], self.X[:k], info, self.pivot_floor)
         out = torch.empty_like(self.Q)
         solve_upper_right(self.Q, self.U[:k], self.X[:k], self.gram, out)      # the Gram matrix is used up: scratch
