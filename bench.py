@@ -161,8 +161,8 @@ def fused_gemm_gpu(torch, code):
     G = 0.02 * torch.randn(m, n, device="cuda", generator=g)
 
     def inverse_root_like(order):
-        q, _ = torch.linalg.qr(torch.randn(order, order, device="cuda", generator=g))
-        torch.cuda.synchronize()
+        q, _ = X.cholesky_qr(torch.randn(1, order, order, device="cuda", generator=g))     # a random orthonormal basis
+        q = q[0]
         lam = torch.exp(torch.rand(order, device="cuda", generator=g) * (-6.0 * 2.302585093))   # log-uniform in [1e-6, 1]
         return ((q * lam.pow(-0.25)) @ q.T).contiguous()
 

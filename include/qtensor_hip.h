@@ -176,10 +176,12 @@ typedef struct {
                                  * on and above the diagonal are multiplied out and every off-diagonal
                                  * tile is also stored mirrored; an addend is read at the mirrored place   */
         float *workspace;       /* optional scratch (16-byte aligned) of workspace_floats floats: a plain-store
-                                 * product with few output tiles and a long k range is then cut along k into
-                                 * slices whose partial products land here and are summed in a fixed order    */
+                                 * product with few output tiles and a long k range is then cut along k (equal
+                                 * slices per output tile, or equal runs over the k tiles of all output tiles);
+                                 * the partial products land here and are summed in a fixed order             */
         long long workspace_floats;
         int split_k_;           /* ignored (set by the library)                                             */
+        int batch_count_, stream_per_, stream_lcm_;   /* ignored (set by the library)                        */
         int batch_inner;        /* > 1: two-level batch for the strided dense operands A, B, C, E (blocks inside the
                                  * matrices of a stack): entry b lives at base + (b / batch_inner) * stride +
                                  * (b % batch_inner) * inner_x elements; 0 or 1: plain batch                    */

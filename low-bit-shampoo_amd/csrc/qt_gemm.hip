@@ -67,6 +67,10 @@ struct GemmArgs {
     float *workspace;             // optional scratch for splitting k (plain-store products only)
     long long workspace_floats;
     int split_k;                  // set by the library: slices of the k range (1 = no split)
+    int batch_count;              // set by the library: batch entries of this launch
+    int stream_per, stream_lcm;   // set by the library: > 0 = the k tiles of all output tiles, laid end to end, are dealt
+                                  // out in runs of stream_per to the workgroups (a run may end inside one output tile and
+                                  // go on in the next); stream_lcm = lcm(stream_per, k tiles per output tile)
     int batch_inner;              // > 1: batch entry b of the strided dense operands A, B, C, E lives at
     long long inner_a, inner_b, inner_c, inner_e;   // base + (b / batch_inner) * stride + (b % batch_inner) * inner_x
     int triangular;               // bit 0: A is upper triangular (A[m][k] = 0 for k < m): k starts at the tile's first row;
@@ -379,25 +383,22 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     const uint32_t die = blockIdx.x % kDies, slot = blockIdx.x / kDies;
     const uint32_t per = total / kDies, extra = total % kDies;
     uint32_t id = die * per + min(die, extra) + slot;
-    const int slices = EPI == kStore ? args.split_k : 1;
+    // Plain-store products with few output tiles and a long k range run in one of two ways that cut k:
+    // equal slices per output tile (split_k), or runs of stream_per k tiles dealt out over the k tiles of all
+    // output tiles laid end to end (every workgroup the same share of the arithmetic, whatever the number of
+    // tiles).  Either way a part of a tile's k range goes to the workspace and a second kernel adds the parts
+    // of a tile in order.
+    const bool streamed = EPI == kStore && args.stream_per > 0;
+    const int k_tiles_all = args.K / BK;                 // (only used when streamed: K is then a multiple of BK)
+    long long run_at = 0, run_end = 0;                   // streamed: this workgroup's run of k tiles, [run_at, run_end)
+    if (streamed) {
+        run_at = (long long)id * args.stream_per;
+        run_end = min(run_at + args.stream_per, (long long)tiles_m * tiles_n * args.batch_count * k_tiles_all);
+        if (run_at >= run_end) return;
+    }
+    const int slices = EPI == kStore && !streamed ? args.split_k : 1;
     const int slice = id % slices;
     id /= slices;
-    int tile_m, tile_n, b;
-    if (args.symmetric) {                  // row-major walk over the tiles on and above the diagonal
-        const uint32_t upper = (uint32_t)tiles_n * (tiles_n + 1) / 2;
-        b = id / upper;
-        uint32_t rest = id % upper, width = tiles_n;
-        tile_m = 0;
-        while (rest >= width) { rest -= width; --width; ++tile_m; }
-        tile_n = tile_m + rest;
-    } else {
-        tile_n = id % tiles_n;
-        id /= tiles_n;
-        tile_m = id % tiles_m;
-        b = id / tiles_m;
-    }
-    if (args.skip != nullptr && args.skip[b] != 0) return;
-
     using LoaderA = typename std::conditional<KA == kDense, LoadKContig<BM>,
         typename std::conditional<KA == kDenseT, LoadRowContig<BM>,
             LoadQuant<BM, KA == kQuant4 ? 4 : 8, true>>::type>::type;
@@ -430,10 +431,38 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
         if ((int)threadIdx.x < NCODE) s_code[threadIdx.x] = args.code[threadIdx.x];
         __syncthreads();
     }
-
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+
+  for (;;) {                                   // one pass, or one per piece of this workgroup's run when streamed
+    int tile_m, tile_n, b;
+    int seg_first = 0, seg_tiles = 0;          // streamed: first k tile and number of k tiles of this piece
+    long long seg_slot = -1;                   // streamed: workspace slot of a piece that is not a whole tile
+    uint32_t tile_id = id;
+    if (streamed) {
+        const long long t = run_at / k_tiles_all;
+        seg_first = (int)(run_at - t * k_tiles_all);
+        seg_tiles = (int)min((long long)(k_tiles_all - seg_first), run_end - run_at);
+        tile_id = (uint32_t)t;
+        // pieces are numbered in the order of their first k tile: one starts at every multiple of stream_per
+        // and at every multiple of the k tiles per output tile
+        if (seg_tiles != k_tiles_all) seg_slot = run_at / args.stream_per + t - run_at / args.stream_lcm;
+    }
+    if (args.symmetric) {                  // row-major walk over the tiles on and above the diagonal
+        const uint32_t upper = (uint32_t)tiles_n * (tiles_n + 1) / 2;
+        b = tile_id / upper;
+        uint32_t rest = tile_id % upper, width = tiles_n;
+        tile_m = 0;
+        while (rest >= width) { rest -= width; --width; ++tile_m; }
+        tile_n = tile_m + rest;
+    } else {
+        tile_n = tile_id % tiles_n;
+        tile_id /= tiles_n;
+        tile_m = tile_id % tiles_m;
+        b = tile_id / tiles_m;
+    }
+    if (args.skip != nullptr && args.skip[b] != 0) return;       // (never set together with `streamed`)
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     const float *A = (KA < kQuant4) ? dense_ptr(args.A, b, args.batch_inner, args.inner_a) : nullptr;
     const float *B = (KB < kQuant4) ? dense_ptr(args.B, b, args.batch_inner, args.inner_b) : nullptr;
@@ -485,8 +514,8 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     // (a triangular operand shortens the range to where it is not zero: tile origins are multiples of BK)
     const int k_first = (args.triangular & 1) ? min(m0, args.K) : 0;
     const int k_last = (args.triangular & 2) ? min(n0 + BN, args.K) : args.K;
-    const int n_tiles = max((k_last - k_first + BK - 1) / BK, 1) / slices;
-    const int k_begin = k_first + slice * n_tiles * BK;
+    const int n_tiles = streamed ? seg_tiles : max((k_last - k_first + BK - 1) / BK, 1) / slices;
+    const int k_begin = streamed ? seg_first * BK : k_first + slice * n_tiles * BK;
     fetch(k_begin);
     la.commit(s_a[0], s_code);
     lb.commit(s_b[0], s_code);
@@ -556,6 +585,10 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     if (slices > 1) {                              // partial product of this slice: summed by reduce_slices_kernel
         C = args.workspace + ((long long)b * slices + slice) * args.M * args.N;
         ldc = args.N;
+    }
+    if (seg_slot >= 0) {                           // a piece of a tile: kept as a BM x BN square, summed by reduce_pieces_kernel
+        C = args.workspace + seg_slot * (BM * BN) - ((long long)m0 * BN + n0);
+        ldc = BN;
     }
     float *T = EPI == kNewton ? const_cast<float *>(batch_ptr<float>(args.T, b)) : nullptr;
     const float *E = EPI == kAxpbyDense ? dense_ptr(args.E, b, args.batch_inner, args.inner_e) : nullptr;
@@ -771,6 +804,48 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
         uint32_t e = group_max_u32<64>(__float_as_uint(local_err));   // non-negative floats order like their bits
         if (lane == 0) atomicMax(reinterpret_cast<unsigned int *>(args.err) + b, e);
     }
+    if (!streamed) return;
+    run_at += seg_tiles;
+    if (run_at >= run_end) return;
+    __syncthreads();                               // the staging squares of the epilogue overlap the operand tiles
+  }
+}
+
+// Streamed products: out tile = sum of its pieces in the workspace, in the order of their k ranges.  A tile that
+// one workgroup did as a whole is already in place.  Grid (tiles, 4 row bands of the tile).
+__global__ __launch_bounds__(256) void reduce_pieces_kernel(const float *workspace, BatchPtr C, int ldc, int M, int N, int bm, int bn,
+                                                            int tiles_m, int tiles_n, int k_tiles, int stream_per, int stream_lcm) {
+    uint32_t t = blockIdx.x;
+    const long long first = (long long)t * k_tiles, next = first + k_tiles;
+    const long long s0 = first / stream_per + first / k_tiles - first / stream_lcm;
+    const long long s1 = next / stream_per + next / k_tiles - next / stream_lcm;
+    if (s1 - s0 <= 1) return;
+    const int tile_n = t % tiles_n;
+    t /= tiles_n;
+    const int tile_m = t % tiles_m, b = t / tiles_m;
+    float *out = const_cast<float *>(batch_ptr<float>(C, b));
+    const int m0 = tile_m * bm, n0 = tile_n * bn, plane = bm * bn, quads_per_row = bn >> 2;
+    const bool vec = (ldc & 3) == 0 && is_aligned16(out) && (N & 3) == 0;
+    const int rows = bm / 4;                           // this block's band of rows
+    for (int q = threadIdx.x; q < rows * quads_per_row; q += 256) {
+        const int r = blockIdx.y * rows + q / quads_per_row, c = (q % quads_per_row) << 2;
+        const int row = m0 + r, col = n0 + c;
+        if (row >= M || col >= N) continue;
+        const float *w = workspace + s0 * plane + r * bn + c;
+        float4 sum = gload4(w);
+        for (long long k = 1; k < s1 - s0; ++k) {
+            const float4 x = gload4(w + k * plane);
+            sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+        }
+        float *o = out + (long long)row * ldc + col;
+        if (vec) { const float y[4] = {sum.x, sum.y, sum.z, sum.w}; gstore4(o, y); }
+        else {
+            gstore(o, sum.x);
+            if (col + 1 < N) gstore(o + 1, sum.y);
+            if (col + 2 < N) gstore(o + 2, sum.z);
+            if (col + 3 < N) gstore(o + 3, sum.w);
+        }
+    }
 }
 
 
@@ -807,9 +882,18 @@ template <int BM, int BN, int KA, int KB, int EPI>
 void launch_gemm(const GemmArgs &a, int batch, hipStream_t stream) {
     const long long tn = (a.N + BN - 1) / BN, tm = (a.M + BM - 1) / BM;
     if (a.symmetric && BM != BN) { set_error(kBadArgument, "gemm: symmetric products need square tiles"); return; }
-    const long long blocks = (a.symmetric ? tn * (tn + 1) / 2 : tn * tm) * batch * (EPI == kStore ? a.split_k : 1);
+    long long blocks = (a.symmetric ? tn * (tn + 1) / 2 : tn * tm) * batch * (EPI == kStore ? a.split_k : 1);
+    if (EPI == kStore && a.stream_per > 0) {
+        const long long runs = tn * tm * batch * (a.K / BK);
+        blocks = (runs + a.stream_per - 1) / a.stream_per;
+    }
     if (blocks > 0x7fffffffLL) { set_error(kBadArgument, "gemm: too many tiles (%lld)", blocks); return; }
     hipLaunchKernelGGL((gemm_kernel<BM, BN, KA, KB, EPI>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    if (EPI == kStore && a.stream_per > 0) {
+        hipLaunchKernelGGL(reduce_pieces_kernel, dim3((unsigned)(tn * tm * batch), 4), dim3(256), 0, stream, a.workspace, a.C, a.ldc,
+                           a.M, a.N, BM, BN, (int)tm, (int)tn, a.K / BK, a.stream_per, a.stream_lcm);
+        return;
+    }
     if (EPI == kStore && a.split_k > 1) {
         const long long quads = ((long long)a.M * a.N + 1023) / 1024;
         const unsigned grid = (unsigned)(quads < 4096 ? quads : 4096);
@@ -952,6 +1036,8 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
     }
     if (ep == kNewton && (!has_host_ptr(a.T) || a.ldt < d->N || !a.err)) { set_error(kBadArgument, "gemm: Newton epilogue needs T and err"); return; }
     a.symmetric = a.symmetric != 0;
+    a.batch_count = d->batch;
+    a.stream_per = a.stream_lcm = 0;
     if (a.triangular != 0 && (ka >= kQuant4 || kb >= kQuant4 || a.symmetric || (a.triangular & ~3) != 0)) {
         set_error(kBadArgument, "gemm: triangular operands must be dense, in a product that is not marked symmetric");
         return;
@@ -1018,6 +1104,34 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
             else if (cost < best) { best = cost; best_split = sp; }
         }
         if (forced_split != nullptr || best < 0.95 * whole) a.split_k = best_split;
+        // The other way to cut k: lay the k tiles of all output tiles end to end and deal them out in equal
+        // runs over a fixed number of workgroups per compute unit.  Every workgroup then has the same share of
+        // the arithmetic whatever the number of output tiles, so the big, efficient tile shape can be kept
+        // where it alone would leave half of the units idle (144 tiles of 128 x 128 on 256 units for a
+        // 768 x 3072 result).  Taken when the output tiles of that shape would not fill the units twice over.
+        static const int stream_wgs = getenv("QT_GEMM_STREAM_WGS") != nullptr ? atoi(getenv("QT_GEMM_STREAM_WGS")) : 2;
+        const int big = d->M >= 96 && d->N >= 96 ? 0 : pick;
+        const Shape &bs = shapes[big];
+        const long long btm = (d->M + bs.bm - 1) / bs.bm, btn = (d->N + bs.bn - 1) / bs.bn;
+        const long long big_tiles = btm * btn * d->batch, runs = big_tiles * k_tiles;
+        if (stream_wgs > 0 && a.skip == nullptr && k_tiles >= 16 && big_tiles < 2 * (long long)units) {
+            long long groups = (long long)units * stream_wgs;
+            static const int min_run = getenv("QT_GEMM_STREAM_MIN") != nullptr ? atoi(getenv("QT_GEMM_STREAM_MIN")) : 24;
+            if (groups > runs / min_run) groups = runs / min_run;         // at least that many k tiles per workgroup
+            const long long per_group = groups > 0 ? (runs + groups - 1) / groups : 0;
+            const long long used = per_group > 0 ? (runs + per_group - 1) / per_group : 0;
+            if (per_group > 0 && per_group < 0x7fffffff && (used + big_tiles) * bs.bm * bs.bn <= a.workspace_floats) {
+                long long x = per_group, y = k_tiles;
+                while (y != 0) { const long long r = x % y; x = y; y = r; }
+                const long long lcm = per_group / x * k_tiles;
+                if (lcm < 0x7fffffff) {
+                    a.stream_per = (int)per_group;
+                    a.stream_lcm = (int)lcm;
+                    a.split_k = 1;
+                    pick = big;
+                }
+            }
+        }
     }
     const int combo = ka * 100 + kb * 10 + ep;
 #define QT_GEMM_CASE(KA, KB, EP)                                                                             \

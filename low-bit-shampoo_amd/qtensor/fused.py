@@ -40,6 +40,7 @@ class GemmArgs(ct.Structure):
                 ("newton_w", ct.c_float),
                 ("err", ct.c_void_p), ("skip", ct.c_void_p), ("code", ct.c_void_p), ("symmetric", ct.c_int),
                 ("workspace", ct.c_void_p), ("workspace_floats", ct.c_longlong), ("split_k_", ct.c_int),
+                ("batch_count_", ct.c_int), ("stream_per_", ct.c_int), ("stream_lcm_", ct.c_int),
                 ("batch_inner", ct.c_int), ("inner_a", ct.c_longlong), ("inner_b", ct.c_longlong),
                 ("inner_c", ct.c_longlong), ("inner_e", ct.c_longlong), ("triangular", ct.c_int)]
 
