@@ -28,6 +28,10 @@
 #include <mutex>
 #include <type_traits>
 
+#ifndef QT_STREAMK
+#define QT_STREAMK 1
+#endif
+
 namespace qt {
 
 enum OperandKind : int { kDense = 0, kDenseT = 1, kQuant4 = 2, kQuant8 = 3 };
@@ -388,7 +392,10 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     // output tiles laid end to end (every workgroup the same share of the arithmetic, whatever the number of
     // tiles).  Either way a part of a tile's k range goes to the workspace and a second kernel adds the parts
     // of a tile in order.
-    const bool streamed = EPI == kStore && args.stream_per > 0;
+    // (only built into the products with a quantized operand: the loop around the tile costs the plain
+    // products of the big stacks, which never need it, a percent)
+    constexpr bool kCanStream = QT_STREAMK && EPI == kStore && (KA >= kQuant4 || KB >= kQuant4);
+    const bool streamed = kCanStream && args.stream_per > 0;
     const int k_tiles_all = args.K / BK;                 // (only used when streamed: K is then a multiple of BK)
     long long run_at = 0, run_end = 0;                   // streamed: this workgroup's run of k tiles, [run_at, run_end)
     if (streamed) {
@@ -1114,7 +1121,7 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         const Shape &bs = shapes[big];
         const long long btm = (d->M + bs.bm - 1) / bs.bm, btn = (d->N + bs.bn - 1) / bs.bn;
         const long long big_tiles = btm * btn * d->batch, runs = big_tiles * k_tiles;
-        if (stream_wgs > 0 && a.skip == nullptr && k_tiles >= 16 && big_tiles < 2 * (long long)units) {
+        if (stream_wgs > 0 && (ka >= kQuant4 || kb >= kQuant4) && a.skip == nullptr && k_tiles >= 16 && big_tiles < 2 * (long long)units) {
             long long groups = (long long)units * stream_wgs;
             static const int min_run = getenv("QT_GEMM_STREAM_MIN") != nullptr ? atoi(getenv("QT_GEMM_STREAM_MIN")) : 24;
             if (groups > runs / min_run) groups = runs / min_run;         // at least that many k tiles per workgroup
