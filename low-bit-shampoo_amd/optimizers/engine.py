@@ -135,10 +135,11 @@ class ShampooBank:
             g.scratch = [torch.empty(len(g), o, o, device=self.device) for o in (g.bm, g.bn)]
         return g.scratch[side]
 
-    def _fan_out(self, jobs):
+    def _fan_out(self, jobs, inline=False):
         """Run the callables round-robin on the side streams, after everything already queued on the
-        current stream; the current stream then waits for all of them."""
-        if not self.streams:
+        current stream; the current stream then waits for all of them.  inline: one after the other on
+        the current stream (for a caller that is itself a side job next to another fan-out)."""
+        if inline or not self.streams:
             for job in jobs:
                 job()
             return
@@ -207,6 +208,13 @@ class ShampooBank:
             if grad.numel() != m * n or not grad.is_contiguous() or grad.dtype != torch.float32 or not grad.is_cuda:
                 raise ValueError("gradients must be contiguous fp32 GPU tensors of the parameters' shapes")
 
+    def prepare(self, grads):
+        """Checks the gradients and writes the device tables of their block addresses, so that operations
+        started afterwards from several threads only read them."""
+        self._check(grads)
+        for g in self.groups:
+            self._grad_list(g, grads)
+
     # ---- the three operations of the reference's Preconditioner, for all parameters at once ------
     @torch.no_grad()
     def add_statistics(self, grads):
@@ -250,8 +258,9 @@ class ShampooBank:
         self._active = True
 
     @torch.no_grad()
-    def preconditioned_grads(self, grads):
-        """List of P_L G P_R per parameter (buffers owned by the bank, overwritten by the next call)."""
+    def preconditioned_grads(self, grads, inline=False):
+        """List of P_L G P_R per parameter (buffers owned by the bank, overwritten by the next call).
+        inline: every launch on the current stream."""
         self._check(grads)
 
         def job(g):
@@ -262,7 +271,7 @@ class ShampooBank:
 
         for g in self.groups:
             self._grad_list(g, grads)
-        self._fan_out([job(g) for g in self.groups])
+        self._fan_out([job(g) for g in self.groups], inline=inline)
         return [out.view(p.shape) for out, p in zip(self.outputs, self.params)]
 
     def is_active(self):

@@ -36,12 +36,18 @@ class ShampooBank2(ShampooBank):
         self.rect_t1, self.rect_t2, self.inv_root_mode = rect_t1, rect_t2, inv_root_mode
         self.qr_fallbacks = 0                     # matrices that went through torch.linalg.qr so far
         self.qr_rounds = 0                        # Cholesky QR rounds so far, summed over the stacks
+        self.alongside = None                     # callable that the next add_statistics runs next to its factorisations
         super().__init__(params, name2qmap, code, **kwargs)
 
     def _early_stream(self):
         if getattr(self, "_early", None) is None:
             self._early = torch.cuda.Stream(device=self.device)
         return self._early
+
+    def _beside_stream(self):
+        if getattr(self, "_beside", None) is None:
+            self._beside = torch.cuda.Stream(device=self.device)
+        return self._beside
 
     def _init_statistics(self):
         """Basis = quantized identity, every kept quotient and the largest one = matrix_eps
@@ -134,6 +140,11 @@ class ShampooBank2(ShampooBank):
         # (_fan_out gives job i the stream i % streams, so an order keeps its stream from call to call.)
         solver, redone = {}, {}
         self._fan_out([project(o) for o in orders])
+        # work of the caller that does not depend on the statistics (bank.alongside, consumed here) fills the device
+        # next to the factorisations, on a thread and a stream of its own
+        beside, self.alongside = self.alongside, None
+        if beside is not None:
+            beside = SideJob(self.device, self._beside_stream(), beside)
         # The stacks whose factorisation is complete go on (Rayleigh quotients, requantize) on a thread and a
         # stream of their own while the others still iterate: the later rounds of a few ill-conditioned
         # matrices are chains of small launches that leave most of the device, and this thread, waiting.
@@ -151,6 +162,8 @@ class ShampooBank2(ShampooBank):
         finally:
             if early is not None:
                 early.join()
+            if beside is not None:
+                beside.join()
         self.qr_fallbacks += sum(redone.values())
         self.qr_rounds += sum(solver[o].rounds for o in orders)
 

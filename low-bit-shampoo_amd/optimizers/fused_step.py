@@ -31,6 +31,11 @@ class _FusedStep:
     # are computed on a thread of their own while the bank's batched iteration runs; their power-iteration start
     # vectors are then drawn first, on the calling thread, so that the generator is used in a fixed order
     overlap_unbatched_inverse_roots = True
+    # True: on steps that update the statistics and keep the inverse roots, the bank applies the stored roots to
+    # the gradients on a thread and a stream of its own while the factorisations of the statistics update run
+    # (chains of small launches that leave part of the device waiting; the two read the same gradients and
+    # share nothing else).  Needs a bank whose add_statistics runs the callable it finds in bank.alongside.
+    overlap_precondition = False
 
     @staticmethod
     def bank_class():
@@ -130,6 +135,12 @@ def fused_step(opt, group, update, group_index=0):
         side_job = _SideJob(unbatched[0].device, entry['side_stream'], update_unbatched)
     if bank is not None:
         bgrads = [grads[id(p)] for p in banked]
+        applied = None
+        if (opt.overlap_precondition and step % group['stat_compute_steps'] == 0 and step % group['prec_compute_steps'] != 0
+                and step >= group['start_prec_step'] and bank.is_active() and hasattr(bank, 'alongside')):
+            applied = []
+            bank.prepare(bgrads)                                       # address tables: written once, by this thread
+            bank.alongside = lambda: applied.extend(bank.preconditioned_grads(bgrads, inline=True))
         if step % group['stat_compute_steps'] == 0:
             try:
                 bank.add_statistics(bgrads)
@@ -165,7 +176,9 @@ def fused_step(opt, group, update, group_index=0):
                     roots_done = True
         if step >= group['start_prec_step'] and bank.is_active():
             # the rescaling to each gradient's norm happens inside the fused update
-            directions = {id(p): o for p, o in zip(banked, bank.preconditioned_grads(bgrads))}
+            if applied is None:
+                applied = bank.preconditioned_grads(bgrads)
+            directions = {id(p): o for p, o in zip(banked, applied)}
             grafted = set(directions)
     for p in params:
         if id(p) not in entry['ids']:

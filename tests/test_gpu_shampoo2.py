@@ -407,6 +407,43 @@ def test_statistics_of_unbatched_parameters_on_a_side_thread_change_nothing(mods
         assert all(torch.equal(x, y) for x, y in zip(a, b))
 
 
+def test_roots_applied_next_to_the_factorisations_change_nothing(mods, tmp_path, monkeypatch):
+    """On steps that keep the inverse roots the bank applies them to the gradients on a thread and stream of its own
+    while the statistics update factorises; parameters and stored bases must be bit-identical to the run in line."""
+    S2, _ = mods
+    import optimizers.matrix_functions as MF
+    monkeypatch.chdir(tmp_path)
+    real_rand = torch.rand
+    monkeypatch.setattr(MF.torch, "rand", lambda *size, **kw: torch.full(size, 0.75, **kw))
+    g = torch.Generator().manual_seed(12)
+    init = [real_rand(s, generator=g) for s in SHAPES]
+    gs = [[0.02 * torch.randn(s, generator=g) for s in SHAPES] for _ in range(7)]
+    overlapped = []
+
+    def run(overlap):
+        monkeypatch.setattr(S2.ShampooAdamW, "overlap_precondition", overlap)
+        params = [torch.nn.Parameter(x.clone().cuda()) for x in init]
+        opt = S2.ShampooAdamW(params, lr=1e-2, weight_decay=0.05, start_prec_step=2, stat_compute_steps=1,
+                              prec_compute_steps=3, fused=True, inv_root_mode=1, **KW)
+        bank = None
+        for grads in gs:
+            for p, gr in zip(params, grads):
+                p.grad = gr.clone().cuda()
+            if bank is not None and overlap and not hasattr(bank, "wrapped"):
+                real, bank.wrapped = bank.preconditioned_grads, True
+                monkeypatch.setattr(bank, "preconditioned_grads",
+                                    lambda gr, inline=False, real=real: (overlapped.append(inline), real(gr, inline=inline))[1])
+            opt.step()
+            bank = next(iter(opt._fused_cache.values()))["bank"]
+        torch.cuda.synchronize()
+        return [p.detach().cpu() for p in params], [t.cpu() for t in bank.state_dict().values() if torch.is_tensor(t)]
+
+    beside, inline = run(True), run(False)
+    assert overlapped.count(True) >= 3                      # steps 4, 5 and 7 keep their roots
+    for a, b in zip(beside[0] + beside[1], inline[0] + inline[1]):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("variant,fused", [("shampoo1", True), ("shampoo1", False), ("shampoo2", True)])
 def test_optimizers_reduce_a_small_regression_loss(variant, fused, tmp_path, monkeypatch):
     """End-to-end sanity: a two-layer network fitted to a random teacher with 4-bit Shampoo + AdamW."""
