@@ -1124,7 +1124,10 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         if (stream_wgs > 0 && (ka >= kQuant4 || kb >= kQuant4) && a.skip == nullptr && k_tiles >= 16 && big_tiles < 2 * (long long)units) {
             long long groups = (long long)units * stream_wgs;
             static const int min_run = getenv("QT_GEMM_STREAM_MIN") != nullptr ? atoi(getenv("QT_GEMM_STREAM_MIN")) : 24;
-            if (groups > runs / min_run) groups = runs / min_run;         // at least that many k tiles per workgroup
+            if (groups > runs / min_run) {                                // at least that many k tiles per workgroup,
+                groups = runs / min_run;                                  // and no unit with one workgroup more than another
+                if (groups > (long long)units) groups -= groups % (long long)units;
+            }
             const long long per_group = groups > 0 ? (runs + groups - 1) / groups : 0;
             const long long used = per_group > 0 ? (runs + per_group - 1) / per_group : 0;
             if (per_group > 0 && per_group < 0x7fffffff && (used + big_tiles) * bs.bm * bs.bn <= a.workspace_floats) {
