@@ -212,6 +212,22 @@ void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
 #define QTENSOR_STATIC_SCRATCH_FLOATS (1 << 24)
 void qtensor_hip_gemm_static(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
 
+/* Which matrix pipe multiplies products of two dense operands, for the whole process (no counterpart in the
+ * reference, whose products are torch's fp32 matmul).
+ *   0: the fp32 pipe (v_mfma_f32_32x32x2_f32) on the operands as they are;
+ *   1: the bf16 pipe on split operands: every fp32 element x is written as h + m + l, three bf16 numbers, each the
+ *      round-to-nearest of what the ones before leave over (|x - h - m - l| <= 2^-24 |x|), and a b is taken as
+ *      a_h b_h + a_h b_m + a_m b_h + a_h b_l + a_l b_h + a_m b_m -- six bf16 products, each exact in fp32, summed
+ *      in fp32 by v_mfma_f32_32x32x16_bf16.  What is left out is below 2^-24 |a b| per product, so a dot product
+ *      carries the error of fp32 arithmetic (tests/test_gpu_gemm.py measures both pipes against float64), while the
+ *      bf16 pipe does sixteen multiply-adds per cycle for every one of the fp32 pipe.  Differences: an infinite
+ *      operand element gives NaN where the fp32 pipe gives infinity; elements below 2^-110 lose their low pieces.
+ *      Taken for dense operands, K a multiple of 16 and at least 32, under the 128 x 128 tile shape; every other
+ *      product runs on the fp32 pipe whatever the mode.
+ * mode < 0 only queries.  Returns the mode in force before the call.  The initial mode is 1 unless the environment
+ * variable QT_GEMM_PIPE is "f32". */
+int qtensor_hip_gemm_pipe(int mode);
+
 /* ---- batched Cholesky factorisation and triangular solve (Cholesky QR) ---------------------------
  * Replace, for a whole stack of statistics at once, the QR factorisation the reference calls per
  * matrix in QTensorSVDFast.quantize (torch.linalg.qr, qtensor/utils.py:157): one round of

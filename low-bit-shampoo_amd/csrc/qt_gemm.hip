@@ -22,7 +22,9 @@
 #include "qt_common.h"
 #include "qt_tables.h"
 
+#include <atomic>
 #include <cmath>
+#include <cstring>
 #include <cstdio>
 #include <cstdlib>
 #include <mutex>
@@ -84,6 +86,13 @@ struct GemmArgs {
 namespace {
 
 constexpr int BK = 16;
+// Which matrix pipe multiplies.  kPipeF32: v_mfma_f32_32x32x2_f32 on the operands as they are.  kPipeSplit: every fp32
+// operand element is written as the sum of three bf16 numbers (x = h + m + l, each the rounding of what the ones before
+// leave over: |x - h - m - l| <= 2^-24 |x|) and a product a b is the six bf16 products a_h b_h + a_h b_m + a_m b_h +
+// a_h b_l + a_l b_h + a_m b_m, each exact in fp32, accumulated in fp32 by v_mfma_f32_32x32x16_bf16.  The terms left out
+// are below 2^-24 |a b|: the error of a dot product stays that of fp32 arithmetic, and the bf16 pipe does sixteen times
+// the multiply-adds per cycle of the fp32 pipe, six of which make one fp32 multiply-add.
+constexpr int kPipeF32 = 0, kPipeSplit = 1;
 constexpr uint32_t kDies = 8;          // accelerator dies (XCDs) of an MI355X
 constexpr int LDS_PAD = 4;   // k-major tiles ([k][row]): row stride = rows + 4 floats, 16-byte aligned rows
 constexpr int LDK = BK + 4;  // row-major tiles ([row][k], for sources whose k is contiguous): 20 floats per row, so
@@ -264,6 +273,135 @@ struct LoadRowContig {
     }
 };
 
+// ---- loaders of the split pipe: global -> registers (fp32) -> LDS (three bf16 planes) -----------
+// A plane of an operand tile of ROWS rows holds, for each half of the 16 k of a tile, the 8 values of every row as 16
+// bytes: [half][row][8 bf16], the halves kSplitHalfPad bytes further apart than they need be so that the 16-byte
+// stores of two threads that differ in the half fall into different banks.  A lane's MFMA fragment (8 consecutive k of
+// one row) is then one 16-byte read, and the 32 lanes of a half read 512 contiguous bytes.
+typedef __bf16 qt_bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 qt_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float qt_f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t qt_u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kSplitHalfPad = 64;
+template <int ROWS> struct SplitLayout {
+    static constexpr int kHalf = ROWS * 16 + kSplitHalfPad, kPlane = 2 * kHalf, kOperand = 3 * kPlane;   // bytes
+};
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {       // round to nearest even, a in the low half
+    const qt_f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, qt_bf16x2));
+}
+__device__ __forceinline__ float low_bf16(uint32_t p) { return __builtin_bit_cast(float, p << 16); }
+__device__ __forceinline__ float high_bf16(uint32_t p) { return __builtin_bit_cast(float, p & 0xffff0000u); }
+
+// 8 floats -> their three bf16 planes (4 packed words each); the subtractions are exact
+__device__ __forceinline__ void split_eight(const float x[8], qt_u32x4 &h, qt_u32x4 &m, qt_u32x4 &l) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float a = x[2 * i], b = x[2 * i + 1];
+        const uint32_t ph = pack_bf16(a, b);
+        const float ra = a - low_bf16(ph), rb = b - high_bf16(ph);
+        const uint32_t pm = pack_bf16(ra, rb);
+        const float sa = ra - low_bf16(pm), sb = rb - high_bf16(pm);
+        h[i] = ph; m[i] = pm; l[i] = pack_bf16(sa, sb);
+    }
+}
+
+template <int ROWS>
+__device__ __forceinline__ void commit_split_eight(unsigned char *operand, int row, int half, const float x[8]) {
+    using L = SplitLayout<ROWS>;
+    qt_u32x4 h, m, l;
+    split_eight(x, h, m, l);
+    unsigned char *at = operand + half * L::kHalf + row * 16;
+    *reinterpret_cast<qt_u32x4 *>(at) = h;
+    *reinterpret_cast<qt_u32x4 *>(at + L::kPlane) = m;
+    *reinterpret_cast<qt_u32x4 *>(at + 2 * L::kPlane) = l;
+}
+
+// 4 floats -> their three bf16 planes (2 packed words each)
+__device__ __forceinline__ void split_four(const float x[4], uint2 &h, uint2 &m, uint2 &l) {
+    uint32_t hh[2], mm[2], ll[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const float a = x[2 * i], b = x[2 * i + 1];
+        const uint32_t ph = pack_bf16(a, b);
+        const float ra = a - low_bf16(ph), rb = b - high_bf16(ph);
+        const uint32_t pm = pack_bf16(ra, rb);
+        const float sa = ra - low_bf16(pm), sb = rb - high_bf16(pm);
+        hh[i] = ph; mm[i] = pm; ll[i] = pack_bf16(sa, sb);
+    }
+    h = make_uint2(hh[0], hh[1]); m = make_uint2(mm[0], mm[1]); l = make_uint2(ll[0], ll[1]);
+}
+
+template <int ROWS>
+__device__ __forceinline__ void commit_split_four(unsigned char *operand, int row, int quarter, const float x[4]) {
+    using L = SplitLayout<ROWS>;
+    uint2 h, m, l;
+    split_four(x, h, m, l);
+    unsigned char *at = operand + (quarter >> 1) * L::kHalf + row * 16 + (quarter & 1) * 8;
+    *reinterpret_cast<uint2 *>(at) = h;
+    *reinterpret_cast<uint2 *>(at + L::kPlane) = m;
+    *reinterpret_cast<uint2 *>(at + 2 * L::kPlane) = l;
+}
+
+// Dense, k contiguous in memory (element (row, k) at base[row * ld + k]); whole k tiles.  128 rows: thread t takes 8
+// consecutive k (half t & 1) of row t >> 1; 64 rows: 4 consecutive k (quarter t & 3) of row t >> 2.  Rows beyond the
+// matrix are clamped (their products are never stored).  `vec`: rows are 16-byte aligned (the same for the whole
+// workgroup); otherwise word loads.
+template <int ROWS>
+struct SplitKContig {
+    static_assert(ROWS == 128 || ROWS == 64, "tile rows");
+    static constexpr int PER = ROWS * BK / 256;
+    float v[PER];
+    int off;
+    bool vec = true;
+    __device__ __forceinline__ void prepare(int ld, int row0, int rows) {
+        const int row = ROWS == 128 ? threadIdx.x >> 1 : threadIdx.x >> 2, part = ROWS == 128 ? threadIdx.x & 1 : threadIdx.x & 3;
+        off = min(row0 + row, rows - 1) * ld + part * PER;
+    }
+    __device__ __forceinline__ void fetch_fast(const float *tile_base) {
+        if (vec) {
+#pragma unroll
+            for (int q = 0; q < PER / 4; ++q) {
+                const float4 x = gload4(tile_base + off + 4 * q);
+                v[4 * q] = x.x; v[4 * q + 1] = x.y; v[4 * q + 2] = x.z; v[4 * q + 3] = x.w;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < PER; ++j) v[j] = gload(tile_base + off + j);
+        }
+    }
+    __device__ __forceinline__ void commit_split(unsigned char *operand) const {
+        if constexpr (ROWS == 128) commit_split_eight<ROWS>(operand, threadIdx.x >> 1, threadIdx.x & 1, v);
+        else commit_split_four<ROWS>(operand, threadIdx.x >> 2, threadIdx.x & 3, v);
+    }
+};
+
+// Dense, row index contiguous in memory (element (row, k) at base[k * ld + row]); whole k tiles.  128 rows: thread t
+// takes row t & 127 and the 8 k of half t >> 7; 64 rows: row t & 63 and the 4 k of quarter t >> 6; one word per load,
+// a wave's load covers 64 consecutive words.
+template <int ROWS>
+struct SplitRowContig {
+    static_assert(ROWS == 128 || ROWS == 64, "tile rows");
+    static constexpr int PER = ROWS * BK / 256;
+    float v[PER];
+    int off, ld_;
+    bool vec = true;                         // (unused: word loads need no alignment)
+    __device__ __forceinline__ void prepare(int ld, int row0, int rows) {
+        ld_ = ld;
+        const int row = threadIdx.x & (ROWS - 1), part = ROWS == 128 ? threadIdx.x >> 7 : threadIdx.x >> 6;
+        off = part * PER * ld + min(row0 + row, rows - 1);
+    }
+    __device__ __forceinline__ void fetch_fast(const float *tile_base) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) v[j] = gload(tile_base + off + j * ld_);
+    }
+    __device__ __forceinline__ void commit_split(unsigned char *operand) const {
+        if constexpr (ROWS == 128) commit_split_eight<ROWS>(operand, threadIdx.x & 127, threadIdx.x >> 7, v);
+        else commit_split_four<ROWS>(operand, threadIdx.x & 63, threadIdx.x >> 6, v);
+    }
+};
+
 // Quantized square matrix (order x order, flat layout).  ALONG_K: the tile's k runs along the
 // matrix columns (left factor); otherwise the tile's rows run along the matrix columns (right
 // factor).  Each thread expands 8 consecutive codes of one matrix row.
@@ -376,7 +514,7 @@ struct LoadQuant {
     }
 };
 
-template <int BM, int BN, int KA, int KB, int EPI>
+template <int BM, int BN, int KA, int KB, int EPI, int PREC = kPipeF32>
 __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   // three waves per SIMD: at most 168 registers
     constexpr int WM = BM / 2, WN = BN / 2, MI = WM / 32, NI = WN / 32;
     // Workgroups are dealt round-robin to the 8 accelerator dies, each with its own L2.  Renumber
@@ -406,23 +544,31 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     const int slices = EPI == kStore && !streamed ? args.split_k : 1;
     const int slice = id % slices;
     id /= slices;
-    using LoaderA = typename std::conditional<KA == kDense, LoadKContig<BM>,
+    constexpr bool kSplit = PREC == kPipeSplit;
+    static_assert(!kSplit || (KA < kQuant4 && KB < kQuant4), "split pipe: dense operands");
+    using PlainA = typename std::conditional<KA == kDense, LoadKContig<BM>,
         typename std::conditional<KA == kDenseT, LoadRowContig<BM>,
             LoadQuant<BM, KA == kQuant4 ? 4 : 8, true>>::type>::type;
-    using LoaderB = typename std::conditional<KB == kDense, LoadRowContig<BN>,
+    using PlainB = typename std::conditional<KB == kDense, LoadRowContig<BN>,
         typename std::conditional<KB == kDenseT, LoadKContig<BN>,
             LoadQuant<BN, KB == kQuant4 ? 4 : 8, false>>::type>::type;
+    constexpr int SPLIT_ROWS_A = BM, SPLIT_ROWS_B = BN;
+    using LoaderA = typename std::conditional<!kSplit, PlainA,
+        typename std::conditional<KA == kDense, SplitKContig<SPLIT_ROWS_A>, SplitRowContig<SPLIT_ROWS_A>>::type>::type;
+    using LoaderB = typename std::conditional<!kSplit, PlainB,
+        typename std::conditional<KB == kDense, SplitRowContig<SPLIT_ROWS_B>, SplitKContig<SPLIT_ROWS_B>>::type>::type;
     // An operand whose k is contiguous at the source sits in LDS as [row][k] (16-byte commits, one
     // 16-byte fragment read per four MFMA steps); the others as [k][row] (16-byte commits, one word
     // per step).  Which k a lane feeds into which step is free as long as both operands agree:
     // step s of a tile takes k = 8 (s / 4) + 4 (lane / 32) + s % 4.
-    constexpr bool A_RM = LoaderA::kRowMajor, B_RM = LoaderB::kRowMajor;
+    constexpr bool A_RM = PlainA::kRowMajor, B_RM = PlainB::kRowMajor;
     constexpr int LDA = BM + LDS_PAD, LDB = BN + LDS_PAD;
     constexpr int SIZE_A = A_RM ? BM * LDK : BK * LDA, SIZE_B = B_RM ? BN * LDK : BK * LDB;
     // one buffer: the two stages of both operand tiles during the main loop, then (symmetric products)
     // a 32 x 32 staging square per wave that turns accumulator blocks around for the mirrored stores
     constexpr bool kRequant = EPI == kRequant4 || EPI == kRequant8;
-    constexpr int STAGE_LD = 36, REQUANT_LD = 68, SIZE_MAIN = 2 * SIZE_A + 2 * SIZE_B;
+    constexpr int SPLIT_A = SplitLayout<BM>::kOperand, SPLIT_STAGE = SPLIT_A + SplitLayout<BN>::kOperand;     // bytes
+    constexpr int STAGE_LD = 36, REQUANT_LD = 68, SIZE_MAIN = kSplit ? 2 * SPLIT_STAGE / 4 : 2 * SIZE_A + 2 * SIZE_B;
     constexpr int SIZE_STAGE = kRequant ? 4 * 32 * REQUANT_LD : 4 * 32 * STAGE_LD;
     __shared__ __attribute__((aligned(16))) float s_mem[SIZE_MAIN > SIZE_STAGE ? SIZE_MAIN : SIZE_STAGE];
     float (*s_a)[SIZE_A] = reinterpret_cast<float (*)[SIZE_A]>(s_mem);
@@ -483,27 +629,49 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     // offsets inside 31 bits: the loads of the main loop then need no predicates at all
     const bool whole_k = args.K % BK == 0;
     bool a_fast = false, b_fast = false;
-    if constexpr (KA < kQuant4) {
-        a_fast = whole_k && a_vec && (KA == kDense || (args.M & 3) == 0) &&
-                 (long long)(KA == kDense ? args.M : args.K) * args.lda < 0x7fffffffLL;
-        if (a_fast) la.prepare(args.lda, m0, args.M);
-    }
-    if constexpr (KB < kQuant4) {
-        b_fast = whole_k && b_vec && (KB == kDenseT || (args.N & 3) == 0) &&
-                 (long long)(KB == kDenseT ? args.N : args.K) * args.ldb < 0x7fffffffLL;
-        if (b_fast) lb.prepare(args.ldb, n0, args.N);
-    }
-    if constexpr (KA >= kQuant4) la.prepare(args.Aq, b, m0);
-    if constexpr (KB >= kQuant4) lb.prepare(args.Bq, b, n0);
-    auto fetch = [&](int k0) {
+    if constexpr (kSplit) {                    // the host only picks this pipe where the fast loads apply
+        la.prepare(args.lda, m0, args.M);
+        lb.prepare(args.ldb, n0, args.N);
+        if constexpr (KA == kDense) la.vec = a_vec;
+        if constexpr (KB == kDenseT) lb.vec = b_vec;
+    } else {
         if constexpr (KA < kQuant4) {
-            if (a_fast) la.fetch_fast(A + (KA == kDense ? (long long)k0 : (long long)k0 * args.lda));
-            else la.fetch(A, args.lda, m0, k0, args.M, args.K, a_vec);
-        } else la.fetch(k0);
+            a_fast = whole_k && a_vec && (KA == kDense || (args.M & 3) == 0) &&
+                     (long long)(KA == kDense ? args.M : args.K) * args.lda < 0x7fffffffLL;
+            if (a_fast) la.prepare(args.lda, m0, args.M);
+        }
         if constexpr (KB < kQuant4) {
-            if (b_fast) lb.fetch_fast(B + (KB == kDenseT ? (long long)k0 : (long long)k0 * args.ldb));
-            else lb.fetch(B, args.ldb, n0, k0, args.N, args.K, b_vec);
-        } else lb.fetch(k0);
+            b_fast = whole_k && b_vec && (KB == kDenseT || (args.N & 3) == 0) &&
+                     (long long)(KB == kDenseT ? args.N : args.K) * args.ldb < 0x7fffffffLL;
+            if (b_fast) lb.prepare(args.ldb, n0, args.N);
+        }
+        if constexpr (KA >= kQuant4) la.prepare(args.Aq, b, m0);
+        if constexpr (KB >= kQuant4) lb.prepare(args.Bq, b, n0);
+    }
+    auto fetch = [&](int k0) {
+        if constexpr (kSplit) {
+            la.fetch_fast(A + (KA == kDense ? (long long)k0 : (long long)k0 * args.lda));
+            lb.fetch_fast(B + (KB == kDenseT ? (long long)k0 : (long long)k0 * args.ldb));
+        } else {
+            if constexpr (KA < kQuant4) {
+                if (a_fast) la.fetch_fast(A + (KA == kDense ? (long long)k0 : (long long)k0 * args.lda));
+                else la.fetch(A, args.lda, m0, k0, args.M, args.K, a_vec);
+            } else la.fetch(k0);
+            if constexpr (KB < kQuant4) {
+                if (b_fast) lb.fetch_fast(B + (KB == kDenseT ? (long long)k0 : (long long)k0 * args.ldb));
+                else lb.fetch(B, args.ldb, n0, k0, args.N, args.K, b_vec);
+            } else lb.fetch(k0);
+        }
+    };
+    auto commit = [&](int stage) {
+        if constexpr (kSplit) {
+            unsigned char *at = reinterpret_cast<unsigned char *>(s_mem) + stage * SPLIT_STAGE;
+            la.commit_split(at);
+            lb.commit_split(at + SPLIT_A);
+        } else {
+            la.commit(s_a[stage], s_code);
+            lb.commit(s_b[stage], s_code);
+        }
     };
 
     f32x16 acc[MI][NI];
@@ -524,12 +692,43 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     const int n_tiles = streamed ? seg_tiles : max((k_last - k_first + BK - 1) / BK, 1) / slices;
     const int k_begin = streamed ? seg_first * BK : k_first + slice * n_tiles * BK;
     fetch(k_begin);
-    la.commit(s_a[0], s_code);
-    lb.commit(s_b[0], s_code);
+    commit(0);
     if (n_tiles > 1) fetch(k_begin + BK);
     __syncthreads();
     const int frag_row = lane & 31, half = lane >> 5;
     constexpr int STEPS = BK / 2;
+    if constexpr (kSplit) {
+        using LA = SplitLayout<BM>;
+        using LB = SplitLayout<BN>;
+        // products in the order of their size, smallest first: (h, l), (l, h), (m, m), (h, m), (m, h), (h, h)
+        constexpr int pa_of[6] = {0, 2, 1, 0, 1, 0}, pb_of[6] = {2, 0, 1, 1, 0, 0};
+        for (int t = 0; t < n_tiles; ++t) {
+            const int cur = t & 1;
+            const unsigned char *sa = reinterpret_cast<const unsigned char *>(s_mem) + cur * SPLIT_STAGE + half * LA::kHalf + (wm + frag_row) * 16;
+            const unsigned char *sb = reinterpret_cast<const unsigned char *>(s_mem) + cur * SPLIT_STAGE + SPLIT_A + half * LB::kHalf + (wn + frag_row) * 16;
+            qt_bf16x8 fa[3][MI], fb[3][NI];
+#pragma unroll
+            for (int p = 0; p < 3; ++p) {
+#pragma unroll
+                for (int i = 0; i < MI; ++i) fa[p][i] = *reinterpret_cast<const qt_bf16x8 *>(sa + p * LA::kPlane + i * 32 * 16);
+#pragma unroll
+                for (int j = 0; j < NI; ++j) fb[p][j] = *reinterpret_cast<const qt_bf16x8 *>(sb + p * LB::kPlane + j * 32 * 16);
+            }
+#pragma unroll
+            for (int q = 0; q < 6; ++q) {
+                if (q == 3 && t + 1 < n_tiles) {
+                    commit(cur ^ 1);
+                    if (t + 2 < n_tiles) fetch(k_begin + (t + 2) * BK);
+                }
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[pa_of[q]][i], fb[pb_of[q]][j], acc[i][j], 0, 0, 0);
+            }
+            __syncthreads();
+        }
+    } else
     for (int t = 0; t < n_tiles; ++t) {
         const int cur = t & 1;
         const float *pa = s_a[cur] + (A_RM ? (wm + frag_row) * LDK + 4 * half : 4 * half * LDA + wm + frag_row);
@@ -570,8 +769,7 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
             if (!A_RM && s + 1 < STEPS) load_a(s + 1);
             if (!B_RM && s + 1 < STEPS) load_b(s + 1);
             if (s == STEPS / 2 && t + 1 < n_tiles) {
-                la.commit(s_a[cur ^ 1], s_code);
-                lb.commit(s_b[cur ^ 1], s_code);
+                commit(cur ^ 1);
                 if (t + 2 < n_tiles) fetch(k_begin + (t + 2) * BK);
             }
 #pragma unroll
@@ -584,6 +782,60 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
                 }
         }
         __syncthreads();
+    }
+
+    // Split pipe, diagonal tile of a symmetric product: a b and b a add the pieces of a product in different orders,
+    // so an element below the diagonal that is multiplied out differs in its last bits from the mirror image of
+    // its partner above -- and which of the two a tile shape produces depends on the shape.  Every element below
+    // the diagonal therefore takes the value of its partner above, here as in the mirrored tiles: the result is
+    // exactly symmetric and does not depend on the tiling.  (On the fp32 pipe the products of G G^T commute.)
+    if constexpr (kSplit && BM == BN) {
+        if (args.symmetric && tile_m == tile_n) {
+            constexpr int XLD = WN + 1;
+            float *X = s_mem;                                   // one quadrant (WM x WN) at a time; the operand tiles are done with
+            auto put = [&](bool turned) {
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const int lr = i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + r % 4, lc = j * 32 + (lane & 31);
+                            X[turned ? lc * XLD + lr : lr * XLD + lc] = acc[i][j][r];
+                        }
+            };
+            if (wm < wn) put(true);                             // the quadrant above the diagonal, turned around ...
+            __syncthreads();
+            if (wm > wn) {                                      // ... is the one below
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const int lr = i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + r % 4, lc = j * 32 + (lane & 31);
+                            acc[i][j][r] = X[lr * XLD + lc];
+                        }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int w = 0; w < 2; ++w) {                       // the two quadrants on the diagonal, one after the other
+                if (wm == wn && (wm != 0) == (w == 1)) {
+                    put(false);
+                    wave_lds_sync();
+#pragma unroll
+                    for (int i = 0; i < MI; ++i)
+#pragma unroll
+                        for (int j = 0; j < NI; ++j)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                const int lr = i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + r % 4, lc = j * 32 + (lane & 31);
+                                if (lr > lc) acc[i][j][r] = X[lc * XLD + lr];
+                            }
+                }
+                __syncthreads();
+            }
+        }
     }
 
     // ---- epilogue
@@ -885,7 +1137,7 @@ __global__ __launch_bounds__(256) void reduce_slices_kernel(const float *workspa
     }
 }
 
-template <int BM, int BN, int KA, int KB, int EPI>
+template <int BM, int BN, int KA, int KB, int EPI, int PREC = kPipeF32>
 void launch_gemm(const GemmArgs &a, int batch, hipStream_t stream) {
     const long long tn = (a.N + BN - 1) / BN, tm = (a.M + BM - 1) / BM;
     if (a.symmetric && BM != BN) { set_error(kBadArgument, "gemm: symmetric products need square tiles"); return; }
@@ -895,7 +1147,7 @@ void launch_gemm(const GemmArgs &a, int batch, hipStream_t stream) {
         blocks = (runs + a.stream_per - 1) / a.stream_per;
     }
     if (blocks > 0x7fffffffLL) { set_error(kBadArgument, "gemm: too many tiles (%lld)", blocks); return; }
-    hipLaunchKernelGGL((gemm_kernel<BM, BN, KA, KB, EPI>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((gemm_kernel<BM, BN, KA, KB, EPI, PREC>), dim3((unsigned)blocks), dim3(256), 0, stream, a);
     if (EPI == kStore && a.stream_per > 0) {
         hipLaunchKernelGGL(reduce_pieces_kernel, dim3((unsigned)(tn * tm * batch), 4), dim3(256), 0, stream, a.workspace, a.C, a.ldc,
                            a.M, a.N, BM, BN, (int)tm, (int)tn, a.K / BK, a.stream_per, a.stream_lcm);
@@ -970,7 +1222,28 @@ float *static_scratch() {
 }
 
 void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream);
+
+// Process-wide choice of the matrix pipe for products of dense operands (qtensor_hip_gemm_pipe); starts from the
+// environment variable QT_GEMM_PIPE ("f32" or "split"), else the split pipe.
+std::atomic<int> &pipe_mode_slot() {
+    static std::atomic<int> mode{[] {
+        const char *e = getenv("QT_GEMM_PIPE");
+        return e != nullptr && (strcmp(e, "f32") == 0 || strcmp(e, "0") == 0) ? qt::kPipeF32 : qt::kPipeSplit;
+    }()};
+    return mode;
+}
+int gemm_pipe_mode() { return pipe_mode_slot().load(std::memory_order_relaxed); }
 }  // namespace
+
+extern "C" int qtensor_hip_gemm_pipe(int mode) {
+    qt::clear_error();
+    if (mode < 0) return gemm_pipe_mode();
+    if (mode != qt::kPipeF32 && mode != qt::kPipeSplit) {
+        qt::set_error(qt::kBadArgument, "gemm_pipe: mode must be 0 (fp32 pipe), 1 (split bf16 pipe) or negative (query), got %d", mode);
+        return gemm_pipe_mode();
+    }
+    return pipe_mode_slot().exchange(mode, std::memory_order_relaxed);
+}
 
 extern "C" void qtensor_hip_gemm(const qtensor_gemm_desc *d, void *stream_v) {
     qt::clear_error();
@@ -1063,6 +1336,14 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
     // 128-wide tile on their side unless QT_GEMM_TILE=MxN (a tuning knob) says otherwise.
     struct Shape { int bm, bn; double eff; };
     static const Shape shapes[4] = {{128, 128, 1.0}, {128, 64, 0.92}, {64, 128, 0.92}, {64, 64, 0.82}};
+    // The split pipe: for dense operands in whole k tiles, where the offsets of its loads fit 31 bits -- whatever the
+    // tile shape, so that the bits of a product do not depend on how it is tiled.
+    bool split_pipe = false;
+    if (gemm_pipe_mode() == kPipeSplit && ka < kQuant4 && kb < kQuant4 && d->K % BK == 0 && d->K >= 2 * BK) {
+        const long long reach_a = ka == kDense ? (long long)d->M * a.lda : (long long)BK * a.lda + d->M;
+        const long long reach_b = kb == kDenseT ? (long long)d->N * a.ldb : (long long)BK * a.ldb + d->N;
+        split_pipe = reach_a < 0x7fffffffLL && reach_b < 0x7fffffffLL;
+    }
     int pick = 0;
     static const char *forced = getenv("QT_GEMM_TILE");
     if (forced != nullptr) {
@@ -1144,6 +1425,24 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         }
     }
     const int combo = ka * 100 + kb * 10 + ep;
+#define QT_GEMM_CASE_DENSE(KA, KB, EP)                                                                       \
+    case (KA) * 100 + (KB) * 10 + (EP):                                                                      \
+        if (split_pipe) {                                                                                    \
+            if (pick == 0) launch_gemm<128, 128, KA, KB, EP, kPipeSplit>(a, d->batch, stream);               \
+            else if (pick == 1) launch_gemm<128, 64, KA, KB, EP, kPipeSplit>(a, d->batch, stream);           \
+            else if (pick == 2) launch_gemm<64, 128, KA, KB, EP, kPipeSplit>(a, d->batch, stream);           \
+            else launch_gemm<64, 64, KA, KB, EP, kPipeSplit>(a, d->batch, stream);                           \
+        }                                                                                                    \
+        else if (pick == 0) launch_gemm<128, 128, KA, KB, EP>(a, d->batch, stream);                          \
+        else if (pick == 1) launch_gemm<128, 64, KA, KB, EP>(a, d->batch, stream);                           \
+        else if (pick == 2) launch_gemm<64, 128, KA, KB, EP>(a, d->batch, stream);                           \
+        else launch_gemm<64, 64, KA, KB, EP>(a, d->batch, stream);                                           \
+        break;
+#define QT_GEMM_CASE_REQUANT(KA, KB, EP)                                                                     \
+    case (KA) * 100 + (KB) * 10 + (EP):                                                                      \
+        if (split_pipe) launch_gemm<128, 128, KA, KB, EP, kPipeSplit>(a, d->batch, stream);                  \
+        else launch_gemm<128, 128, KA, KB, EP>(a, d->batch, stream);                                         \
+        break;
 #define QT_GEMM_CASE(KA, KB, EP)                                                                             \
     case (KA) * 100 + (KB) * 10 + (EP):                                                                      \
         if (pick == 0) launch_gemm<128, 128, KA, KB, EP>(a, d->batch, stream);                               \
@@ -1156,21 +1455,21 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         QT_GEMM_CASE(kQuant8, kDense, kStore)
         QT_GEMM_CASE(kDense, kQuant4, kStore)
         QT_GEMM_CASE(kDense, kQuant8, kStore)
-        QT_GEMM_CASE(kDense, kDenseT, kStore)
-        QT_GEMM_CASE(kDense, kDenseT, kAxpbyDense)
-        QT_GEMM_CASE(kDense, kDenseT, kAxpbyQuant4)
-        QT_GEMM_CASE(kDense, kDenseT, kAxpbyQuant8)
-        case kDense * 100 + kDenseT * 10 + kRequant4: launch_gemm<128, 128, kDense, kDenseT, kRequant4>(a, d->batch, stream); break;
-        case kDense * 100 + kDenseT * 10 + kRequant8: launch_gemm<128, 128, kDense, kDenseT, kRequant8>(a, d->batch, stream); break;
-        case kDenseT * 100 + kDense * 10 + kRequant4: launch_gemm<128, 128, kDenseT, kDense, kRequant4>(a, d->batch, stream); break;
-        case kDenseT * 100 + kDense * 10 + kRequant8: launch_gemm<128, 128, kDenseT, kDense, kRequant8>(a, d->batch, stream); break;
-        QT_GEMM_CASE(kDenseT, kDense, kStore)
-        QT_GEMM_CASE(kDenseT, kDense, kAxpbyDense)
-        QT_GEMM_CASE(kDenseT, kDense, kAxpbyQuant4)
-        QT_GEMM_CASE(kDenseT, kDense, kAxpbyQuant8)
-        QT_GEMM_CASE(kDense, kDense, kStore)
-        QT_GEMM_CASE(kDense, kDense, kAxpbyDense)
-        QT_GEMM_CASE(kDense, kDense, kNewton)
+        QT_GEMM_CASE_DENSE(kDense, kDenseT, kStore)
+        QT_GEMM_CASE_DENSE(kDense, kDenseT, kAxpbyDense)
+        QT_GEMM_CASE_DENSE(kDense, kDenseT, kAxpbyQuant4)
+        QT_GEMM_CASE_DENSE(kDense, kDenseT, kAxpbyQuant8)
+        QT_GEMM_CASE_REQUANT(kDense, kDenseT, kRequant4)
+        QT_GEMM_CASE_REQUANT(kDense, kDenseT, kRequant8)
+        QT_GEMM_CASE_REQUANT(kDenseT, kDense, kRequant4)
+        QT_GEMM_CASE_REQUANT(kDenseT, kDense, kRequant8)
+        QT_GEMM_CASE_DENSE(kDenseT, kDense, kStore)
+        QT_GEMM_CASE_DENSE(kDenseT, kDense, kAxpbyDense)
+        QT_GEMM_CASE_DENSE(kDenseT, kDense, kAxpbyQuant4)
+        QT_GEMM_CASE_DENSE(kDenseT, kDense, kAxpbyQuant8)
+        QT_GEMM_CASE_DENSE(kDense, kDense, kStore)
+        QT_GEMM_CASE_DENSE(kDense, kDense, kAxpbyDense)
+        QT_GEMM_CASE_DENSE(kDense, kDense, kNewton)
         default:
             set_error(kBadArgument, "gemm: combination A kind %d, B kind %d, epilogue %d is not built", ka, kb, ep);
             return;

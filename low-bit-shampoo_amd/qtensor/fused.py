@@ -51,6 +51,8 @@ class GemmDesc(ct.Structure):
 
 
 if F.lib is not None:
+    F.lib.qtensor_hip_gemm_pipe.restype = ct.c_int
+    F.lib.qtensor_hip_gemm_pipe.argtypes = [ct.c_int]
     F.lib.qtensor_hip_gemm.restype = None
     F.lib.qtensor_hip_gemm.argtypes = [ct.POINTER(GemmDesc), ct.c_void_p]
 
@@ -135,6 +137,18 @@ def _launch(desc: GemmDesc, device: torch.device) -> None:
     if F.lib is None:
         raise RuntimeError("libqtensor_hip.so is not available")
     F._call(lambda d, s: F.lib.qtensor_hip_gemm(d, s), device, ct.byref(desc))
+
+
+def gemm_pipe(mode: Optional[str] = None) -> str:
+    """Which matrix pipe multiplies products of dense operands, for the whole process: "f32" (fp32 MFMA) or "split"
+    (operands split into three bf16 pieces, six bf16 products per fp32 product, fp32 accumulation: fp32-grade
+    results at a multiple of the fp32 pipe's rate).  Sets the mode when given; returns the one in force before."""
+    if F.lib is None:
+        raise RuntimeError("libqtensor_hip.so is not available")
+    names = ("f32", "split")
+    if mode is not None and mode not in names:
+        raise ValueError(f"mode must be one of {names}")
+    return names[F.lib.qtensor_hip_gemm_pipe(-1 if mode is None else names.index(mode))]
 
 
 def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, alpha=1.0, beta=0.0,

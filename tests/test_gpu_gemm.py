@@ -187,11 +187,11 @@ def test_symmetric_products_compute_the_upper_half_and_mirror_it(mods, n, batch)
         assert torch.equal(o[off], o.T[off])
     plain = X.gemm(S.cuda(), P.cuda())
     sym = X.gemm(S.cuda(), P.cuda(), symmetric=True)
-    tile = torch.arange(n) // 64
-    upper_tiles = tile[:, None] <= tile[None, :]
-    # on and above the diagonal tiles both modes run the same arithmetic
+    upper = torch.arange(n)[:, None] <= torch.arange(n)[None, :]
+    # on and above the diagonal both modes run the same arithmetic (below it the symmetric mode mirrors: tile by tile,
+    # and on the split pipe inside the diagonal tiles as well)
     if n <= 192:
-        assert torch.equal(plain.cpu()[:, upper_tiles], sym.cpu()[:, upper_tiles])
+        assert torch.equal(plain.cpu()[:, upper], sym.cpu()[:, upper])
     with pytest.raises(ValueError):
         X.gemm(torch.zeros(64, 32, device="cuda"), torch.zeros(32, 48, device="cuda"), symmetric=True)
 
@@ -272,11 +272,24 @@ def test_quantizer_reading_the_transpose_equals_the_oracle_on_the_transposed_mat
 @pytest.mark.parametrize("bits,name,n,k,batch,diag", [(4, "linear-2", 768, 256, 3, True), (4, "linear-2", 320, 100, 2, True),
                                                        (8, "dynamic", 256, 512, 2, True), (4, "dynamic", 128, 64, 5, False),
                                                        (4, "linear-2", 64, 32, 4, True)])
-def test_statistics_update_encoded_in_place_equals_update_then_quantize_bit_for_bit(mods, code_maps, bits, name, n, k, batch, diag):
+@pytest.mark.parametrize("pipe", ["f32", "split"])
+def test_statistics_update_encoded_in_place_equals_update_then_quantize_bit_for_bit(mods, code_maps, bits, name, n, k, batch, diag, pipe):
     """L <- beta L + (1 - beta) G G^T (and G^T G) with the result re-encoded inside the product's epilogue: codes,
     maxima and exact diagonal must be those of the two-step path (fused product to fp32, then the stack quantizer,
-    which the other tests pin to the oracle) -- including zero, tiny, huge and NaN segments."""
+    which the other tests pin to the oracle) -- including zero, tiny, huge and NaN segments.
+
+    On both matrix pipes.  (On the split pipe a b and b a add the pieces of a product in different orders; symmetric
+    products there give every element below the diagonal the value of its partner above, whatever the tile shape,
+    so the two paths -- whose tile shapes differ -- still agree bit for bit, mirrored or multiplied out.)"""
     F, X = mods
+    before = X.gemm_pipe(pipe)
+    try:
+        _encoded_in_place_case(X, code_maps, bits, name, n, k, batch, diag)
+    finally:
+        X.gemm_pipe(before)
+
+
+def _encoded_in_place_case(X, code_maps, bits, name, n, k, batch, diag):
     g = torch.Generator().manual_seed(n + k)
     code = code_maps[(name, bits)]
     code_d = torch.from_numpy(code).cuda()
@@ -294,7 +307,9 @@ def test_statistics_update_encoded_in_place_equals_update_then_quantize_bit_for_
             one = X.quantize_stack(L0.cuda(), X.empty_quantized(batch, n, 64, bits, code_d, diag))
             kw = dict(trans_b=True) if side == 0 else dict(trans_a=True)
             half = not (side == 1 and beta == 0.0)          # once with every tile multiplied out
-            dense = X.gemm(Gd, Gd, addend=two, alpha=1.0 - beta, beta=beta, symmetric=True, **kw)
+            # (the two-step path likewise: on the split pipe an element multiplied out below the diagonal differs in
+            # its last bits from the mirror image of its partner above)
+            dense = X.gemm(Gd, Gd, addend=two, alpha=1.0 - beta, beta=beta, symmetric=half, **kw)
             X.quantize_stack(dense, two)
             got = X.gemm(Gd, Gd, addend=one, alpha=1.0 - beta, beta=beta, symmetric=half, requantize=True, **kw)
             torch.cuda.synchronize()
@@ -374,3 +389,74 @@ def test_random_shapes_strides_and_alignments_all_dense_layouts(mods):
         got = X.gemm(A, B, trans_a=ta, trans_b=tb)
         assert got.shape == (batch, m, n)
         assert rel_err(got, want) <= TOL, (case, m, n, k, batch, ta, tb, pad_a, pad_b, shift_a, shift_b)
+
+
+@pytest.mark.parametrize("batch,m,n,k", [(64, 256, 384, 64), (40, 512, 512, 1024), (6, 1024, 1024, 2048), (50, 500, 392, 336),
+                                         (3, 200, 72, 160), (1, 64, 64, 32)])
+@pytest.mark.parametrize("spread", [0.0, 3.0])
+def test_split_pipe_is_as_accurate_as_the_fp32_pipe(mods, batch, m, n, k, spread):
+    """Products of dense operands on the bf16 pipe (each operand split into three bf16 pieces, six products per fp32
+    product) against the same products on the fp32 pipe, both measured against float64 element by element in units of
+    sum_k |a_ik| |b_kj| (the scale of the rounding errors of a dot product): the split pipe must not be worse -- it
+    measures 0.7-0.9 of the fp32 pipe's error, because each MFMA instruction adds sixteen products before it rounds
+    where the fp32 instruction adds two.  All three operand layouts, every tile shape (the batch and extents decide
+    it), well scaled entries and entries spread over e^(+-9)."""
+    _, X = mods
+    g = torch.Generator().manual_seed(batch * 7 + k)
+    before = X.gemm_pipe()
+    try:
+        for trans_a, trans_b in ((False, False), (False, True), (True, False)):
+            A = torch.randn((batch, k, m) if trans_a else (batch, m, k), generator=g)
+            B = torch.randn((batch, n, k) if trans_b else (batch, k, n), generator=g)
+            A = (A * torch.exp(spread * torch.randn(A.shape, generator=g))).cuda()
+            B = (B * torch.exp(spread * torch.randn(B.shape, generator=g))).cuda()
+            a64 = (A.transpose(1, 2) if trans_a else A).double()
+            b64 = (B.transpose(1, 2) if trans_b else B).double()
+            want, scale = a64 @ b64, a64.abs() @ b64.abs()
+            out = {}
+            for pipe in ("f32", "split"):
+                X.gemm_pipe(pipe)
+                out[pipe] = X.gemm(A, B, trans_a=trans_a, trans_b=trans_b)
+            assert not torch.equal(out["f32"], out["split"])                     # the split pipe was taken
+            err = {p: ((o.double() - want).abs() / scale) for p, o in out.items()}
+            assert float(err["split"].max()) <= 1.05 * float(err["f32"].max()) + 1e-8, (trans_a, trans_b)
+            assert float(err["split"].mean()) <= 1.02 * float(err["f32"].mean()), (trans_a, trans_b)
+            assert float(err["split"].max()) <= 2e-5 and float(err["f32"].max()) <= 2e-5
+    finally:
+        X.gemm_pipe(before)
+
+
+def test_split_pipe_switch_epilogues_and_special_values(mods):
+    _, X = mods
+    before = X.gemm_pipe()
+    try:
+        assert X.gemm_pipe("f32") == before and X.gemm_pipe() == "f32"
+        assert X.gemm_pipe("split") == "f32" and X.gemm_pipe() == "split"
+        with pytest.raises(ValueError):
+            X.gemm_pipe("bf16")
+        g = torch.Generator().manual_seed(5)
+        B, n = 20, 256
+        A, Bm, E = (torch.randn(B, n, n, generator=g).cuda() for _ in range(3))
+        # fused epilogue and symmetric mirroring on the split pipe
+        got = X.gemm(A, Bm, addend=E, alpha=-0.5, beta=1.5)
+        assert rel_err(got, (1.5 * E.double() - 0.5 * (A.double() @ Bm.double())).cpu()) <= TOL
+        sym = X.gemm(A, A, trans_b=True, symmetric=True)
+        assert rel_err(sym, (A.double() @ A.double().transpose(1, 2)).cpu()) <= TOL
+        assert torch.equal(sym, sym.transpose(1, 2))                       # exactly symmetric, diagonal tiles included
+        one = X.gemm(A[:1], A[:1], trans_b=True, symmetric=True)           # a single matrix takes smaller tiles: same bits
+        assert torch.equal(one[0], sym[0])
+        # a k extent that is not a whole number of tiles goes to the fp32 pipe: same bits in both modes
+        odd = [X.gemm(A[:, :, :100].contiguous(), Bm[:, :100].contiguous()) for _ in (X.gemm_pipe("f32"), X.gemm_pipe("split"))]
+        assert torch.equal(odd[0], odd[1])
+        X.gemm_pipe("split")
+        # tiny and huge entries keep fp32 accuracy; an infinite entry poisons its row with NaN (the fp32 pipe gives inf)
+        tiny = X.gemm(A * 1e-30, Bm * 1e-5)
+        assert rel_err(tiny, ((A.double() * 1e-30) @ (Bm.double() * 1e-5)).cpu()) <= TOL
+        huge = X.gemm(A * 1e18, Bm * 1e15)
+        assert rel_err(huge, ((A.double() * 1e18) @ (Bm.double() * 1e15)).cpu()) <= TOL
+        bad = A.clone()
+        bad[3, 7, 9] = float("inf")
+        out = X.gemm(bad, Bm)
+        assert bool(out[3, 7].isnan().all()) and bool(torch.isfinite(out[3, 8]).all()) and bool(torch.isfinite(out[2]).all())
+    finally:
+        X.gemm_pipe(before)
