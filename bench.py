@@ -7,8 +7,8 @@ on one MI355X, reported as achieved HBM GB/s over the algorithmic bytes.
 One "step" = one quantize launch + one dequantize launch over the whole tensor, inputs
 resident in HBM.  The same JSON line also carries, under "precond_step", the second half of the
 metric: ms per full 4-bit Shampoo2 step (eigenbasis variant, coupled-Newton inverse roots) over the
-ViT-B/32 weight shapes, with its own roofline entry (the batched fp32 MFMA product that dominates
-it) and the CPU restatement timed on a bounded sample beside it; under "precond_step_naive" the
+ViT-B/32 weight shapes, with its own roofline entry (the batched product of fp32 matrices that dominates
+it: on the bf16 matrix pipe with split operands, fp32-grade results; the fp32 pipe's rate beside it) and the CPU restatement timed on a bounded sample beside it; under "precond_step_naive" the
 same for the variant that stores the statistics themselves; under "fused_gemm" the fused
 dequantize -> MFMA products deq(L) G deq(R) against the fp32 matrix peak; under "other_formats"
 the 8-bit and blocksize-256 variants of the headline tensor.  Prints one JSON line.
@@ -132,6 +132,10 @@ def precond_step_gpu(torch, variant="shampoo1"):
         more["matrices_redone_with_library_qr"] = bank.qr_fallbacks
         more["cholesky_qr_rounds_per_stack_and_update"] = round(bank.qr_rounds / (30 * len(bank.per_order)), 2)
         more["subspace_iteration_updates"] = 30 * sum(bank.per_order.values())
+    import qtensor.fused as X
+    more["gemm_pipe"] = ("products of dense fp32 operands on the %s matrix pipe" %
+                         ("bf16 (operands split into three bf16 pieces, six products per fp32 product, fp32 accumulation)"
+                          if X.gemm_pipe() == "split" else "fp32"))
     return {
         **more,
         "workload": "ViT-B/32 2-D weights (50 parameters, %d blocks of at most 1024, %d quantized statistics and as many "
@@ -276,32 +280,55 @@ def precond_step_cpu(torch, code_host, variant):
     }
 
 
+BF16_MATRIX_PEAK_TFLOPS = 2500.0
+SPLIT_PRODUCTS = 6            # bf16 products that make one fp32 product on the split pipe
+
+
 def dominant_product_gpu(torch):
-    """The kernel most of a step's time goes to -- gemm_kernel<128,128,dense,dense,store>, the batched plain fp32
-    product (L Q, the Newton products, the solve panels) -- on the step's biggest stack (99 statistics of order
-    1024), timed per launch with events on the launch stream."""
+    """The kernel most of a step's time goes to -- gemm_kernel<128,128,dense,dense,store>, the batched plain product
+    of fp32 matrices (L Q, the Newton products, the projections of the Gram-Schmidt sweep) -- on the step's biggest
+    stack (99 statistics of order 1024), timed per launch with events on the launch stream, on both matrix pipes.
+    The default pipe splits every fp32 operand into three bf16 pieces and takes six bf16 MFMA products per fp32
+    product (fp32 accumulation, fp32-grade results): its roofline is the bf16 matrix peak over six."""
     import qtensor.fused as X
     g = torch.Generator(device="cuda").manual_seed(5)
     batch, n = 99, 1024
     A = torch.randn(batch, n, n, device="cuda", generator=g)
     B = torch.randn(batch, n, n, device="cuda", generator=g)
     C = torch.empty(batch, n, n, device="cuda")
-    for _ in range(3):
-        X.gemm(A, B, out=C)
-    reps = 10
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
-    ev[0].record()
-    for i in range(reps):
-        X.gemm(A, B, out=C)
-        ev[i + 1].record()
-    torch.cuda.synchronize()
-    ms = sum(ev[i].elapsed_time(ev[i + 1]) for i in range(reps)) / reps
     flop = 2.0 * batch * n ** 3
-    tf = flop / (ms * 1e-3) / 1e12
-    return {"bound": "mfma", "kernel": "gemm_kernel<128,128,dense,dense,store> on 99 x (1024 x 1024 x 1024)",
-            "achieved": round(tf, 1), "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(tf / FP32_MATRIX_PEAK_TFLOPS, 4), "traffic": None, "avg_launch_ms": round(ms, 4),
-            "algorithmic_flop_per_launch": flop}
+    reps = 10
+
+    def rate():
+        for _ in range(20):                      # the clocks settle over the first dozen launches
+            X.gemm(A, B, out=C)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+        ev[0].record()
+        for i in range(reps):
+            X.gemm(A, B, out=C)
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        ms = sum(ev[i].elapsed_time(ev[i + 1]) for i in range(reps)) / reps
+        return ms, flop / (ms * 1e-3) / 1e12
+
+    before = X.gemm_pipe("f32")
+    try:
+        ms32, tf32 = rate()
+        X.gemm_pipe("split")
+        ms, tf = rate()
+    finally:
+        X.gemm_pipe(before)
+    peak = BF16_MATRIX_PEAK_TFLOPS / SPLIT_PRODUCTS
+    return {"bound": "mfma", "kernel": "gemm_kernel<128,128,dense,dense,store,split> on 99 x (1024 x 1024 x 1024)",
+            "achieved": round(tf, 1), "peak": round(peak, 1), "unit": "TFLOP/s", "frac": round(tf / peak, 4), "traffic": None,
+            "avg_launch_ms": round(ms, 4), "algorithmic_flop_per_launch": flop,
+            "pipe": "v_mfma_f32_32x32x16_bf16 on operands split into three bf16 pieces: %d bf16 products per fp32 product, "
+                    "so peak = bf16 dense peak %.0f / %d; achieved counts the algorithmic fp32 flops (2 m n k)"
+                    % (SPLIT_PRODUCTS, BF16_MATRIX_PEAK_TFLOPS, SPLIT_PRODUCTS),
+            "bf16_mfma_tflops": round(tf * SPLIT_PRODUCTS, 1),
+            "fp32_pipe": {"kernel": "gemm_kernel<128,128,dense,dense,store> (v_mfma_f32_32x32x2_f32)", "achieved": round(tf32, 1),
+                          "peak": FP32_MATRIX_PEAK_TFLOPS, "frac": round(tf32 / FP32_MATRIX_PEAK_TFLOPS, 4),
+                          "avg_launch_ms": round(ms32, 4)}}
 
 
 def main():
@@ -315,6 +342,8 @@ def main():
     ap.add_argument("--bank-streams", type=int, default=None,
                     help="side streams of the batched preconditioner engine (0 serialises its launches, which "
                          "keeps per-kernel durations in a profile free of overlap)")
+    ap.add_argument("--gemm-pipe", choices=["f32", "split"], default=None,
+                    help="matrix pipe of the products of dense operands (default: the library's, the split bf16 pipe)")
     ap.add_argument("--no-step", action="store_true", help="skip the fused-product, other-format and Shampoo-step measurements")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -330,12 +359,16 @@ def main():
 
     code_host = F.create_linear_map(True, BITS, 2)
     code = code_host.cuda()
+    if args.gemm_pipe is not None:
+        import qtensor.fused as X
+        X.gemm_pipe(args.gemm_pipe)
     if args.bank_streams is not None:
         from optimizers.engine import ShampooBank
         ShampooBank.DEFAULT_STREAMS = args.bank_streams
         if args.bank_streams == 0:           # profiling: nothing may overlap, the side thread of shampoo2 neither
             from optimizers import shampoo2
             shampoo2.ShampooAdamW.overlap_unbatched_statistics = False
+            shampoo2.ShampooAdamW.overlap_precondition = False
     if args.section in ("gemm", "step", "step2", "product"):
         if args.section == "gemm":
             part = {"fused_gemm": fused_gemm_gpu(torch, code)}
