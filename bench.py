@@ -311,6 +311,23 @@ def dominant_product_gpu(torch):
         ms = sum(ev[i].elapsed_time(ev[i + 1]) for i in range(reps)) / reps
         return ms, flop / (ms * 1e-3) / 1e12
 
+    def pipe_alone(pipe):
+        """TFLOP/s of a launch that is nothing but matrix instructions on register operands of random bits."""
+        import ctypes as ct
+        import qtensor.functional as F
+        F.lib.qtensor_hip_mfma_rate_flop.restype = ct.c_double
+        F.lib.qtensor_hip_mfma_rate_flop.argtypes = [ct.c_int, ct.c_int, ct.c_int, ct.c_void_p, ct.c_void_p]
+        sink = torch.zeros(1, device="cuda")
+        stream = torch.cuda.current_stream().cuda_stream
+        rounds = 20000 if pipe == 1 else 5000
+        F.lib.qtensor_hip_mfma_rate_flop(pipe, rounds, 3, sink.data_ptr(), stream)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        done = F.lib.qtensor_hip_mfma_rate_flop(pipe, rounds, 3, sink.data_ptr(), stream)
+        e1.record()
+        torch.cuda.synchronize()
+        return done / (e0.elapsed_time(e1) * 1e-3) / 1e12
+
     before = X.gemm_pipe("f32")
     try:
         ms32, tf32 = rate()
@@ -326,6 +343,10 @@ def dominant_product_gpu(torch):
                     "so peak = bf16 dense peak %.0f / %d; achieved counts the algorithmic fp32 flops (2 m n k)"
                     % (SPLIT_PRODUCTS, BF16_MATRIX_PEAK_TFLOPS, SPLIT_PRODUCTS),
             "bf16_mfma_tflops": round(tf * SPLIT_PRODUCTS, 1),
+            "matrix_instructions_alone": {
+                "what": "one launch of nothing but matrix instructions on register operands of random bits, three "
+                        "workgroups per compute unit: the rate each pipe sustains at the clock it holds under that load",
+                "bf16_tflops": round(pipe_alone(1), 1), "fp32_tflops": round(pipe_alone(0), 1)},
             "fp32_pipe": {"kernel": "gemm_kernel<128,128,dense,dense,store> (v_mfma_f32_32x32x2_f32)", "achieved": round(tf32, 1),
                           "peak": FP32_MATRIX_PEAK_TFLOPS, "frac": round(tf32 / FP32_MATRIX_PEAK_TFLOPS, 4),
                           "avg_launch_ms": round(ms32, 4)}}

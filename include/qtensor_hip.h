@@ -228,6 +228,13 @@ void qtensor_hip_gemm_static(const qtensor_gemm_desc *desc, qtensor_stream_t str
  * variable QT_GEMM_PIPE is "f32". */
 int qtensor_hip_gemm_pipe(int mode);
 
+/* Yardstick for the product kernels (no counterpart in the reference): one launch in which every wave of
+ * workgroups_per_unit workgroups per compute unit does nothing but matrix instructions on register operands of
+ * pseudo-random bits -- per round 24 x v_mfma_f32_32x32x16_bf16 (pipe 1) or 32 x v_mfma_f32_32x32x2_f32 (pipe 0).
+ * Returns the floating-point operations of the launch (0 and the error slot on bad arguments); time it with
+ * events: the rate is what the pipe sustains at the clock it holds under that load.  `sink`: a device word. */
+double qtensor_hip_mfma_rate_flop(int pipe, int rounds, int workgroups_per_unit, float *sink, qtensor_stream_t stream);
+
 /* ---- batched Cholesky factorisation and triangular solve (Cholesky QR) ---------------------------
  * Replace, for a whole stack of statistics at once, the QR factorisation the reference calls per
  * matrix in QTensorSVDFast.quantize (torch.linalg.qr, qtensor/utils.py:157): one round of

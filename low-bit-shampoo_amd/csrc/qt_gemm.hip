@@ -1070,6 +1070,51 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
   }
 }
 
+// What the matrix pipes sustain with nothing else going on: every wave multiplies register operands of pseudo-random
+// bits (the power a pipe draws, and with it the clock it holds, depends on how many bits toggle) into four accumulator
+// blocks, 24 bf16 instructions (32x32x16) or 32 fp32 instructions (32x32x2) per round.  A yardstick for the rates of the
+// product kernels beside the published peaks.
+template <int PIPE>
+__global__ __launch_bounds__(256) void mfma_rate_kernel(float *sink, int rounds) {
+    f32x16 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
+    auto noise = [&](uint32_t q) {                          // in (-0.5, 0.5), different per lane, register and block
+        uint32_t h = (threadIdx.x * 2654435761u) ^ (q * 40503u + blockIdx.x * 7919u);
+        h ^= h >> 13; h *= 0x5bd1e995u; h ^= h >> 15;
+        return (float)(int)(h & 0xffffu) / 65536.0f - 0.5f;
+    };
+    if constexpr (PIPE == kPipeSplit) {
+        qt_bf16x8 a[6], b[6];
+#pragma unroll
+        for (int q = 0; q < 6; ++q)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { a[q][e] = (__bf16)noise(16 * q + e); b[q][e] = (__bf16)noise(16 * q + 8 + e); }
+        for (int it = 0; it < rounds; ++it)
+#pragma unroll
+            for (int q = 0; q < 6; ++q)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[q], b[(q + i) % 6], acc[i], 0, 0, 0);
+    } else {
+        float a[8], b[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) { a[q] = noise(2 * q); b[q] = noise(2 * q + 1); }
+        for (int it = 0; it < rounds; ++it)
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[q], b[(q + i) % 8], acc[i], 0, 0, 0);
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s += acc[i][r];
+    if (s == 12345.678f) sink[0] = s;                       // keeps the products alive; practically never taken
+}
+
 // Streamed products: out tile = sum of its pieces in the workspace, in the order of their k ranges.  A tile that
 // one workgroup did as a whole is already in place.  Grid (tiles, 4 row bands of the tile).
 __global__ __launch_bounds__(256) void reduce_pieces_kernel(const float *workspace, BatchPtr C, int ldc, int M, int N, int bm, int bn,
@@ -1234,6 +1279,20 @@ std::atomic<int> &pipe_mode_slot() {
 }
 int gemm_pipe_mode() { return pipe_mode_slot().load(std::memory_order_relaxed); }
 }  // namespace
+
+extern "C" double qtensor_hip_mfma_rate_flop(int pipe, int rounds, int workgroups_per_unit, float *sink, void *stream_v) {
+    using namespace qt;
+    clear_error();
+    if ((pipe != kPipeF32 && pipe != kPipeSplit) || rounds < 1 || workgroups_per_unit < 1 || workgroups_per_unit > 8 || sink == nullptr) {
+        set_error(kBadArgument, "mfma_rate: pipe 0 or 1, rounds >= 1, 1..8 workgroups per unit, a device word to write to");
+        return 0.0;
+    }
+    const unsigned grid = (unsigned)(compute_units() * workgroups_per_unit);
+    if (pipe == kPipeSplit) hipLaunchKernelGGL(mfma_rate_kernel<kPipeSplit>, dim3(grid), dim3(256), 0, (hipStream_t)stream_v, sink, rounds);
+    else hipLaunchKernelGGL(mfma_rate_kernel<kPipeF32>, dim3(grid), dim3(256), 0, (hipStream_t)stream_v, sink, rounds);
+    // multiply-adds x 2 of one launch: 4 waves, per round 24 instructions of 32x32x16 or 32 of 32x32x2
+    return (double)grid * 4.0 * rounds * (pipe == kPipeSplit ? 24.0 * 32768.0 : 32.0 * 4096.0);
+}
 
 extern "C" int qtensor_hip_gemm_pipe(int mode) {
     qt::clear_error();
