@@ -102,6 +102,10 @@ class ShampooBank:
                 g.slot[side] = (order, per_order[order])
                 per_order[order] += len(g)
         self.per_order = dict(per_order)
+        too_many = {o: c for o, c in self.per_order.items() if c > 65535}
+        if too_many:
+            raise ValueError(f"the batched engine takes at most 65535 blocks per order in one launch, got {too_many}; "
+                             "use a larger prec_maxorder or the per-parameter path (fused=False)")
         self.precs = {}
         for order, count in per_order.items():
             eye = torch.eye(order, device=self.device).expand(count, order, order)

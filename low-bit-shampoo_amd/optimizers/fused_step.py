@@ -11,6 +11,12 @@ class _FusedStep:
     """fused=True (not in the reference) runs all eligible GPU parameters through one batched
     ShampooBank instead of one Preconditioner object per parameter; the arithmetic is the same.
 
+    Differences from the reference's step(), which walks the parameters one by one and skips those without a
+    gradient (optimizers/shampoo1.py:371-377): the parameters that have a gradient at the first step form the bank,
+    and every one of them needs a gradient at every later step (RuntimeError otherwise); state['step'] is the
+    group's step count for every parameter, so a parameter that first gets a gradient later shares the group's
+    bias corrections and schedules.
+
     Checkpoints: state_dict() then carries, next to torch's usual entries, 'shampoo_bank': one
     dict of plain tensors per parameter group -- per block order n the stacked 4/8-bit
     preconditioners ('precs.n.codes' uint8 [count, n*n*bits/8] with the first element of a pair in
@@ -19,8 +25,11 @@ class _FusedStep:
     'basis.n.absmax', 'basis.n.svalue' fp32 [count, n/2], 'basis.n.keep' int64 [count, n/2],
     'basis.n.max_eigenvalue' fp32 [count]), 'block_table' int64 [statistics, 5] = (parameter index
     in the group, block index within the parameter, side, order, row in that order's stack), and
-    the step count.  Nothing in it is a pickled Python object, so
-    torch.load(..., weights_only=True) reads it."""
+    the step count.  Nothing in 'shampoo_bank' is a pickled Python object, so torch.load(..., weights_only=True) reads
+    that part; parameters outside the bank (an order that the blocksize does not divide, non-fp32 tensors) keep the
+    reference's state['preconditioner'] object in the usual per-parameter state, which needs weights_only=False like
+    the reference's own checkpoints.  A checkpoint with 'shampoo_bank' can only be loaded into an optimizer built with
+    fused=True (ValueError otherwise: the banked parameters have no per-parameter preconditioner state)."""
 
     _update = None                 # _adamw_update or _sgd_update
     bank_keys = ()                 # group entries handed to the bank besides the common ones
@@ -73,6 +82,9 @@ class _FusedStep:
     def load_state_dict(self, state_dict):
         state_dict = dict(state_dict)
         banks = state_dict.pop('shampoo_bank', None)
+        if banks is not None and any(b is not None for b in banks) and not self._fused:
+            raise ValueError("this checkpoint was written by an optimizer with fused=True (it carries 'shampoo_bank'); "
+                             "load it into an optimizer constructed with fused=True")
         super().load_state_dict(state_dict)
         if banks is not None:
             self.__dict__.pop('_fused_cache', None)          # rebuilt, then filled, by the next step
@@ -109,6 +121,9 @@ def fused_step(opt, group, update, group_index=0):
                     raise ValueError("checkpoint was written for other parameter shapes or block sizes")
                 bank.load_state_dict(saved)
             pending[group_index] = None
+    if any(p.grad is None for p in entry['banked']):                  # before anything of this step is counted or launched
+        raise RuntimeError("fused=True batches the parameters that had a gradient at the first step; "
+                           "every one of them needs a gradient at every later step")
     entry['step'] += 1
     step, bank, banked = entry['step'], entry['bank'], entry['banked']
     for p in params:
@@ -117,9 +132,6 @@ def fused_step(opt, group, update, group_index=0):
         if id(p) not in entry['ids'] and 'preconditioner' not in state:      # first gradient after the bank was built
             state['preconditioner'] = opt._make_preconditioner(p, group)
     grads = {id(p): p.grad.contiguous() for p in params}
-    if any(id(p) not in grads for p in banked):
-        raise RuntimeError("fused=True batches the parameters that had a gradient at the first step; "
-                           "every one of them needs a gradient at every later step")
     directions, grafted = {}, set()
     unbatched = [p for p in params if id(p) not in entry['ids']]
     side_job, roots_done, statistics_done = None, False, False

@@ -34,7 +34,8 @@ class TailPlan:
         self.partial = None
 
     def _prepare(self, params, dirs, grads, m, v, graft):
-        key = tuple((p.data_ptr(), d.data_ptr(), g.data_ptr(), a.data_ptr(), 0 if b is None else b.data_ptr(), bool(f))
+        # (the gradient's address only where the row is grafted: the kernels do not read it otherwise)
+        key = tuple((p.data_ptr(), d.data_ptr(), g.data_ptr() if f else 0, a.data_ptr(), 0 if b is None else b.data_ptr(), bool(f))
                     for p, d, g, a, b, f in zip(params, dirs, grads, m, v, graft))
         if key == self.key:
             return
@@ -59,7 +60,11 @@ class TailPlan:
         self.n_chunks = first
         self.any_graft = any(graft)
         self.key = key
-        self.keep = (list(params), list(dirs), list(grads), list(m), list(v))     # the table holds raw addresses
+        # The table holds raw addresses.  Parameters and moment buffers are kept alive here; gradients and directions
+        # are not: they are only read by the launch that follows, while their owners still hold them, and keeping
+        # them would pin one full set of gradients after zero_grad(set_to_none=True).  A tensor that comes back at
+        # another address changes the key and the table is rebuilt.
+        self.keep = (list(params), list(m), list(v))
 
     def adamw(self, params, dirs, grads, exp_avg, exp_avg_sq, graft, lr, betas, eps, weight_decay, step):
         self._prepare(params, dirs, grads, exp_avg, exp_avg_sq, graft)

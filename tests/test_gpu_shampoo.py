@@ -269,3 +269,35 @@ def test_fused_optimizer_checkpoint_round_trip(setup, which, monkeypatch):
     other[0].grad = torch.ones(128, 64, device="cuda")
     with pytest.raises(ValueError):
         opt3.step()
+
+
+def test_fused_step_error_paths_that_differ_from_the_per_parameter_step(setup):
+    """What fused=True does where the reference's step() would skip a parameter, and what it refuses to load."""
+    S1 = setup[0]
+    g = torch.Generator().manual_seed(8)
+    params = [torch.nn.Parameter(torch.rand(s, generator=g).cuda()) for s in SHAPES]
+    opt = S1.ShampooAdamW(params, lr=1e-2, start_prec_step=2, stat_compute_steps=1, prec_compute_steps=2, fused=True, **KW)
+    for p in params:
+        p.grad = 0.02 * torch.randn(p.shape, generator=g).cuda()
+    opt.step()
+    assert all(opt.state[p]["step"] == 1 for p in params)
+    # a banked parameter without a gradient on a later step: refused, nothing is skipped silently
+    before = [p.detach().clone() for p in params]
+    params[0].grad = None
+    with pytest.raises(RuntimeError, match="needs a gradient at every later step"):
+        opt.step()
+    assert all(torch.equal(a, p.detach()) for a, p in zip(before, params))           # and nothing was updated
+    # a checkpoint of the fused optimizer does not load into the per-parameter one
+    params[0].grad = 0.02 * torch.randn(params[0].shape, generator=g).cuda()
+    sd = opt.state_dict()
+    plain = S1.ShampooAdamW([torch.nn.Parameter(p.detach().clone()) for p in params], lr=1e-2, start_prec_step=2,
+                            stat_compute_steps=1, prec_compute_steps=2, fused=False, **KW)
+    with pytest.raises(ValueError, match="fused=True"):
+        plain.load_state_dict(sd)
+    # more blocks of one order than one launch takes
+    from optimizers.engine import ShampooBank
+    import qtensor.functional as F
+    many = [torch.nn.Parameter(torch.zeros(64 * 65536, 64, device="meta"))]
+    with pytest.raises((ValueError, NotImplementedError, RuntimeError)):
+        ShampooBank(many, {"code": F.create_linear_map(True, 4, 2)}, "code", prec_maxorder=64, prec_bits=4, min_lowbit_size=4096,
+                    quan_blocksize=64)
