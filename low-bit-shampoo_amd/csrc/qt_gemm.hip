@@ -512,6 +512,19 @@ struct LoadQuant {
             d[1] = make_float4(v[4], v[5], v[6], v[7]);
         }
     }
+    // Split pipe, left factor: a group is 8 consecutive k of one tile row, which is what a lane's fragment reads.
+    __device__ __forceinline__ void commit_split(unsigned char *operand, const float *s_code) const {
+        static_assert(ALONG_K, "the right factor's groups run along the tile rows");
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g) {
+            if (!active(g)) continue;
+            int tr, tc;
+            locate(g, tr, tc);
+            float v[8];
+            expand(g, s_code, v);
+            commit_split_eight<ROWS>(operand, tr, tc >> 3, v);
+        }
+    }
 };
 
 template <int BM, int BN, int KA, int KB, int EPI, int PREC = kPipeF32>
@@ -545,7 +558,7 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     const int slice = id % slices;
     id /= slices;
     constexpr bool kSplit = PREC == kPipeSplit;
-    static_assert(!kSplit || (KA < kQuant4 && KB < kQuant4), "split pipe: dense operands");
+    static_assert(!kSplit || KB < kQuant4, "split pipe: dense operands, or a quantized left factor");
     using PlainA = typename std::conditional<KA == kDense, LoadKContig<BM>,
         typename std::conditional<KA == kDenseT, LoadRowContig<BM>,
             LoadQuant<BM, KA == kQuant4 ? 4 : 8, true>>::type>::type;
@@ -553,7 +566,7 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
         typename std::conditional<KB == kDenseT, LoadKContig<BN>,
             LoadQuant<BN, KB == kQuant4 ? 4 : 8, false>>::type>::type;
     constexpr int SPLIT_ROWS_A = BM, SPLIT_ROWS_B = BN;
-    using LoaderA = typename std::conditional<!kSplit, PlainA,
+    using LoaderA = typename std::conditional<!kSplit || KA >= kQuant4, PlainA,
         typename std::conditional<KA == kDense, SplitKContig<SPLIT_ROWS_A>, SplitRowContig<SPLIT_ROWS_A>>::type>::type;
     using LoaderB = typename std::conditional<!kSplit, PlainB,
         typename std::conditional<KB == kDense, SplitRowContig<SPLIT_ROWS_B>, SplitKContig<SPLIT_ROWS_B>>::type>::type;
@@ -630,7 +643,8 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     const bool whole_k = args.K % BK == 0;
     bool a_fast = false, b_fast = false;
     if constexpr (kSplit) {                    // the host only picks this pipe where the fast loads apply
-        la.prepare(args.lda, m0, args.M);
+        if constexpr (KA >= kQuant4) la.prepare(args.Aq, b, m0);
+        else la.prepare(args.lda, m0, args.M);
         lb.prepare(args.ldb, n0, args.N);
         if constexpr (KA == kDense) la.vec = a_vec;
         if constexpr (KB == kDenseT) lb.vec = b_vec;
@@ -650,7 +664,8 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     }
     auto fetch = [&](int k0) {
         if constexpr (kSplit) {
-            la.fetch_fast(A + (KA == kDense ? (long long)k0 : (long long)k0 * args.lda));
+            if constexpr (KA >= kQuant4) la.fetch(k0);
+            else la.fetch_fast(A + (KA == kDense ? (long long)k0 : (long long)k0 * args.lda));
             lb.fetch_fast(B + (KB == kDenseT ? (long long)k0 : (long long)k0 * args.ldb));
         } else {
             if constexpr (KA < kQuant4) {
@@ -666,7 +681,8 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     auto commit = [&](int stage) {
         if constexpr (kSplit) {
             unsigned char *at = reinterpret_cast<unsigned char *>(s_mem) + stage * SPLIT_STAGE;
-            la.commit_split(at);
+            if constexpr (KA >= kQuant4) la.commit_split(at, s_code);
+            else la.commit_split(at);
             lb.commit_split(at + SPLIT_A);
         } else {
             la.commit(s_a[stage], s_code);
@@ -1398,8 +1414,8 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
     // The split pipe: for dense operands in whole k tiles, where the offsets of its loads fit 31 bits -- whatever the
     // tile shape, so that the bits of a product do not depend on how it is tiled.
     bool split_pipe = false;
-    if (gemm_pipe_mode() == kPipeSplit && ka < kQuant4 && kb < kQuant4 && d->K % BK == 0 && d->K >= 2 * BK) {
-        const long long reach_a = ka == kDense ? (long long)d->M * a.lda : (long long)BK * a.lda + d->M;
+    if (gemm_pipe_mode() == kPipeSplit && kb < kQuant4 && d->K % BK == 0 && d->K >= 2 * BK) {
+        const long long reach_a = ka >= kQuant4 ? 0 : ka == kDense ? (long long)d->M * a.lda : (long long)BK * a.lda + d->M;
         const long long reach_b = kb == kDenseT ? (long long)d->N * a.ldb : (long long)BK * a.ldb + d->N;
         split_pipe = reach_a < 0x7fffffffLL && reach_b < 0x7fffffffLL;
     }
@@ -1509,9 +1525,22 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         else if (pick == 2) launch_gemm<64, 128, KA, KB, EP>(a, d->batch, stream);                           \
         else launch_gemm<64, 64, KA, KB, EP>(a, d->batch, stream);                                           \
         break;
+#define QT_GEMM_CASE_LEFT(KA, KB, EP)                                                                        \
+    case (KA) * 100 + (KB) * 10 + (EP):                                                                      \
+        if (split_pipe) {                                                                                    \
+            if (pick == 0) launch_gemm<128, 128, KA, KB, EP, kPipeSplit>(a, d->batch, stream);               \
+            else if (pick == 1) launch_gemm<128, 64, KA, KB, EP, kPipeSplit>(a, d->batch, stream);           \
+            else if (pick == 2) launch_gemm<64, 128, KA, KB, EP, kPipeSplit>(a, d->batch, stream);           \
+            else launch_gemm<64, 64, KA, KB, EP, kPipeSplit>(a, d->batch, stream);                           \
+        }                                                                                                    \
+        else if (pick == 0) launch_gemm<128, 128, KA, KB, EP>(a, d->batch, stream);                          \
+        else if (pick == 1) launch_gemm<128, 64, KA, KB, EP>(a, d->batch, stream);                           \
+        else if (pick == 2) launch_gemm<64, 128, KA, KB, EP>(a, d->batch, stream);                           \
+        else launch_gemm<64, 64, KA, KB, EP>(a, d->batch, stream);                                           \
+        break;
     switch (combo) {
-        QT_GEMM_CASE(kQuant4, kDense, kStore)
-        QT_GEMM_CASE(kQuant8, kDense, kStore)
+        QT_GEMM_CASE_LEFT(kQuant4, kDense, kStore)
+        QT_GEMM_CASE_LEFT(kQuant8, kDense, kStore)
         QT_GEMM_CASE(kDense, kQuant4, kStore)
         QT_GEMM_CASE(kDense, kQuant8, kStore)
         QT_GEMM_CASE_DENSE(kDense, kDenseT, kStore)
