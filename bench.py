@@ -10,7 +10,7 @@ metric: ms per full 4-bit Shampoo2 step (eigenbasis variant, coupled-Newton inve
 ViT-B/32 weight shapes, with its own roofline entry (the batched product of fp32 matrices that dominates
 it: on the bf16 matrix pipe with split operands, fp32-grade results; the fp32 pipe's rate beside it) and the CPU restatement timed on a bounded sample beside it; under "precond_step_naive" the
 same for the variant that stores the statistics themselves; under "fused_gemm" the fused
-dequantize -> MFMA products deq(L) G deq(R) against the fp32 matrix peak; under "other_formats"
+dequantize -> MFMA products deq(L) G deq(R) on both matrix pipes; under "other_formats"
 the 8-bit and blocksize-256 variants of the headline tensor.  Prints one JSON line.
 """
 import argparse
@@ -154,6 +154,8 @@ def precond_step_gpu(torch, variant="shampoo1"):
 
 
 FP32_MATRIX_PEAK_TFLOPS = 157.3
+BF16_MATRIX_PEAK_TFLOPS = 2500.0
+SPLIT_PRODUCTS = 6            # bf16 products that make one fp32 product on the split pipe
 
 
 def fused_gemm_gpu(torch, code):
@@ -178,25 +180,42 @@ def fused_gemm_gpu(torch, code):
         X.gemm(Lq, G, out=half)
         X.gemm(half, Rq, out=out)
 
-    for _ in range(3):
-        run()
-    reps = 20
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
-    ev[0].record()
-    for i in range(reps):
-        run()
-        ev[i + 1].record()
-    torch.cuda.synchronize()
-    ms = sum(ev[i].elapsed_time(ev[i + 1]) for i in range(reps)) / reps
     flop = 2.0 * m * m * n + 2.0 * m * n * n
-    tf = flop / (ms * 1e-3) / 1e12
+
+    def rate():
+        for _ in range(10):
+            run()
+        reps = 20
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+        ev[0].record()
+        for i in range(reps):
+            run()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        ms = sum(ev[i].elapsed_time(ev[i + 1]) for i in range(reps)) / reps
+        return ms, flop / (ms * 1e-3) / 1e12
+
+    before = X.gemm_pipe("f32")
+    try:
+        ms32, tf32 = rate()
+        X.gemm_pipe("split")
+        ms, tf = rate()
+    finally:
+        X.gemm_pipe(before)
+    peak = BF16_MATRIX_PEAK_TFLOPS / SPLIT_PRODUCTS
     return {
         "workload": "deq(Lq 768x768) @ G(768x3072) @ deq(Rq 3072x3072), 4-bit linear-2 blocksize 64 factors with exact "
-                    "diagonal, fp32 MFMA (v_mfma_f32_32x32x2_f32), two fused launches",
+                    "diagonal, expanded inside the two product launches; bf16 MFMA on operands split into three bf16 "
+                    "pieces (six products per fp32 product, fp32 accumulation)",
         "ms": round(ms, 4),
         "gflop": round(flop / 1e9, 2),
-        "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tf / FP32_MATRIX_PEAK_TFLOPS, 4), "traffic": None},
+        "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": round(peak, 1), "unit": "TFLOP/s",
+                     "frac": round(tf / peak, 4), "traffic": None,
+                     "pipe": "peak = bf16 dense peak %.0f / %d products; achieved counts the algorithmic fp32 flops"
+                             % (BF16_MATRIX_PEAK_TFLOPS, SPLIT_PRODUCTS),
+                     "achieved_over_fp32_matrix_peak": round(tf / FP32_MATRIX_PEAK_TFLOPS, 4),
+                     "fp32_pipe": {"ms": round(ms32, 4), "achieved": round(tf32, 1), "peak": FP32_MATRIX_PEAK_TFLOPS,
+                                   "frac": round(tf32 / FP32_MATRIX_PEAK_TFLOPS, 4)}},
     }
 
 
@@ -278,10 +297,6 @@ def precond_step_cpu(torch, code_host, variant):
                      " and QR" if variant == "shampoo2" else "", torch.get_num_threads()),
         "seconds_for_sample": round(regular, 3),
     }
-
-
-BF16_MATRIX_PEAK_TFLOPS = 2500.0
-SPLIT_PRODUCTS = 6            # bf16 products that make one fp32 product on the split pipe
 
 
 def dominant_product_gpu(torch):

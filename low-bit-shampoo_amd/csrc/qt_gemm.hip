@@ -405,8 +405,11 @@ struct SplitRowContig {
 // Quantized square matrix (order x order, flat layout).  ALONG_K: the tile's k runs along the
 // matrix columns (left factor); otherwise the tile's rows run along the matrix columns (right
 // factor).  Each thread expands 8 consecutive codes of one matrix row.
-template <int ROWS, int BITS, bool ALONG_K>
+// TURNED (split pipe, right factor): the 8 lanes of a group take 8 consecutive k, so that a group holds an 8 x 8 square
+// (k x tile row) which one pass through LDS turns around into 8 consecutive k per tile row.
+template <int ROWS, int BITS, bool ALONG_K, bool TURNED = false>
 struct LoadQuant {
+    static_assert(!(TURNED && ALONG_K), "only the right factor is turned");
     static constexpr bool kRowMajor = ALONG_K;               // 8 consecutive k of one row: [row][k]; else [k][row]
     static constexpr int TOTAL = ROWS * BK / 8;              // 8-element groups in the tile
     static constexpr int GROUPS = (TOTAL + 255) / 256;       // per thread
@@ -428,6 +431,11 @@ struct LoadQuant {
     __device__ __forceinline__ void locate(int g, int &mr, int &mc) const {
         const int f = threadIdx.x + g * 256;
         if (ALONG_K) { mr = f % ROWS; mc = (f / ROWS) << 3; }               // tile row = matrix row, 2 groups per row
+        else if (TURNED) {                                                  // wave: half of k and 64 tile rows; lane: k and group
+            const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+            mr = 8 * (wave & 1) + (lane & 7);
+            mc = (8 * (wave >> 1) + ((lane >> 3) & 7)) << 3;
+        }
         else { mr = f / (ROWS / 8); mc = (f % (ROWS / 8)) << 3; }           // tile k = matrix row
     }
     __device__ __forceinline__ void prepare(const QuantRef &q, int b, int row0) {
@@ -512,23 +520,69 @@ struct LoadQuant {
             d[1] = make_float4(v[4], v[5], v[6], v[7]);
         }
     }
-    // Split pipe, left factor: a group is 8 consecutive k of one tile row, which is what a lane's fragment reads.
-    __device__ __forceinline__ void commit_split(unsigned char *operand, const float *s_code) const {
-        static_assert(ALONG_K, "the right factor's groups run along the tile rows");
-#pragma unroll
-        for (int g = 0; g < GROUPS; ++g) {
-            if (!active(g)) continue;
-            int tr, tc;
-            locate(g, tr, tc);
-            float v[8];
-            expand(g, s_code, v);
+    // Split pipe.  Left factor: a group is 8 consecutive k of one tile row, which is what a lane's fragment reads.
+    // Right factor (TURNED): a group is 8 consecutive tile rows at one k; the 8 lanes of a group write their 8 x 8 square
+    // into the wave's own part of the operand (64 tile rows of one half of k: 1 KiB in each of the three planes, used
+    // as fp32 scratch first), read it back the other way round, and only then split and store: all inside the wave.
+    __device__ __forceinline__ void commit_split(unsigned char *operand, const float *s_code) {
+        static_assert(ALONG_K || TURNED, "the right factor's groups must be turned");
+        static_assert(GROUPS == 1, "one group per thread");
+        if (!active(0)) return;                               // whole waves
+        int tr, tc;
+        locate(0, tr, tc);
+        float v[8];
+        expand(0, s_code, v);
+        if constexpr (ALONG_K) {
             commit_split_eight<ROWS>(operand, tr, tc >> 3, v);
+        } else {
+            stage_values(operand, v);
+            turn(operand);
+            finish(operand);
         }
+    }
+    // The three phases of the turned commit, so that the caller can put matrix instructions between them (each phase
+    // starts by waiting for the LDS traffic of the one before): stage = expand and write the 8 x 8 squares, turn = read
+    // them back the other way round, finish = split and store.
+    float turned[8];
+    __device__ __forceinline__ float *scratch_word(unsigned char *operand, int i) const {
+        using L = SplitLayout<ROWS>;
+        const int wave = threadIdx.x >> 6;
+        unsigned char *mine = operand + (wave & 1) * L::kHalf + 64 * (wave >> 1) * 16;
+        return reinterpret_cast<float *>(mine + (i >> 8) * L::kPlane) + (i & 255);
+    }
+    __device__ __forceinline__ void stage_values(unsigned char *operand, const float v[8]) const {
+        const int lane = threadIdx.x & 63, kk = lane & 7, gg = (lane >> 3) & 7;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) *scratch_word(operand, 72 * gg + 8 * e + kk) = v[e];   // [group][tile row][k], groups 72 words apart
+    }
+    __device__ __forceinline__ void stage(unsigned char *operand, const float *s_code) const {
+        if (!active(0)) return;
+        float v[8];
+        expand(0, s_code, v);
+        stage_values(operand, v);
+    }
+    __device__ __forceinline__ void turn(unsigned char *operand) {
+        if (!active(0)) return;
+        const int lane = threadIdx.x & 63, kk = lane & 7, gg = (lane >> 3) & 7;
+        wave_lds_sync();
+        const float4 lo = *reinterpret_cast<const float4 *>(scratch_word(operand, 72 * gg + 8 * kk));
+        const float4 hi = *reinterpret_cast<const float4 *>(scratch_word(operand, 72 * gg + 8 * kk + 4));
+        turned[0] = lo.x; turned[1] = lo.y; turned[2] = lo.z; turned[3] = lo.w;
+        turned[4] = hi.x; turned[5] = hi.y; turned[6] = hi.z; turned[7] = hi.w;                // tile row 8 gg + kk of the wave's 64, its 8 k
+    }
+    __device__ __forceinline__ void finish(unsigned char *operand) const {
+        if (!active(0)) return;
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, kk = lane & 7, gg = (lane >> 3) & 7;
+        wave_lds_sync();
+        commit_split_eight<ROWS>(operand, 64 * (wave >> 1) + 8 * gg + kk, wave & 1, turned);
     }
 };
 
+template <int BM, int BN, int KA, int KB, int PREC>
+constexpr int kWavesPerSimd = (PREC == kPipeSplit && (KA >= kQuant4 || KB >= kQuant4) && BM == 128 && BN == 128) ? 2 : 3;
+
 template <int BM, int BN, int KA, int KB, int EPI, int PREC = kPipeF32>
-__global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   // three waves per SIMD: at most 168 registers
+__global__ __launch_bounds__(256, (kWavesPerSimd<BM, BN, KA, KB, PREC>)) void gemm_kernel(const GemmArgs args) {   // three waves per SIMD: at most 168 registers
     constexpr int WM = BM / 2, WN = BN / 2, MI = WM / 32, NI = WN / 32;
     // Workgroups are dealt round-robin to the 8 accelerator dies, each with its own L2.  Renumber
     // them so that every die works through one contiguous run of (batch entry, tile row, tile
@@ -558,7 +612,7 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     const int slice = id % slices;
     id /= slices;
     constexpr bool kSplit = PREC == kPipeSplit;
-    static_assert(!kSplit || KB < kQuant4, "split pipe: dense operands, or a quantized left factor");
+
     using PlainA = typename std::conditional<KA == kDense, LoadKContig<BM>,
         typename std::conditional<KA == kDenseT, LoadRowContig<BM>,
             LoadQuant<BM, KA == kQuant4 ? 4 : 8, true>>::type>::type;
@@ -569,7 +623,8 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     using LoaderA = typename std::conditional<!kSplit || KA >= kQuant4, PlainA,
         typename std::conditional<KA == kDense, SplitKContig<SPLIT_ROWS_A>, SplitRowContig<SPLIT_ROWS_A>>::type>::type;
     using LoaderB = typename std::conditional<!kSplit, PlainB,
-        typename std::conditional<KB == kDense, SplitRowContig<SPLIT_ROWS_B>, SplitKContig<SPLIT_ROWS_B>>::type>::type;
+        typename std::conditional<KB >= kQuant4, LoadQuant<BN, KB == kQuant4 ? 4 : 8, false, true>,
+            typename std::conditional<KB == kDense, SplitRowContig<SPLIT_ROWS_B>, SplitKContig<SPLIT_ROWS_B>>::type>::type>::type;
     // An operand whose k is contiguous at the source sits in LDS as [row][k] (16-byte commits, one
     // 16-byte fragment read per four MFMA steps); the others as [k][row] (16-byte commits, one word
     // per step).  Which k a lane feeds into which step is free as long as both operands agree:
@@ -645,7 +700,8 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
     if constexpr (kSplit) {                    // the host only picks this pipe where the fast loads apply
         if constexpr (KA >= kQuant4) la.prepare(args.Aq, b, m0);
         else la.prepare(args.lda, m0, args.M);
-        lb.prepare(args.ldb, n0, args.N);
+        if constexpr (KB >= kQuant4) lb.prepare(args.Bq, b, n0);
+        else lb.prepare(args.ldb, n0, args.N);
         if constexpr (KA == kDense) la.vec = a_vec;
         if constexpr (KB == kDenseT) lb.vec = b_vec;
     } else {
@@ -666,7 +722,8 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
         if constexpr (kSplit) {
             if constexpr (KA >= kQuant4) la.fetch(k0);
             else la.fetch_fast(A + (KA == kDense ? (long long)k0 : (long long)k0 * args.lda));
-            lb.fetch_fast(B + (KB == kDenseT ? (long long)k0 : (long long)k0 * args.ldb));
+            if constexpr (KB >= kQuant4) lb.fetch(k0);
+            else lb.fetch_fast(B + (KB == kDenseT ? (long long)k0 : (long long)k0 * args.ldb));
         } else {
             if constexpr (KA < kQuant4) {
                 if (a_fast) la.fetch_fast(A + (KA == kDense ? (long long)k0 : (long long)k0 * args.lda));
@@ -678,12 +735,13 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
             } else lb.fetch(k0);
         }
     };
-    auto commit = [&](int stage) {
+    auto commit = [&](int stage, bool right_in_phases = false) {
         if constexpr (kSplit) {
             unsigned char *at = reinterpret_cast<unsigned char *>(s_mem) + stage * SPLIT_STAGE;
             if constexpr (KA >= kQuant4) la.commit_split(at, s_code);
             else la.commit_split(at);
-            lb.commit_split(at + SPLIT_A);
+            if constexpr (KB >= kQuant4) { if (!right_in_phases) lb.commit_split(at + SPLIT_A, s_code); }
+            else lb.commit_split(at + SPLIT_A);
         } else {
             la.commit(s_a[stage], s_code);
             lb.commit(s_b[stage], s_code);
@@ -732,8 +790,16 @@ __global__ __launch_bounds__(256, 3) void gemm_kernel(const GemmArgs args) {   /
             }
 #pragma unroll
             for (int q = 0; q < 6; ++q) {
+                if constexpr (KB >= kQuant4) {        // the turned commit of the right factor, spread over the products
+                    unsigned char *next_b = reinterpret_cast<unsigned char *>(s_mem) + (cur ^ 1) * SPLIT_STAGE + SPLIT_A;
+                    if (t + 1 < n_tiles) {
+                        if (q == 1) lb.stage(next_b, s_code);
+                        if (q == 2) lb.turn(next_b);
+                        if (q == 4) lb.finish(next_b);
+                    }
+                }
                 if (q == 3 && t + 1 < n_tiles) {
-                    commit(cur ^ 1);
+                    commit(cur ^ 1, true);
                     if (t + 2 < n_tiles) fetch(k_begin + (t + 2) * BK);
                 }
 #pragma unroll
@@ -1411,12 +1477,12 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
     // 128-wide tile on their side unless QT_GEMM_TILE=MxN (a tuning knob) says otherwise.
     struct Shape { int bm, bn; double eff; };
     static const Shape shapes[4] = {{128, 128, 1.0}, {128, 64, 0.92}, {64, 128, 0.92}, {64, 64, 0.82}};
-    // The split pipe: for dense operands in whole k tiles, where the offsets of its loads fit 31 bits -- whatever the
-    // tile shape, so that the bits of a product do not depend on how it is tiled.
+    // The split pipe: for whole k tiles, where the offsets of the dense operands' loads fit 31 bits -- whatever the tile
+    // shape, so that the bits of a product do not depend on how it is tiled.
     bool split_pipe = false;
-    if (gemm_pipe_mode() == kPipeSplit && kb < kQuant4 && d->K % BK == 0 && d->K >= 2 * BK) {
+    if (gemm_pipe_mode() == kPipeSplit && d->K % BK == 0 && d->K >= 2 * BK) {
         const long long reach_a = ka >= kQuant4 ? 0 : ka == kDense ? (long long)d->M * a.lda : (long long)BK * a.lda + d->M;
-        const long long reach_b = kb == kDenseT ? (long long)d->N * a.ldb : (long long)BK * a.ldb + d->N;
+        const long long reach_b = kb >= kQuant4 ? 0 : kb == kDenseT ? (long long)d->N * a.ldb : (long long)BK * a.ldb + d->N;
         split_pipe = reach_a < 0x7fffffffLL && reach_b < 0x7fffffffLL;
     }
     int pick = 0;
@@ -1518,14 +1584,7 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         if (split_pipe) launch_gemm<128, 128, KA, KB, EP, kPipeSplit>(a, d->batch, stream);                  \
         else launch_gemm<128, 128, KA, KB, EP>(a, d->batch, stream);                                         \
         break;
-#define QT_GEMM_CASE(KA, KB, EP)                                                                             \
-    case (KA) * 100 + (KB) * 10 + (EP):                                                                      \
-        if (pick == 0) launch_gemm<128, 128, KA, KB, EP>(a, d->batch, stream);                               \
-        else if (pick == 1) launch_gemm<128, 64, KA, KB, EP>(a, d->batch, stream);                           \
-        else if (pick == 2) launch_gemm<64, 128, KA, KB, EP>(a, d->batch, stream);                           \
-        else launch_gemm<64, 64, KA, KB, EP>(a, d->batch, stream);                                           \
-        break;
-#define QT_GEMM_CASE_LEFT(KA, KB, EP)                                                                        \
+#define QT_GEMM_CASE_QUANT(KA, KB, EP)                                                                        \
     case (KA) * 100 + (KB) * 10 + (EP):                                                                      \
         if (split_pipe) {                                                                                    \
             if (pick == 0) launch_gemm<128, 128, KA, KB, EP, kPipeSplit>(a, d->batch, stream);               \
@@ -1539,10 +1598,10 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         else launch_gemm<64, 64, KA, KB, EP>(a, d->batch, stream);                                           \
         break;
     switch (combo) {
-        QT_GEMM_CASE_LEFT(kQuant4, kDense, kStore)
-        QT_GEMM_CASE_LEFT(kQuant8, kDense, kStore)
-        QT_GEMM_CASE(kDense, kQuant4, kStore)
-        QT_GEMM_CASE(kDense, kQuant8, kStore)
+        QT_GEMM_CASE_QUANT(kQuant4, kDense, kStore)
+        QT_GEMM_CASE_QUANT(kQuant8, kDense, kStore)
+        QT_GEMM_CASE_QUANT(kDense, kQuant4, kStore)
+        QT_GEMM_CASE_QUANT(kDense, kQuant8, kStore)
         QT_GEMM_CASE_DENSE(kDense, kDenseT, kStore)
         QT_GEMM_CASE_DENSE(kDense, kDenseT, kAxpbyDense)
         QT_GEMM_CASE_DENSE(kDense, kDenseT, kAxpbyQuant4)
@@ -1562,7 +1621,9 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
             set_error(kBadArgument, "gemm: combination A kind %d, B kind %d, epilogue %d is not built", ka, kb, ep);
             return;
     }
-#undef QT_GEMM_CASE
+#undef QT_GEMM_CASE_DENSE
+#undef QT_GEMM_CASE_REQUANT
+#undef QT_GEMM_CASE_QUANT
     launch_ok("gemm");
 }
 }  // namespace
