@@ -133,7 +133,7 @@ def precond_step_gpu(torch, variant="shampoo1"):
         more["cholesky_qr_rounds_per_stack_and_update"] = round(bank.qr_rounds / (30 * len(bank.per_order)), 2)
         more["subspace_iteration_updates"] = 30 * sum(bank.per_order.values())
     import qtensor.fused as X
-    more["gemm_pipe"] = ("products of dense fp32 operands on the %s matrix pipe" %
+    more["gemm_pipe"] = ("products on the %s matrix pipe" %
                          ("bf16 (operands split into three bf16 pieces, six products per fp32 product, fp32 accumulation)"
                           if X.gemm_pipe() == "split" else "fp32"))
     return {

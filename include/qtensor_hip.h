@@ -212,7 +212,7 @@ void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
 #define QTENSOR_STATIC_SCRATCH_FLOATS (1 << 24)
 void qtensor_hip_gemm_static(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
 
-/* Which matrix pipe multiplies products of two dense operands, for the whole process (no counterpart in the
+/* Which matrix pipe multiplies, for the whole process (no counterpart in the
  * reference, whose products are torch's fp32 matmul).
  *   0: the fp32 pipe (v_mfma_f32_32x32x2_f32) on the operands as they are;
  *   1: the bf16 pipe on split operands: every fp32 element x is written as h + m + l, three bf16 numbers, each the
@@ -222,8 +222,11 @@ void qtensor_hip_gemm_static(const qtensor_gemm_desc *desc, qtensor_stream_t str
  *      carries the error of fp32 arithmetic (tests/test_gpu_gemm.py measures both pipes against float64), while the
  *      bf16 pipe does sixteen multiply-adds per cycle for every one of the fp32 pipe.  Differences: an infinite
  *      operand element gives NaN where the fp32 pipe gives infinity; elements below 2^-110 lose their low pieces.
- *      Taken for dense operands, K a multiple of 16 and at least 32, under the 128 x 128 tile shape; every other
- *      product runs on the fp32 pipe whatever the mode.
+ *      Taken for K a multiple of 16 and at least 32 (dense operands within 31-bit offsets; quantized operands are
+ *      expanded to fp32 and split the same way), under every tile shape, so that the bits of a product do not
+ *      depend on how it is tiled; every other product runs on the fp32 pipe whatever the mode.  In a symmetric
+ *      product every element below the diagonal takes the value of its partner above (a b and b a add their
+ *      pieces in different orders): the result is exactly symmetric.
  * mode < 0 only queries.  Returns the mode in force before the call.  The initial mode is 1 unless the environment
  * variable QT_GEMM_PIPE is "f32". */
 int qtensor_hip_gemm_pipe(int mode);

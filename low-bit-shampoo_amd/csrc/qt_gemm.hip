@@ -1350,7 +1350,7 @@ float *static_scratch() {
 
 void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream);
 
-// Process-wide choice of the matrix pipe for products of dense operands (qtensor_hip_gemm_pipe); starts from the
+// Process-wide choice of the matrix pipe (qtensor_hip_gemm_pipe); starts from the
 // environment variable QT_GEMM_PIPE ("f32" or "split"), else the split pipe.
 std::atomic<int> &pipe_mode_slot() {
     static std::atomic<int> mode{[] {

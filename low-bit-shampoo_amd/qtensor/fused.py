@@ -140,7 +140,7 @@ def _launch(desc: GemmDesc, device: torch.device) -> None:
 
 
 def gemm_pipe(mode: Optional[str] = None) -> str:
-    """Which matrix pipe multiplies products of dense operands, for the whole process: "f32" (fp32 MFMA) or "split"
+    """Which matrix pipe multiplies (dense and quantized operands alike), for the whole process: "f32" (fp32 MFMA) or "split"
     (operands split into three bf16 pieces, six bf16 products per fp32 product, fp32 accumulation: fp32-grade
     results at a multiple of the fp32 pipe's rate).  Sets the mode when given; returns the one in force before."""
     if F.lib is None:
