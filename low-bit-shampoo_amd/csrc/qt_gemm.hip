@@ -1520,15 +1520,26 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         const long long tm = (d->M + sh.bm - 1) / sh.bm, tn = (d->N + sh.bn - 1) / sh.bn;
         const double tiles = (double)tm * tn * d->batch;
         const int k_tiles = d->K / 16;
-        const double fixed = 64.0;
-        const double whole = ceil(tiles / units) * (d->K + fixed);
+        // Cost of a way to cut, in k steps of one workgroup that has its unit to itself: the workgroups of a launch run
+        // three to a unit side by side, each at its own pace while the unit's matrix pipe has room (a lone workgroup
+        // uses about half of it) -- so the time is the longer of (rounds of resident workgroups) x (k range + a fixed
+        // cost per workgroup: prologue, epilogue) and (a unit's share of all k steps) x 0.5; a cut adds the launch that
+        // sums the slices, worth about 200 k steps.
+        const double fixed = 64.0, resident = 3.0, pipe_share = 0.5, sum_launch = 200.0;
+        auto cost_of = [&](int sp) {
+            const double groups = tiles * sp, range = (double)d->K / sp + fixed;
+            const double rounds = ceil(groups / (units * resident)) * range;
+            const double share = groups / units * range * pipe_share;
+            return (rounds > share ? rounds : share) + (sp > 1 ? sum_launch : 0.0);
+        };
+        const double whole = cost_of(1);
         double best = whole;
         int best_split = 1;
         static const char *forced_split = getenv("QT_GEMM_SPLIT");
         for (int sp = 2; sp <= 8; ++sp) {
             if (k_tiles % sp != 0 || k_tiles / sp < 8) continue;
             if ((long long)sp * d->batch * d->M * d->N > a.workspace_floats) continue;
-            const double cost = ceil(tiles * sp / units) * ((double)d->K / sp + fixed);
+            const double cost = cost_of(sp);
             if (forced_split != nullptr) { if (sp == atoi(forced_split)) best_split = sp; }
             else if (cost < best) { best = cost; best_split = sp; }
         }
