@@ -161,6 +161,19 @@ class ShampooBank:
             done.record(side)
             main.wait_event(done)
 
+    def _run_on(self, slot, job):
+        """Run one callable on side stream `slot` (the stream _fan_out gives job number `slot`), after what the
+        current stream holds; the current stream then waits for it."""
+        if not self.streams:
+            job()
+            return
+        main = torch.cuda.current_stream(self.device)
+        side = self.streams[slot % len(self.streams)]
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            job()
+        main.wait_stream(side)
+
     # ---- eligibility -----------------------------------------------------------------------------
     @staticmethod
     def matrix_shape(p):

@@ -111,16 +111,6 @@ class ShampooBank2(ShampooBank):
                 solver[order] = X.CholeskyQR(X.gemm(stat[order], basis[order], trans_b=True))     # L Vt^T
             return run
 
-        def check(order):
-            return lambda: None if solver[order].finished else solver[order].check()
-
-        def poll(order):
-            return lambda: None if solver[order].finished else solver[order].poll()
-
-        def advance(order):
-            return lambda: None if solver[order].finished else solver[order].advance()
-
-
         def iterate(order):
             def run():
                 L = stat[order]
@@ -148,11 +138,26 @@ class ShampooBank2(ShampooBank):
         # The stacks whose factorisation is complete go on (Rayleigh quotients, requantize) on a thread and a
         # stream of their own while the others still iterate: the later rounds of a few ill-conditioned
         # matrices are chains of small launches that leave most of the device, and this thread, waiting.
+        # The test after the sweep needs the host (it reads the sweep's flags, then the deviations of the flagged
+        # matrices), so the stacks are looked at in the order in which their sweeps end, cheapest first, and each
+        # goes through test, reading and polishing round in one go: the polishing of a few matrices of a cheap stack
+        # then runs while the sweep of the most expensive one is still under way.
+        slot = {o: i for i, o in enumerate(orders)}
+        by_finish = sorted(orders, key=lambda o: o ** 3 * self.per_order[o])
+
+        def look_at(order):
+            def run():
+                s = solver[order]
+                s.check()
+                if not s.finished and not s.poll():
+                    s.advance()
+            return run
+
         early, waiting = None, list(orders)
         while not all(solver[o].finished for o in orders):
-            self._fan_out([check(o) for o in orders])
-            self._fan_out([poll(o) for o in orders])
-            self._fan_out([advance(o) for o in orders])
+            for o in by_finish:
+                if not solver[o].finished:
+                    self._run_on(slot[o], look_at(o))
             ready = [o for o in waiting if solver[o].finished]
             if self.streams and early is None and ready and len(ready) < len(waiting):
                 waiting = [o for o in waiting if o not in ready]
