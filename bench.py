@@ -32,7 +32,7 @@ BITS = 4
 BYTES_PER_ELEMENT = 4 + BITS / 8 + 4 / BLOCK      # fp32 in/out + packed code + share of the fp32 maximum
 # HBM bytes per launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE on this workload, scaled by
 # the library's plain copy kernel (summary: profiles/quantize_dequantize_16384sq_4bit_bs64_hbm_traffic.txt)
-MEASURED_TRAFFIC = {"quantize": 1225662500, "dequantize": 1225738000}
+MEASURED_TRAFFIC = {"quantize": 1225675980, "dequantize": 1225393971}
 TRAFFIC_SOURCE = ("profiles/quantize_dequantize_16384sq_4bit_bs64_hbm_traffic.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of "
                   "this workload, scaled by the same counters over the library's plain copy kernel; a kept profile, "
                   "not re-measured by this run")
