@@ -510,7 +510,7 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_step:
         result["fused_gemm"] = fused_gemm_gpu(torch, code)
-        # the step BASELINE's configuration names: eigenbasis variant with coupled-Newton inverse roots
+        # the step the headline configuration names: eigenbasis variant with coupled-Newton inverse roots
         result["precond_step"] = precond_step_gpu(torch, "shampoo2")
         result["precond_step"]["roofline"] = dominant_product_gpu(torch)
         result["precond_step_naive"] = precond_step_gpu(torch, "shampoo1")
