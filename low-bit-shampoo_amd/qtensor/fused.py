@@ -541,7 +541,9 @@ class CholeskyQR:
         if self.swept:
             self.swept = False
             clean = self.info.cpu().numpy() == 0                                # (a host synchronisation)
-            self._finish(np.nonzero(clean)[0], self.Q)
+            # the clean matrices are final where they are; only the flagged ones are copied out into a working
+            # set of their own and written back when they are done
+            self.final = self.Q
             self._keep(~clean)
             self.finished = self.ids.size == 0
             if self.finished:
