@@ -56,7 +56,21 @@ def cpu_baseline(torch, x_slice, code):
     QL.dequantize_loop(out, code, order, absmax, BLOCK, BITS)
     dt = time.perf_counter() - t0
     nbytes = 2 * BYTES_PER_ELEMENT * order * order
+    # informational: the same sample through the scalar C restatement (one core, no Python in the loop)
+    strong = None
+    try:
+        from oracle import quant_np as QN
+        xs, cs = x_slice.numpy(), code.numpy()
+        t1 = time.perf_counter()
+        c_out, c_absmax = QN.quantize_c(xs, cs, order, BLOCK, BITS)
+        QN.dequantize_c(c_out, cs, order, c_absmax, BLOCK, BITS)
+        dc = time.perf_counter() - t1
+        strong = {"value": nbytes / dc / 1e9, "unit": "GB/s", "cores": 1, "seconds": dc,
+                  "what": "the same sample through the scalar C restatement (oracle/qoracle.c), one core"}
+    except (OSError, ImportError, RuntimeError) as exc:      # the compiled checker is not there: say so, go on
+        strong = {"value": None, "what": "scalar C restatement not available: %s" % exc}
     return {
+        "strong_cpu_baseline": strong,
         "value": nbytes / dt / 1e9,
         "unit": "GB/s",
         "cores": 1,
