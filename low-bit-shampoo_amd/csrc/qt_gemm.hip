@@ -1,5 +1,7 @@
-// fp32 matrix products on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32), with blockwise
-// quantized operands expanded on their way into LDS and the Shampoo epilogues fused in.
+// Products of fp32 matrices on the gfx950 matrix cores, with blockwise quantized operands expanded on their
+// way into LDS and the Shampoo epilogues fused in.  Two pipes: the fp32 one (v_mfma_f32_32x32x2_f32) and, by
+// default, the bf16 one on operands split into three bf16 pieces each (v_mfma_f32_32x32x16_bf16, six products
+// per fp32 product, fp32 accumulation: fp32-grade results at a multiple of the rate; see kPipeSplit below).
 //
 // What the reference does with separate steps
 //   P = dequantize(Pq);  out = P @ G            (optimizers/shampoo2.py:255-268, shampoo1.py:224-237)
@@ -18,7 +20,7 @@
 // contiguous -- [row][k] (stride 20) when k is, [k][row] (stride rows + 4) otherwise -- so every
 // commit is a 16-byte store; fragments come out as one 16-byte read per four MFMA steps or as
 // consecutive words per step.  Global loads run two tiles ahead of the MFMAs; the LDS commit sits
-// in the middle of the MFMA stream.
+// in the middle of the MFMA stream.  (Split pipe: three bf16 planes per operand tile, [half of k][row][8].)
 #include "qt_common.h"
 #include "qt_tables.h"
 
@@ -386,7 +388,6 @@ struct SplitRowContig {
     static constexpr int PER = ROWS * BK / 256;
     float v[PER];
     int off, ld_;
-    bool vec = true;                         // (unused: word loads need no alignment)
     __device__ __forceinline__ void prepare(int ld, int row0, int rows) {
         ld_ = ld;
         const int row = threadIdx.x & (ROWS - 1), part = ROWS == 128 ? threadIdx.x >> 7 : threadIdx.x >> 6;
@@ -619,12 +620,11 @@ __global__ __launch_bounds__(256, (kWavesPerSimd<BM, BN, KA, KB, PREC>)) void ge
     using PlainB = typename std::conditional<KB == kDense, LoadRowContig<BN>,
         typename std::conditional<KB == kDenseT, LoadKContig<BN>,
             LoadQuant<BN, KB == kQuant4 ? 4 : 8, false>>::type>::type;
-    constexpr int SPLIT_ROWS_A = BM, SPLIT_ROWS_B = BN;
     using LoaderA = typename std::conditional<!kSplit || KA >= kQuant4, PlainA,
-        typename std::conditional<KA == kDense, SplitKContig<SPLIT_ROWS_A>, SplitRowContig<SPLIT_ROWS_A>>::type>::type;
+        typename std::conditional<KA == kDense, SplitKContig<BM>, SplitRowContig<BM>>::type>::type;
     using LoaderB = typename std::conditional<!kSplit, PlainB,
         typename std::conditional<KB >= kQuant4, LoadQuant<BN, KB == kQuant4 ? 4 : 8, false, true>,
-            typename std::conditional<KB == kDense, SplitRowContig<SPLIT_ROWS_B>, SplitKContig<SPLIT_ROWS_B>>::type>::type>::type;
+            typename std::conditional<KB == kDense, SplitRowContig<BN>, SplitKContig<BN>>::type>::type>::type;
     // An operand whose k is contiguous at the source sits in LDS as [row][k] (16-byte commits, one
     // 16-byte fragment read per four MFMA steps); the others as [k][row] (16-byte commits, one word
     // per step).  Which k a lane feeds into which step is free as long as both operands agree:
