@@ -170,6 +170,11 @@ def precond_step_gpu(torch, variant="shampoo1"):
 FP32_MATRIX_PEAK_TFLOPS = 157.3
 BF16_MATRIX_PEAK_TFLOPS = 2500.0
 SPLIT_PRODUCTS = 6            # bf16 products that make one fp32 product on the split pipe
+# HBM bytes per launch of the 99 x 1024^3 product (operands 830 MB + result 415 MB algorithmically), kept profile
+PRODUCT_TRAFFIC = 1901545267
+PRODUCT_TRAFFIC_SOURCE = ("profiles/dense_stack_product_99x1024_kernel_stats_and_mfma_counters.txt: rocprofv3 --pmc FETCH_SIZE / "
+                          "WRITE_SIZE of this launch, scaled by the same counters over the library's plain copy kernel; a kept "
+                          "profile, not re-measured by this run")
 
 
 def fused_gemm_gpu(torch, code):
@@ -366,7 +371,8 @@ def dominant_product_gpu(torch):
         X.gemm_pipe(before)
     peak = BF16_MATRIX_PEAK_TFLOPS / SPLIT_PRODUCTS
     return {"bound": "mfma", "kernel": "gemm_kernel<128,128,dense,dense,store,split> on 99 x (1024 x 1024 x 1024)",
-            "achieved": round(tf, 1), "peak": round(peak, 1), "unit": "TFLOP/s", "frac": round(tf / peak, 4), "traffic": None,
+            "achieved": round(tf, 1), "peak": round(peak, 1), "unit": "TFLOP/s", "frac": round(tf / peak, 4),
+            "traffic": PRODUCT_TRAFFIC, "traffic_source": PRODUCT_TRAFFIC_SOURCE,
             "avg_launch_ms": round(ms, 4), "algorithmic_flop_per_launch": flop,
             "pipe": "v_mfma_f32_32x32x16_bf16 on operands split into three bf16 pieces: %d bf16 products per fp32 product, "
                     "so peak = bf16 dense peak %.0f / %d; achieved counts the algorithmic fp32 flops (2 m n k)"
