@@ -210,11 +210,21 @@ __global__ __launch_bounds__(256) void panel_norms_kernel(const float *panel, lo
     const int chunk = blockIdx.x, b = blockIdx.y, c = threadIdx.x & 63, g = threadIdx.x >> 6;
     const float *P = panel + (long long)b * stride;
     const int rows = (n + kNormChunks - 1) / kNormChunks, r0 = chunk * rows, r1 = min(r0 + rows, n);
-    float sum = 0.0f;
-    for (int r = r0 + g; r < r1; r += 4) {
-        const float v = P[(long long)r * ld + c];
-        sum = __builtin_fmaf(v, v, sum);
+    // eight rows in flight per thread: the loop is bound by the latency of its loads, not by their number
+    float part8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    int r = r0 + g;
+    for (; r + 28 < r1; r += 32) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = P[(long long)(r + 4 * i) * ld + c];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) part8[i] = __builtin_fmaf(v[i], v[i], part8[i]);
     }
+    for (; r < r1; r += 4) {
+        const float v = P[(long long)r * ld + c];
+        part8[0] = __builtin_fmaf(v, v, part8[0]);
+    }
+    const float sum = ((part8[0] + part8[1]) + (part8[2] + part8[3])) + ((part8[4] + part8[5]) + (part8[6] + part8[7]));
     __shared__ float part[4][64];
     part[g][c] = sum;
     __syncthreads();
@@ -236,7 +246,15 @@ __global__ __launch_bounds__(256) void panel_rescale_kernel(float *panel, long l
     } else if (norm2 > 0.0f) {
         float scale = __builtin_amdgcn_rsqf(norm2);
         scale = scale * __builtin_fmaf(-0.5f * norm2 * scale, scale, 1.5f);
-        for (int r = r0 + g; r < r1; r += 4) P[(long long)r * ld + c] *= scale;
+        int r = r0 + g;
+        for (; r + 28 < r1; r += 32) {               // eight rows in flight per thread
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = P[(long long)(r + 4 * i) * ld + c];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) P[(long long)(r + 4 * i) * ld + c] = v[i] * scale;
+        }
+        for (; r < r1; r += 4) P[(long long)r * ld + c] *= scale;
     }
 }
 
