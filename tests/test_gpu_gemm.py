@@ -74,16 +74,23 @@ def test_dense_products_all_layouts(mods, m, n, k, batch):
 def test_quantized_factor_times_dense(mods, code_maps, bits, bs, name, diag):
     F, X = mods
     g = torch.Generator().manual_seed(bits + bs)
-    for n, other, batch in ((256, 100, 2), (768, 320, 1), (1024, 64, 1)):
-        if n % bs:
-            continue
-        mats = torch.randn(batch, n, n, generator=g)
-        mats[:, 3, :64] = 0.0                                  # a zero-maximum segment
-        q, deq = make_quantized(F, X, mats, code_maps[(name, bits)], bits, bs, diag)
-        G_left = torch.randn(batch, n, other, generator=g)
-        G_right = torch.randn(batch, other, n, generator=g)
-        assert rel_err(X.gemm(q, G_left.cuda()), deq @ G_left.double()) <= TOL
-        assert rel_err(X.gemm(G_right.cuda(), q), G_right.double() @ deq) <= TOL
+    # (few and many matrices, narrow and wide partners: between them the cases take every tile shape)
+    before = X.gemm_pipe()
+    try:
+        for n, other, batch in ((256, 100, 2), (768, 320, 1), (1024, 64, 1), (256, 200, 40), (512, 128, 24), (128, 64, 60), (64, 256, 30)):
+            if n % bs:
+                continue
+            mats = torch.randn(batch, n, n, generator=g)
+            mats[:, 3, :64] = 0.0                                  # a zero-maximum segment
+            q, deq = make_quantized(F, X, mats, code_maps[(name, bits)], bits, bs, diag)
+            G_left = torch.randn(batch, n, other, generator=g)
+            G_right = torch.randn(batch, other, n, generator=g)
+            for pipe in ("split", "f32"):
+                X.gemm_pipe(pipe)
+                assert rel_err(X.gemm(q, G_left.cuda()), deq @ G_left.double()) <= TOL, (pipe, n, other, batch)
+                assert rel_err(X.gemm(G_right.cuda(), q), G_right.double() @ deq) <= TOL, (pipe, n, other, batch)
+    finally:
+        X.gemm_pipe(before)
 
 
 def test_config3_preconditioned_gradient(mods, code_maps):
