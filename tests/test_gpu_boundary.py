@@ -62,3 +62,39 @@ def test_sixteen_reference_symbols_bound_like_the_reference_binds_them(code_maps
         want_back = Q.dequantize_c(want[0], code_np, order, want[1], blocksize, bits, diag=want[2] if diagreal else None,
                                    to_bf16=dtype == "bf16")
         assert np.array_equal(bits_of(back.float().cpu().numpy()), bits_of(want_back)), (mid, "dequantized")
+
+
+def test_pipe_switch_and_matrix_pipe_yardstick_through_the_bare_library():
+    """The two entry points around the matrix pipes, called as a C program would: the process-wide switch
+    (query, set, refuse) and the launch that is nothing but matrix instructions, whose rate must lie between a
+    tenth of the published peak and the peak itself on either pipe."""
+    lib = ct.cdll.LoadLibrary(str(LIB))
+    lib.qtensor_hip_gemm_pipe.restype = ct.c_int
+    lib.qtensor_hip_mfma_rate_flop.restype = ct.c_double
+    lib.qtensor_hip_mfma_rate_flop.argtypes = [ct.c_int, ct.c_int, ct.c_int, ct.c_void_p, ct.c_void_p]
+    lib.qtensor_hip_last_error.restype = ct.c_int
+    before = lib.qtensor_hip_gemm_pipe(ct.c_int(-1))
+    try:
+        assert before in (0, 1)
+        assert lib.qtensor_hip_gemm_pipe(ct.c_int(0)) == before and lib.qtensor_hip_gemm_pipe(ct.c_int(-1)) == 0
+        assert lib.qtensor_hip_gemm_pipe(ct.c_int(1)) == 0 and lib.qtensor_hip_gemm_pipe(ct.c_int(-1)) == 1
+        assert lib.qtensor_hip_gemm_pipe(ct.c_int(7)) == 1 and lib.qtensor_hip_last_error() != 0      # refused, unchanged
+        assert lib.qtensor_hip_gemm_pipe(ct.c_int(-1)) == 1 and lib.qtensor_hip_last_error() == 0
+    finally:
+        lib.qtensor_hip_gemm_pipe(ct.c_int(before))
+    sink = torch.zeros(1, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.qtensor_hip_mfma_rate_flop(2, 10, 1, sink.data_ptr(), stream) == 0.0 and lib.qtensor_hip_last_error() != 0
+    assert lib.qtensor_hip_mfma_rate_flop(1, 0, 1, sink.data_ptr(), stream) == 0.0 and lib.qtensor_hip_last_error() != 0
+    assert lib.qtensor_hip_mfma_rate_flop(1, 10, 1, None, stream) == 0.0 and lib.qtensor_hip_last_error() != 0
+    for pipe, rounds, peak in ((1, 4000, 2500e12), (0, 1000, 157.3e12)):
+        lib.qtensor_hip_mfma_rate_flop(pipe, rounds, 2, sink.data_ptr(), stream)              # warm-up
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        flop = lib.qtensor_hip_mfma_rate_flop(pipe, rounds, 2, sink.data_ptr(), stream)
+        e1.record()
+        torch.cuda.synchronize()
+        assert lib.qtensor_hip_last_error() == 0 and flop > 0
+        rate = flop / (e0.elapsed_time(e1) * 1e-3)
+        assert 0.1 * peak <= rate <= 1.02 * peak, (pipe, rate)
+    assert float(sink[0]) == 0.0                                                              # the sink is never written
