@@ -798,7 +798,19 @@ __global__ __launch_bounds__(256, (kWavesPerSimd<BM, BN, KA, KB, PREC>)) void ge
                         if (q == 4) lb.finish(next_b);
                     }
                 }
-                if (q == 3 && t + 1 < n_tiles) {
+                if constexpr (KA < kQuant4 && KB < kQuant4) {
+                    // dense operands: the split of the next tile in two halves between the product groups (A, then B),
+                    // each followed by its loads of the tile after
+                    unsigned char *next = reinterpret_cast<unsigned char *>(s_mem) + (cur ^ 1) * SPLIT_STAGE;
+                    if (q == 2 && t + 1 < n_tiles) {
+                        la.commit_split(next);
+                        if (t + 2 < n_tiles) la.fetch_fast(A + (KA == kDense ? (long long)(k_begin + (t + 2) * BK) : (long long)(k_begin + (t + 2) * BK) * args.lda));
+                    }
+                    if (q == 4 && t + 1 < n_tiles) {
+                        lb.commit_split(next + SPLIT_A);
+                        if (t + 2 < n_tiles) lb.fetch_fast(B + (KB == kDenseT ? (long long)(k_begin + (t + 2) * BK) : (long long)(k_begin + (t + 2) * BK) * args.ldb));
+                    }
+                } else if (q == 3 && t + 1 < n_tiles) {
                     commit(cur ^ 1, true);
                     if (t + 2 < n_tiles) fetch(k_begin + (t + 2) * BK);
                 }
