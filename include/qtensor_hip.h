@@ -284,6 +284,10 @@ void qtensor_hip_block_gram_schmidt_batched(float *q, float *w, float *gram, flo
  * gram [batch, n, n], one pass, fixed summation order, NaN if G_b holds one.  partial: scratch of
  * batch * 64 floats.  (No counterpart in the reference: Householder QR needs no such test.) */
 void qtensor_hip_gram_deviation_batched(const float *gram, float *partial, float *out, int n, int batch, qtensor_stream_t stream);
+/* out[b * n + j] = sum_i a[b][i][j] * b[b][i][j] for two stacks [batch, n, n] (n a multiple of 64): the diagonal of
+ * a^T b in one pass over both stacks and a fixed summation order -- the Rayleigh quotients diag(Q^T (L Q)) after a
+ * subspace iteration step, which the reference takes from the full product V^T L V (qtensor/utils.py:158). */
+void qtensor_hip_column_dots_batched(const float *a, const float *b, float *out, int n, int batch, qtensor_stream_t stream);
 /* dst[b] = src[b] (n x n fp32 each) for every b with flags[b] != 0; the other matrices of dst are left
  * alone.  Puts the previous iterate back where a factorisation failed, without a pass over the whole
  * stack and without the host knowing which ones failed.  (No counterpart in the reference.) */

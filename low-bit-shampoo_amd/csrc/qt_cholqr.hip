@@ -198,6 +198,31 @@ __global__ __launch_bounds__(256) void copy_flagged_kernel(float *dst, const flo
     for (long long q = blockIdx.x * 256ll + threadIdx.x; q < quads; q += (long long)gridDim.x * 256) d[q] = s[q];
 }
 
+// out[b][j] = sum_i A[b][i][j] B[b][i][j] for two stacks of n x n matrices: the diagonal of A^T B without the
+// product (the Rayleigh quotients diag(Q^T (L Q)) of a subspace iteration step).  A workgroup takes 64 columns of
+// one matrix; its four waves take every fourth row, eight rows in flight per thread, and add up in a fixed order.
+__global__ __launch_bounds__(256) void column_dots_kernel(const float *A, const float *B, float *out, int n) {
+    const int c = blockIdx.x * 64 + (threadIdx.x & 63), g = threadIdx.x >> 6, b = blockIdx.y;
+    const float *pa = A + (long long)b * n * n + c, *pb = B + (long long)b * n * n + c;
+    float part8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    int r = g;
+    for (; r + 28 < n; r += 32) {
+        float x[8], y[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { x[i] = pa[(long long)(r + 4 * i) * n]; y[i] = pb[(long long)(r + 4 * i) * n]; }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) part8[i] = __builtin_fmaf(x[i], y[i], part8[i]);
+    }
+    for (; r < n; r += 4) part8[0] = __builtin_fmaf(pa[(long long)r * n], pb[(long long)r * n], part8[0]);
+    __shared__ float part[4][64];
+    part[g][threadIdx.x & 63] = ((part8[0] + part8[1]) + (part8[2] + part8[3])) + ((part8[4] + part8[5]) + (part8[6] + part8[7]));
+    __syncthreads();
+    if (g == 0) {
+        const int l = threadIdx.x;
+        out[(long long)b * n + c] = (part[0][l] + part[1][l]) + (part[2][l] + part[3][l]);
+    }
+}
+
 // One 64-column panel of every matrix of a stack: each column is scaled to unit length; with `fill` given, a
 // column whose squared length is below null_norm2 (what projecting out the earlier columns has left of a
 // unit column: rounding noise) is replaced by the same column of `fill` (unit columns in general position)
@@ -561,6 +586,14 @@ extern "C" void qtensor_hip_gram_deviation_batched(const float *gram, float *par
     if (!launch_ok("gram_deviation_batched (bands)")) return;
     hipLaunchKernelGGL(deviation_total_kernel, dim3((batch + 63) / 64), dim3(64), 0, stream, partial, bands, batch, out);
     launch_ok("gram_deviation_batched (totals)");
+}
+
+extern "C" void qtensor_hip_column_dots_batched(const float *a, const float *b, float *out, int n, int batch, void *stream_v) {
+    using namespace qt;
+    clear_error();
+    if (!stack_args_ok("column_dots_batched", n, batch, {a, b, out})) return;
+    hipLaunchKernelGGL(column_dots_kernel, dim3(n / 64, batch), dim3(256), 0, (hipStream_t)stream_v, a, b, out, n);
+    launch_ok("column_dots_batched");
 }
 
 extern "C" void qtensor_hip_copy_flagged_batched(float *dst, const float *src, const int *flags, int n, int batch, void *stream_v) {

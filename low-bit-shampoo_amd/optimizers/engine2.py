@@ -115,7 +115,8 @@ class ShampooBank2(ShampooBank):
             def run():
                 L = stat[order]
                 Q, redone[order] = solver[order].result()
-                quotients = (Q * X.gemm(L, Q)).sum(dim=1)                      # diag(Q^T L Q)
+                LQ = X.gemm(L, Q)
+                quotients = X.column_dots(Q, LQ) if Q.shape[1] % 64 == 0 else (Q * LQ).sum(dim=1)      # diag(Q^T L Q)
                 ascending, where = torch.sort(quotients, dim=1)
                 half = self.keep[order].shape[1]
                 self.keep[order] = where[:, :half].contiguous()

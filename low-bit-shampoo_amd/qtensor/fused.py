@@ -348,6 +348,8 @@ if F.lib is not None:
     F.lib.qtensor_hip_block_gram_schmidt_batched.argtypes = [ct.c_void_p] * 7 + [ct.c_int, ct.c_int, ct.c_float, ct.c_float, ct.c_void_p]
     F.lib.qtensor_hip_gram_deviation_batched.restype = None
     F.lib.qtensor_hip_gram_deviation_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
+    F.lib.qtensor_hip_column_dots_batched.restype = None
+    F.lib.qtensor_hip_column_dots_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
     F.lib.qtensor_hip_copy_flagged_batched.restype = None
     F.lib.qtensor_hip_copy_flagged_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
     F.lib.qtensor_hip_solve_upper_right_batched.restype = None
@@ -417,6 +419,16 @@ def gram_deviation(gram: Tensor) -> Tensor:
     out = torch.empty(B, 2, device=gram.device)
     partial = torch.empty(B, 64, device=gram.device)
     F._call(F.lib.qtensor_hip_gram_deviation_batched, gram.device, gram.data_ptr(), partial.data_ptr(), out.data_ptr(), n, B)
+    return out
+
+
+def column_dots(a: Tensor, b: Tensor) -> Tensor:
+    """[B, n]: sum_i a[:, i, j] * b[:, i, j] for two stacks [B, n, n] (n a multiple of 64) -- the diagonal of a^T b
+    in one pass, fixed summation order."""
+    B, n, _ = a.shape
+    _stack(a, "a", (B, n, n)), _stack(b, "b", (B, n, n))
+    out = torch.empty(B, n, device=a.device)
+    F._call(F.lib.qtensor_hip_column_dots_batched, a.device, a.data_ptr(), b.data_ptr(), out.data_ptr(), n, B)
     return out
 
 

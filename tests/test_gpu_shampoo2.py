@@ -469,3 +469,18 @@ def test_optimizers_reduce_a_small_regression_loss(variant, fused, tmp_path, mon
     # (shampoo2 with inv_root_mode=0 preconditions with the kept half of the eigenpairs only: slower progress)
     bound = 0.3 if variant == "shampoo1" else 0.6
     assert all(l == l for l in losses) and losses[-1] < bound * losses[0], (losses[0], losses[-1])
+
+
+@pytest.mark.parametrize("n,batch", [(64, 3), (320, 4), (1024, 2)])
+def test_column_dots_is_the_diagonal_of_the_product(mods, n, batch):
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(n)
+    A, B = torch.randn(batch, n, n, generator=g), torch.randn(batch, n, n, generator=g)
+    got = X.column_dots(A.cuda(), B.cuda())
+    want = (A.double() * B.double()).sum(dim=1)
+    scale = (A.double().abs() * B.double().abs()).sum(dim=1)
+    assert got.shape == (batch, n)
+    assert float(((got.cpu().double() - want).abs() / scale).max()) <= 1e-6
+    assert torch.equal(got, X.column_dots(A.cuda(), B.cuda()))                 # fixed summation order
+    with pytest.raises(ValueError):
+        X.column_dots(A.cuda(), B[:, :, :32].contiguous().cuda())
