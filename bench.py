@@ -420,7 +420,8 @@ def main():
         X.gemm_pipe(args.gemm_pipe)
     if args.bank_streams is not None:
         from optimizers.engine import ShampooBank
-        ShampooBank.DEFAULT_STREAMS = args.bank_streams
+        from optimizers.engine2 import ShampooBank2
+        ShampooBank.DEFAULT_STREAMS = ShampooBank2.DEFAULT_STREAMS = args.bank_streams
         if args.bank_streams == 0:           # profiling: nothing may overlap, the side thread of shampoo2 neither
             from optimizers import shampoo2
             shampoo2.ShampooAdamW.overlap_unbatched_statistics = False

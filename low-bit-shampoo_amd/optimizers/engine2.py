@@ -32,6 +32,10 @@ cholesky_qr = X.cholesky_qr
 
 
 class ShampooBank2(ShampooBank):
+    # One stream more than there are big stacks: measured on the ViT-B/32 shapes (three orders) 24.1 ms per regular step
+    # with four side streams against 25.7 with three, 24.9-25.2 with five or six (four hardware queues per process).
+    DEFAULT_STREAMS = 4
+
     def __init__(self, params, name2qmap, code, *, rect_t1=1, rect_t2=4, inv_root_mode=0, **kwargs):
         self.rect_t1, self.rect_t2, self.inv_root_mode = rect_t1, rect_t2, inv_root_mode
         self.qr_fallbacks = 0                     # matrices that went through torch.linalg.qr so far
