@@ -49,6 +49,10 @@ class ShampooBank2(ShampooBank):
         return self._early
 
     def _beside_stream(self):
+        # the side stream that no order's chain runs on, if there is one: a stream more would share a hardware queue
+        # with one of the chains (23.3 against 24.1 ms per regular step)
+        if len(self.streams) > len(self.per_order):
+            return self.streams[-1]
         if getattr(self, "_beside", None) is None:
             self._beside = torch.cuda.Stream(device=self.device)
         return self._beside
