@@ -393,13 +393,19 @@ struct Sweep {
     bool project(int a0, int c0, int width) {
         const int k = c0 - a0;
         if (k <= 0) return true;
-        const long long w_stride = (long long)n * w_cols;
+        // The coefficients of matrix b sit k * width floats apart; what is left of w behind them takes the partial
+        // products when the product is cut along k (one 64 x 64 tile per matrix and a k range of n: few, long workgroups).
+        const long long w_stride = (long long)k * width, w_used = w_stride * batch, w_all = (long long)batch * n * w_cols;
         qtensor_gemm_desc p = {};                             // W = Q_a^T Y
         p.M = k; p.N = width; p.K = n; p.batch = batch;
         p.kind_a = QTENSOR_DENSE_T; p.kind_b = QTENSOR_DENSE; p.epilogue = QTENSOR_EPI_STORE;
         p.args.A = strided(q + a0, mat()); p.args.lda = n;
         p.args.B = strided(q + c0, mat()); p.args.ldb = n;
         p.args.C = strided(w, w_stride); p.args.ldc = width;
+        if (k <= NB && width <= NB && w_all > w_used) {
+            p.args.workspace = w + w_used;
+            p.args.workspace_floats = w_all - w_used;
+        }
         if (!run(p, stream)) return false;
         qtensor_gemm_desc r = {};                             // Y -= Q_a W
         r.M = n; r.N = width; r.K = k; r.batch = batch;
