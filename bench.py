@@ -128,6 +128,9 @@ def precond_step_gpu(torch, variant="shampoo1"):
 
     for _ in range(10):
         timed_step()
+    torch.cuda.synchronize()
+    resident = torch.cuda.memory_allocated()             # parameters, four gradient sets, optimizer state, kept scratch
+    torch.cuda.reset_peak_memory_stats()
     regular, newton = [], []
     for i in range(11, 31):
         wall, dev = timed_step()
@@ -162,6 +165,9 @@ def precond_step_gpu(torch, variant="shampoo1"):
         "ms_per_step_amortized_over_10": round((9 * reg + new) / 10, 3),
         "device_ms_regular": round(mean(regular, 1), 3),
         "device_ms_with_inverse_roots": round(mean(newton, 1), 3),
+        "device_memory_gib": {"allocated_between_steps": round(resident / 2 ** 30, 2),
+                              "peak_inside_a_step": round(torch.cuda.max_memory_allocated() / 2 ** 30, 2),
+                              "of_which_parameters_and_the_four_gradient_sets": round(5 * sum(p.numel() for p in params) * 4 / 2 ** 30, 2)},
         "product_gflop_per_regular_step": round(2 * gram_flop / 1e9, 1),
         "product_tflops_regular": round(2 * gram_flop / (mean(regular, 1) * 1e-3) / 1e12, 1),
     }

@@ -394,8 +394,9 @@ struct Sweep {
         const int k = c0 - a0;
         if (k <= 0) return true;
         // The coefficients of matrix b sit k * width floats apart; what is left of w behind them takes the partial
-        // products when the product is cut along k (against few earlier columns: a tile or a few per matrix and a k range
-        // of n, few and long workgroups).
+        // products when the product is cut along k (one 64 x 64 tile per matrix and a k range of n: few, long workgroups).
+        // Only for a panel against its neighbour: cutting the products against all earlier panels as well is a little
+        // faster for one stack alone and costs the optimizer step, where three stacks share the device, a third.
         const long long w_stride = (long long)k * width, w_used = w_stride * batch, w_all = (long long)batch * n * w_cols;
         qtensor_gemm_desc p = {};                             // W = Q_a^T Y
         p.M = k; p.N = width; p.K = n; p.batch = batch;
@@ -403,7 +404,7 @@ struct Sweep {
         p.args.A = strided(q + a0, mat()); p.args.lda = n;
         p.args.B = strided(q + c0, mat()); p.args.ldb = n;
         p.args.C = strided(w, w_stride); p.args.ldc = width;
-        if (w_all > w_used) {
+        if (k <= NB && width <= NB && w_all > w_used) {
             p.args.workspace = w + w_used;
             p.args.workspace_floats = w_all - w_used;
         }
