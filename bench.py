@@ -147,6 +147,7 @@ def precond_step_gpu(torch, variant="shampoo1"):
     if variant == "shampoo2":
         bank = next(iter(opt._fused_cache.values()))["bank"]
         more["matrices_redone_with_library_qr"] = bank.qr_fallbacks
+        more["matrices_swept_again_with_replacement"] = bank.qr_repairs
         more["cholesky_qr_rounds_per_stack_and_update"] = round(bank.qr_rounds / (30 * len(bank.per_order)), 2)
         more["subspace_iteration_updates"] = 30 * sum(bank.per_order.values())
     import qtensor.fused as X

@@ -280,6 +280,16 @@ void qtensor_hip_cholesky_upper_floor_batched(float *gram, float *u, float *x, i
 int qtensor_hip_block_gram_schmidt_width(void);
 void qtensor_hip_block_gram_schmidt_batched(float *q, float *w, float *gram, float *u, float *x, const float *fill, int *info,
                                             int n, int batch, float pivot_floor, float null_norm2, qtensor_stream_t stream);
+/* The same sweep; with replace_dependent != 0 (needs fill and pivot_floor > 0) a column that the first pass finds
+ * dependent on the columns before it inside its 64-column panel (pivot at or below the floor) is replaced by its
+ * stand-in column from fill before the second pass as well (bit 2 of info[b]), instead of being handed to the second pass
+ * as it is (bit 1 if it is dependent there again).  For matrices of low numerical rank, where what a first pass leaves
+ * of such a column is rounding noise: the plain sweep ends with columns that are not orthogonal there.  The last
+ * 4 * batch floats of w then hold which columns were set aside.  (No counterpart in the reference: Householder QR
+ * completes a rank-deficient basis by construction.) */
+void qtensor_hip_block_gram_schmidt_replacing_batched(float *q, float *w, float *gram, float *u, float *x, const float *fill,
+                                                      int *info, int n, int batch, float pivot_floor, float null_norm2,
+                                                      int replace_dependent, qtensor_stream_t stream);
 /* The test that ends the rounds: out[2 b] = max |G_b - I|, out[2 b + 1] = ||G_b - I||_F^2 for the stack
  * gram [batch, n, n], one pass, fixed summation order, NaN if G_b holds one.  partial: scratch of
  * batch * 64 floats.  (No counterpart in the reference: Householder QR needs no such test.) */

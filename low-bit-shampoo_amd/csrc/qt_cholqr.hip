@@ -37,6 +37,8 @@ constexpr int kSolvePanel = 256;       // diagonal blocks of the factor are inve
 // factor that turns G_j,> into the block row U_j,> with zero rows for the dropped columns.
 // With pivot_floor == 0, and for a NaN pivot always, bit 0 of info[b] is set, the pivot is replaced by 1 and
 // the factor of that matrix is meaningless.
+// `set_aside`, if not null: the columns taken out are reported there (bit k of set_aside[b * aside_stride]) instead of in info, and
+// their columns of `inv` are zero, so that Q inv has zero columns in their place for the caller to fill.
 //
 // Lane i keeps row i of the (full, symmetric) trailing matrix in registers.  Step k scales column k
 // (one value per lane) into column k of L = U^T, parks it in LDS, and every lane reads it back as
@@ -52,7 +54,8 @@ __device__ __forceinline__ float lane_value(float x, int lane) {
 
 __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long long g_stride, int ldg, float *u,
                                                         long long u_stride, int ldu, float *inv, long long inv_stride,
-                                                        int ldi, float *panel_inv, int *info, float pivot_floor) {
+                                                        int ldi, float *panel_inv, int *info, float pivot_floor,
+                                                        unsigned long long *set_aside, int aside_stride) {
     __shared__ __attribute__((aligned(16))) float cols[NB][LDC];
     const int b = blockIdx.x, lane = threadIdx.x;
     const float *G = gram + (long long)b * g_stride;
@@ -119,6 +122,13 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
     float *I = inv + (long long)b * inv_stride + (long long)lane * ldi;
 #pragma unroll
     for (int r = 0; r < NB; ++r) U[(long long)r * ldu + lane] = r <= lane ? row[r] : 0.0f;        // U[r][lane] = L[lane][r]
+    if (set_aside != nullptr) {
+#pragma unroll
+        for (int c = 0; c < NB; ++c)
+            if ((dropped >> c) & 1ull) s[c] = 0.0f;
+        if (lane == 0) set_aside[(long long)b * aside_stride] = dropped;
+        dropped = 0;
+    }
 #pragma unroll
     for (int c = 0; c < NB; c += 4)              // U^-1[lane][c] = L^-1[c][lane] = s[c] of this lane (zero for c < lane)
         *reinterpret_cast<float4 *>(I + c) = make_float4(s[c], s[c + 1], s[c + 2], s[c + 3]);
@@ -283,6 +293,25 @@ __global__ __launch_bounds__(256) void panel_rescale_kernel(float *panel, long l
     }
 }
 
+// The columns that the first pass over an outer panel set aside (bit j of aside[b * aside_stride + p]: column 64 p + j of
+// the panel, a zero column by now) take the same columns of `fill`; bit 2 of info[b] is set.  Launched over
+// (kNormChunks row chunks, batch) like the kernels above.
+__global__ __launch_bounds__(256) void fill_aside_kernel(float *panel, long long stride, int ld, int n, int panels, int aside_stride,
+                                                         const unsigned long long *aside, const float *fill, int fill_ld, int *info) {
+    const int chunk = blockIdx.x, b = blockIdx.y, c = threadIdx.x & 63, g = threadIdx.x >> 6;
+    float *P = panel + (long long)b * stride;
+    const int rows = (n + kNormChunks - 1) / kNormChunks, r0 = chunk * rows, r1 = min(r0 + rows, n);
+    bool any = false;
+    for (int p = 0; p < panels; ++p) {
+        const unsigned long long m = aside[(long long)b * aside_stride + p];
+        if (m == 0) continue;
+        any = true;
+        if ((m >> c) & 1ull)
+            for (int r = r0 + g; r < r1; r += 4) P[(long long)r * ld + p * NB + c] = fill[(long long)r * fill_ld + p * NB + c];
+    }
+    if (any && chunk == 0 && threadIdx.x == 0) atomicOr(info + b, 4);
+}
+
 qtensor_batch_ptr strided(const float *base, long long stride) {
     qtensor_batch_ptr p;
     p.base = base;
@@ -332,7 +361,7 @@ extern "C" void qtensor_hip_cholesky_upper_floor_batched(float *gram, float *u, 
             // (the block of u right below the diagonal block is free: it takes the factor for the block row)
             float *panel_inv = rest > 0 ? u + (long long)j1 * n + j0 : nullptr;
             hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram + corner, mat, n, u + corner, mat, n,
-                               x + corner, mat, n, panel_inv, info, pivot_floor);
+                               x + corner, mat, n, panel_inv, info, pivot_floor, (unsigned long long *)nullptr, 0);
             if (!launch_ok("cholesky_upper_batched (diagonal block)")) return;
             if (rest == 0) break;
             const long long row = (long long)j0 * n + j1;
@@ -387,7 +416,12 @@ struct Sweep {
     int n, batch, w_cols;
     float pivot_floor, null_norm2;
     hipStream_t stream;
+    bool replace;                                             // columns a first pass finds dependent inside their panel are replaced too
     long long mat() const { return (long long)n * n; }
+    // replace: the tail of w holds, per matrix and 64-column panel of the current outer panel, which columns the
+    // first pass set aside (w_cols / 64 words of 64 bits per matrix)
+    long long w_floats() const { return (long long)batch * n * w_cols - (replace ? 2LL * batch * (w_cols / NB) : 0); }
+    unsigned long long *aside_words() const { return reinterpret_cast<unsigned long long *>(w + w_floats()); }
 
     // columns [c0, c0 + width) -= Q[:, a0:c0] (Q[:, a0:c0]^T columns): the columns a0..c0 are orthonormal
     bool project(int a0, int c0, int width) {
@@ -397,7 +431,7 @@ struct Sweep {
         // products when the product is cut along k (one 64 x 64 tile per matrix and a k range of n: few, long workgroups).
         // Only for a panel against its neighbour: cutting the products against all earlier panels as well is a little
         // faster for one stack alone and costs the optimizer step, where three stacks share the device, a third.
-        const long long w_stride = (long long)k * width, w_used = w_stride * batch, w_all = (long long)batch * n * w_cols;
+        const long long w_stride = (long long)k * width, w_used = w_stride * batch, w_all = w_floats();
         qtensor_gemm_desc p = {};                             // W = Q_a^T Y
         p.M = k; p.N = width; p.K = n; p.batch = batch;
         p.kind_a = QTENSOR_DENSE_T; p.kind_b = QTENSOR_DENSE; p.epilogue = QTENSOR_EPI_STORE;
@@ -420,43 +454,52 @@ struct Sweep {
         return run(r, stream);
     }
 
-    // The 64 columns from c0 on: `passes` times { take the columns a0..c0 out, unit columns, Cholesky QR rounds
-    // inside (two the first time, one afterwards) }.
-    bool panel(int a0, int c0, int passes, int first_rounds, bool may_fill) {
+    // The 64 columns from c0 on, in pass `pass` of `passes` over their outer panel (which starts at column a0): take the
+    // columns a0..c0 out, unit columns, one Cholesky QR round inside.
+    // Stand-in columns: in the first pass a column shorter than sqrt(null_norm2) after the projections (it was a unit
+    // column before them: what is left is rounding noise) takes its column of `fill`.  In replace mode every pass but
+    // the last also sets aside the columns whose pivot inside the panel is at or below the floor -- they leave the
+    // pass as zero columns and come back as stand-in columns before the next one (fill_aside_kernel) -- and the
+    // passes between the first and the last replace a column that a projection shortens to less than half (it
+    // was orthonormalised a pass earlier: losing most of its length again means it was noise then).
+    bool panel(int a0, int c0, int pass, int passes) {
         float *panel_ptr = q + c0;
+        const bool more = pass + 1 < passes;
+        // (word (c0 - a0) / 64 of the outer panel, matrices w_cols / 64 words apart -- see fill_aside_kernel)
+        unsigned long long *aside = replace && more ? aside_words() + (c0 - a0) / NB : nullptr;
+        const float *stand_in = fill == nullptr ? nullptr : pass == 0 || (replace && more) ? fill + c0 : nullptr;
+        const float too_short = pass == 0 ? null_norm2 : 0.25f;
+        // The last pass of replace mode normalises whatever has a pivot above the noise of the Gram matrix: a stand-in
+        // column for one of the last columns of a matrix has little room left (the complement of a thousand columns in
+        // a space of as many dimensions), which is a small pivot and no dependence.
+        const float floor_here = replace && !more && pivot_floor > 1e-6f ? 1e-6f : pivot_floor;
         const long long small = (long long)NB * NB;
         float *norms = u;                                     // [batch][kNormChunks][64]: u is free between factorisations
-        for (int pass = 0; pass < passes; ++pass) {
-            if (!project(a0, c0, NB)) return false;
-            hipLaunchKernelGGL(panel_norms_kernel, dim3(kNormChunks, batch), dim3(256), 0, stream, panel_ptr, mat(), n, n, norms);
-            hipLaunchKernelGGL(panel_rescale_kernel, dim3(kNormChunks, batch), dim3(256), 0, stream, panel_ptr, mat(), n, n, norms,
-                               may_fill && pass == 0 && fill != nullptr ? fill + c0 : nullptr, n, null_norm2, info);
-            if (!launch_ok("block_gram_schmidt_batched (normalize)")) return false;
-            const int rounds = pass == 0 ? first_rounds : 1;
-            for (int round = 0; round < rounds; ++round) {
-                qtensor_gemm_desc g = {};                     // S = Y_p^T Y_p
-                g.M = NB; g.N = NB; g.K = n; g.batch = batch;
-                g.kind_a = QTENSOR_DENSE_T; g.kind_b = QTENSOR_DENSE; g.epilogue = QTENSOR_EPI_STORE;
-                g.args.A = strided(panel_ptr, mat()); g.args.lda = n;
-                g.args.B = strided(panel_ptr, mat()); g.args.ldb = n;
-                g.args.C = strided(gram, small); g.args.ldc = NB;
-                g.args.workspace = w;                         // one tile per matrix and a long k range: cut along k
-                g.args.workspace_floats = (long long)batch * n * w_cols;
-                if (!run(g, stream)) return false;
-                hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram, small, NB, u, small, NB, x, small, NB,
-                                   (float *)nullptr, info, pivot_floor);
-                if (!launch_ok("block_gram_schmidt_batched (panel factor)")) return false;
-                qtensor_gemm_desc t = {};                     // Y_p <- Y_p U^-1 (one tile column: in place is safe)
-                t.M = n; t.N = NB; t.K = NB; t.batch = batch;
-                t.kind_a = QTENSOR_DENSE; t.kind_b = QTENSOR_DENSE; t.epilogue = QTENSOR_EPI_STORE;
-                t.args.A = strided(panel_ptr, mat()); t.args.lda = n;
-                t.args.B = strided(x, small); t.args.ldb = NB;
-                t.args.C = strided(panel_ptr, mat()); t.args.ldc = n;
-                t.args.triangular = 2;
-                if (!run(t, stream)) return false;
-            }
-        }
-        return true;
+        if (!project(a0, c0, NB)) return false;
+        hipLaunchKernelGGL(panel_norms_kernel, dim3(kNormChunks, batch), dim3(256), 0, stream, panel_ptr, mat(), n, n, norms);
+        hipLaunchKernelGGL(panel_rescale_kernel, dim3(kNormChunks, batch), dim3(256), 0, stream, panel_ptr, mat(), n, n, norms,
+                           stand_in, n, too_short, info);
+        if (!launch_ok("block_gram_schmidt_batched (normalize)")) return false;
+        qtensor_gemm_desc g = {};                             // S = Y_p^T Y_p
+        g.M = NB; g.N = NB; g.K = n; g.batch = batch;
+        g.kind_a = QTENSOR_DENSE_T; g.kind_b = QTENSOR_DENSE; g.epilogue = QTENSOR_EPI_STORE;
+        g.args.A = strided(panel_ptr, mat()); g.args.lda = n;
+        g.args.B = strided(panel_ptr, mat()); g.args.ldb = n;
+        g.args.C = strided(gram, small); g.args.ldc = NB;
+        g.args.workspace = w;                                 // one tile per matrix and a long k range: cut along k
+        g.args.workspace_floats = w_floats();
+        if (!run(g, stream)) return false;
+        hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram, small, NB, u, small, NB, x, small, NB,
+                           (float *)nullptr, info, floor_here, aside, w_cols / NB);
+        if (!launch_ok("block_gram_schmidt_batched (panel factor)")) return false;
+        qtensor_gemm_desc t = {};                             // Y_p <- Y_p U^-1 (one tile column: in place is safe)
+        t.M = n; t.N = NB; t.K = NB; t.batch = batch;
+        t.kind_a = QTENSOR_DENSE; t.kind_b = QTENSOR_DENSE; t.epilogue = QTENSOR_EPI_STORE;
+        t.args.A = strided(panel_ptr, mat()); t.args.lda = n;
+        t.args.B = strided(x, small); t.args.ldb = NB;
+        t.args.C = strided(panel_ptr, mat()); t.args.ldc = n;
+        t.args.triangular = 2;
+        return run(t, stream);
     }
 };
 
@@ -476,12 +519,22 @@ extern "C" int qtensor_hip_block_gram_schmidt_width(void) {
 extern "C" void qtensor_hip_block_gram_schmidt_batched(float *q, float *w, float *gram, float *u, float *x, const float *fill,
                                                        int *info, int n, int batch, float pivot_floor, float null_norm2,
                                                        void *stream_v) {
+    qtensor_hip_block_gram_schmidt_replacing_batched(q, w, gram, u, x, fill, info, n, batch, pivot_floor, null_norm2, 0, stream_v);
+}
+
+extern "C" void qtensor_hip_block_gram_schmidt_replacing_batched(float *q, float *w, float *gram, float *u, float *x,
+                                                                 const float *fill, int *info, int n, int batch, float pivot_floor,
+                                                                 float null_norm2, int replace_dependent, void *stream_v) {
     using namespace qt;
     clear_error();
     if (!stack_args_ok("block_gram_schmidt_batched", n, batch, {q, w, gram, u, x, info})) return;
     if (!(pivot_floor >= 0.0f) || !(null_norm2 >= 0.0f)) { set_error(kBadArgument, "block_gram_schmidt_batched: negative threshold"); return; }
+    if (replace_dependent != 0 && (fill == nullptr || !(pivot_floor > 0.0f))) {
+        set_error(kBadArgument, "block_gram_schmidt_batched: replacing dependent columns needs fill columns and a pivot floor");
+        return;
+    }
     const int outer = qtensor_hip_block_gram_schmidt_width();
-    Sweep s = {q, w, gram, u, x, fill, info, n, batch, outer, pivot_floor, null_norm2, (hipStream_t)stream_v};
+    Sweep s = {q, w, gram, u, x, fill, info, n, batch, outer, pivot_floor, null_norm2, (hipStream_t)stream_v, replace_dependent != 0};
     // Two levels.  An outer panel of `outer` columns has the finished columns taken out of it as a whole (the
     // bulk of the arithmetic, as products with a wide right-hand side) and is then swept inside -- every
     // 64-column panel: take the earlier panels of the same outer panel out, unit columns, one Cholesky QR
@@ -490,12 +543,25 @@ extern "C" void qtensor_hip_block_gram_schmidt_batched(float *q, float *w, float
     // and orthogonal to the earlier columns, to fp32 rounding whatever the conditioning of the matrix (block
     // classical Gram-Schmidt with reorthogonalisation; the Cholesky QR inside a 64-column panel sees at most
     // that panel's own conditioning, and its pivot floor takes care of columns that depend on each other).
+    // replace_dependent: three passes instead of two.  A column that the first or the second pass finds dependent on
+    // the columns before it inside its 64-column panel (pivot at or below the floor) is not handed to the next pass as
+    // it is -- where it is rounding noise it depends on them again -- but leaves the pass as a zero column and enters
+    // the next one as a stand-in column from `fill`; so does a column that the second pass's projections shorten to
+    // less than half.  Every stand-in column is orthogonalised against everything before it at least once after it
+    // came in, every other column three times.
+    const int passes = s.replace ? 3 : 2;
     for (int o0 = 0; o0 < n; o0 += outer) {
         const int width = n - o0 < outer ? n - o0 : outer;
-        for (int pass = 0; pass < 2; ++pass) {
+        for (int pass = 0; pass < passes; ++pass) {
+            if (pass >= 1 && s.replace) {
+                // what the first pass set aside comes back as stand-in columns, ahead of everything the second pass does
+                hipLaunchKernelGGL(fill_aside_kernel, dim3(kNormChunks, batch), dim3(256), 0, s.stream, q + o0, s.mat(), n, n, width / NB,
+                                   outer / NB, s.aside_words(), fill + o0, n, info);
+                if (!launch_ok("block_gram_schmidt_batched (stand-in columns)")) return;
+            }
             if (!s.project(0, o0, width)) return;
             for (int c0 = o0; c0 < o0 + width; c0 += NB)
-                if (!s.panel(o0, c0, 1, 1, pass == 0)) return;
+                if (!s.panel(o0, c0, pass, passes)) return;
         }
     }
 }

@@ -40,6 +40,7 @@ class ShampooBank2(ShampooBank):
         self.rect_t1, self.rect_t2, self.inv_root_mode = rect_t1, rect_t2, inv_root_mode
         self.qr_fallbacks = 0                     # matrices that went through torch.linalg.qr so far
         self.qr_rounds = 0                        # Cholesky QR rounds so far, summed over the stacks
+        self.qr_repairs = 0                       # matrices that went through the replacing sweep so far (low numerical rank)
         self.alongside = None                     # callable that the next add_statistics runs next to its factorisations
         super().__init__(params, name2qmap, code, **kwargs)
 
@@ -180,6 +181,7 @@ class ShampooBank2(ShampooBank):
                 beside.join()
         self.qr_fallbacks += sum(redone.values())
         self.qr_rounds += sum(solver[o].rounds for o in orders)
+        self.qr_repairs += sum(solver[o].repairs for o in orders)
 
     @torch.no_grad()
     def compute_preconditioners(self, v0=None):

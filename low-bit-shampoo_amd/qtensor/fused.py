@@ -346,6 +346,9 @@ if F.lib is not None:
     F.lib.qtensor_hip_block_gram_schmidt_width.argtypes = []
     F.lib.qtensor_hip_block_gram_schmidt_batched.restype = None
     F.lib.qtensor_hip_block_gram_schmidt_batched.argtypes = [ct.c_void_p] * 7 + [ct.c_int, ct.c_int, ct.c_float, ct.c_float, ct.c_void_p]
+    F.lib.qtensor_hip_block_gram_schmidt_replacing_batched.restype = None
+    F.lib.qtensor_hip_block_gram_schmidt_replacing_batched.argtypes = ([ct.c_void_p] * 7 +
+                                                                       [ct.c_int, ct.c_int, ct.c_float, ct.c_float, ct.c_int, ct.c_void_p])
     F.lib.qtensor_hip_gram_deviation_batched.restype = None
     F.lib.qtensor_hip_gram_deviation_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
     F.lib.qtensor_hip_column_dots_batched.restype = None
@@ -392,12 +395,14 @@ def completion_columns(device: torch.device, n: int) -> Tensor:
 
 
 def block_gram_schmidt(q: Tensor, info: Tensor, pivot_floor: float = 2e-4, null_norm2: float = NULL_COLUMN_NORM2,
-                       complete: bool = True) -> Tensor:
+                       complete: bool = True, replace_dependent: bool = False) -> Tensor:
     """Orthonormalise the columns of every matrix of the stack q [B, n, n] (unit columns, n a multiple of 64)
     in place, left to right in panels of 64 columns: block Gram-Schmidt with reorthogonalisation, Cholesky QR
     inside a panel.  span(q[:, :, :k]) is kept for every k.  complete: columns that depend on the earlier ones
     up to rounding noise are replaced by fixed unit columns in general position (bit 2 of info[b]); info int32
-    [B], zeroed by the caller, bits as in cholesky_upper."""
+    [B], zeroed by the caller, bits as in cholesky_upper.  replace_dependent (needs complete): a column that the
+    first pass finds dependent inside its 64-column panel (pivot at or below pivot_floor) is replaced as well,
+    instead of being handed to the second pass as it is -- for matrices of low numerical rank."""
     B, n, _ = q.shape
     _stack(q, "q", (B, n, n))
     if info.dtype != torch.int32 or info.numel() != B or not info.is_cuda:
@@ -405,9 +410,11 @@ def block_gram_schmidt(q: Tensor, info: Tensor, pivot_floor: float = 2e-4, null_
     w = torch.empty(B, n, F.lib.qtensor_hip_block_gram_schmidt_width(), device=q.device)
     small = torch.empty(3, B, 64, 64, device=q.device)
     fill = completion_columns(q.device, n) if complete else None
-    F._call(F.lib.qtensor_hip_block_gram_schmidt_batched, q.device, q.data_ptr(), w.data_ptr(), small[0].data_ptr(),
+    if replace_dependent and fill is None:
+        raise ValueError("replace_dependent needs complete=True")
+    F._call(F.lib.qtensor_hip_block_gram_schmidt_replacing_batched, q.device, q.data_ptr(), w.data_ptr(), small[0].data_ptr(),
             small[1].data_ptr(), small[2].data_ptr(), None if fill is None else fill.data_ptr(), info.data_ptr(), n, B,
-            float(pivot_floor), float(null_norm2))
+            float(pivot_floor), float(null_norm2), int(bool(replace_dependent)))
     return q
 
 
@@ -511,12 +518,16 @@ class CholeskyQR:
         self.redo = []                                # matrices handed to the library at the end
         self.finished = False
         self.rounds = 0                               # factorisation rounds enqueued so far
+        self.repairs = 0                              # matrices swept a second time (see _repair)
         self.gram = self.far = None
         # The bookkeeping lives on the host (it waits once per round anyway), per working-set entry:
         # which matrix of the stack it is and whether it is within ||G - I||_F < 0.5.
         self.ids = np.arange(B)
         self.near = np.zeros(B, dtype=bool)
         self.last = None                              # (pivot flags, near, ids) of the round not yet looked at
+        self.was_far = np.zeros(B, dtype=bool)        # per working-set entry: far at the test before this one
+        self.mended = np.zeros(B, dtype=bool)         # per working-set entry: has been through the replacing sweep
+        self.stale = False                            # the Gram matrices are those of before a repair: no round on them
         self.swept = sweep
         if sweep:
             # One sweep of block Gram-Schmidt with reorthogonalisation.  Where no pivot of a panel factorisation
@@ -547,7 +558,7 @@ class CholeskyQR:
         self.Q = self.Q.index_select(0, index)
         if self.gram is not None:
             self.gram = self.gram.index_select(0, index)
-        self.ids, self.near = self.ids[keep], self.near[keep]
+        self.ids, self.near, self.was_far, self.mended = self.ids[keep], self.near[keep], self.was_far[keep], self.mended[keep]
 
     def check(self):
         if self.swept:
@@ -562,6 +573,20 @@ class CholeskyQR:
                 return
         self.gram = gemm(self.Q, self.Q, trans_a=True, symmetric=True)
         self.far = gram_deviation(self.gram)                                    # max |G - I|, ||G - I||_F^2
+
+    def _repair(self, where):
+        """The working-set entries `where` (host positions) are far from orthonormal after the sweep: matrices of low
+        numerical rank, where what a first pass leaves of a dependent column is rounding noise and a second pass
+        cannot mend it (columns end unnormalised or parallel, and Cholesky QR rounds on such a matrix diverge).  They
+        are swept again from their original columns, three passes, with every column that a pass finds dependent
+        replaced by a stand-in column (block_gram_schmidt(replace_dependent=True))."""
+        original = self.Y.index_select(0, self._index(self.ids[where]))
+        scale = torch.linalg.vector_norm(original, dim=1, keepdim=True).clamp_min(1e-30)
+        again = (original / scale).contiguous()
+        info = torch.zeros(again.shape[0], dtype=torch.int32, device=again.device)
+        block_gram_schmidt(again, info, self.pivot_floor, replace_dependent=True)
+        self.Q.index_copy_(0, self._index(where), again)
+        self.repairs += int(where.size)
 
     def _failures(self):
         """Host mask over the entries of the last round: the factorisation met a NaN."""
@@ -588,9 +613,26 @@ class CholeskyQR:
         self._finish(np.nonzero(done)[0], self.Q)
         self._keep(~(done | failed))
         self.finished = self.ids.size == 0
+        if not self.finished:
+            # A matrix that is far from orthonormal after the sweep usually has a few stand-in columns that are a
+            # little off, and one round mends it.  One that is far again after a round -- or a stack where every
+            # fourth matrix is far (eight at least) -- is of low numerical rank: rounds diverge there, the replacing
+            # sweep does not.
+            far = ~self.near
+            many = far.sum() >= 8 and far.sum() * 4 > self.Y.shape[0]
+            again = far & ~self.mended & (self.was_far | many)
+            if again.any():
+                self._repair(np.nonzero(again)[0])
+                self.mended |= again
+                self.stale = True
+                self.rounds_left = min(self.rounds_left, 3)   # what is far after the repair and three rounds goes to the library
+            self.was_far = far
         return self.finished
 
     def advance(self):
+        if self.stale:                                # repaired matrices are tested first (the next check())
+            self.stale, self.gram = False, None
+            return
         k = self.ids.size
         info = self.info[:k]
         info.zero_()

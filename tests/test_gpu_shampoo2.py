@@ -200,6 +200,83 @@ def test_rank_deficient_stacks_get_a_completed_basis(mods):
     assert float((Q3[1].T @ Q3[1] - torch.eye(n, device="cuda")).abs().max()) < 2e-5
 
 
+@pytest.mark.parametrize("cond", [1e12, 1e16])
+def test_stacks_of_low_numerical_rank_are_swept_again_with_replacement(mods, cond):
+    """Singular values that fall through the whole fp32 range: what the first pass of a plain sweep leaves of the
+    later columns is rounding noise that depends on the earlier columns again in the second pass, so it ends with
+    columns that are not orthogonal, and Cholesky QR rounds on such a matrix diverge.  The state machine sweeps these
+    matrices again with every dependent column replaced by a stand-in: orthonormal to rounding, the leading columns
+    span what Householder's span, nothing goes to the library routine."""
+    import numpy as np
+    import qtensor.fused as X
+    n, batch = 256, 16
+    g = torch.Generator().manual_seed(n + int(np.log10(cond)))
+    U, _ = torch.linalg.qr(torch.randn(batch, n, n, generator=g, dtype=torch.float64))
+    V, _ = torch.linalg.qr(torch.randn(batch, n, n, generator=g, dtype=torch.float64))
+    lam = torch.logspace(0, -float(np.log10(cond)), n, dtype=torch.float64)
+    Y = ((U * lam) @ V.transpose(1, 2)).float()
+    Y = (Y / torch.linalg.vector_norm(Y, dim=1, keepdim=True)).cuda().contiguous()
+    eye = torch.eye(n, device="cuda")
+    plain = Y.clone()
+    info = torch.zeros(batch, dtype=torch.int32, device="cuda")
+    X.block_gram_schmidt(plain, info)
+    far = (plain.transpose(1, 2) @ plain - eye).abs().amax(dim=(1, 2)) > 0.3
+    assert int(far.sum()) >= batch // 2 and bool((info != 0).all())         # the case this test is about
+    state = X.CholeskyQR(Y)
+    while not state.finished:
+        state.check()
+        if not state.poll():
+            state.advance()
+    Q, redone = state.result()
+    assert redone == 0 and state.repairs >= int(far.sum()) and state.rounds <= 3
+    assert float((Q.transpose(1, 2) @ Q - eye).abs().max()) < 5e-5
+    Qh, _ = torch.linalg.qr(Y.double().cpu())
+    k = n // 8                                                               # singular values down to cond^(-1/8)
+    lead = Q[:, :, :k].double().cpu()
+    resid = Qh[:, :, :k] - lead @ (lead.transpose(1, 2) @ Qh[:, :, :k])
+    assert float(resid.norm(dim=1).max()) < 2e-5
+    # the replacing sweep on its own: three passes, stand-ins flagged; what it leaves far (a stand-in for one of the
+    # last columns with next to nothing of it outside the span of the others) is few and within reach of a round
+    again = Y.clone()
+    info.zero_()
+    X.block_gram_schmidt(again, info, replace_dependent=True)
+    assert bool(((info & 4) != 0).all()) and bool(((info & 1) == 0).all())
+    still = (again.transpose(1, 2) @ again - eye).abs().amax(dim=(1, 2)) > 0.3
+    assert int(still.sum()) <= batch // 4 and int(still.sum()) < int(far.sum())
+    with pytest.raises(ValueError):
+        X.block_gram_schmidt(again, info, complete=False, replace_dependent=True)
+
+
+def test_low_rank_gradients_do_not_reach_the_library_qr(mods, tmp_path, monkeypatch):
+    """Gradients of rank two plus a little noise (a small batch): every statistic has a few large directions and a
+    floor, the regime in which the plain sweep is not enough.  The bank must get through on its own kernels."""
+    monkeypatch.chdir(tmp_path)
+    S2, E2 = mods
+    from optimizers.shampoo_common import build_code_maps
+    import qtensor.fused as X
+    g = torch.Generator(device="cuda").manual_seed(5)
+    params = [torch.zeros(512, 384, device="cuda"), torch.zeros(256, 640, device="cuda")]
+    bank = E2.ShampooBank2(params, build_code_maps(4), "linear-2", inv_root_mode=1, **KW)
+    for _ in range(6):
+        grads = []
+        for p in params:
+            a = torch.randn(p.shape[0], 2, device="cuda", generator=g)
+            b = torch.randn(2, p.shape[1], device="cuda", generator=g)
+            grads.append(0.02 * (a @ b) + 1e-4 * torch.randn(p.shape, device="cuda", generator=g))
+        bank.add_statistics(grads)
+    assert bank.qr_fallbacks == 0
+    for order in bank.per_order:
+        vt = X.dequantize_stack(bank.basis[order])
+        gram = vt @ vt.transpose(1, 2)
+        assert bool(torch.isfinite(vt).all())
+        # rows of a 4-bit basis are orthonormal up to the quantization error
+        assert float((gram - torch.eye(order, device="cuda")).abs().max()) < 0.35
+    bank.compute_preconditioners()
+    out = bank.preconditioned_grads(grads)
+    assert all(bool(torch.isfinite(o).all()) for o in out)
+    print("matrices swept again:", bank.qr_repairs, "rounds:", bank.qr_rounds)
+
+
 def test_pivot_floor_takes_a_dependent_column_out_of_the_factorisation(mods):
     import qtensor.fused as X
     g = torch.Generator().manual_seed(23)
