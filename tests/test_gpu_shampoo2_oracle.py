@@ -230,3 +230,33 @@ def test_gaussian_gradients_follow_the_oracle_in_what_the_optimizer_uses(mods, c
     print("preconditioned gradients (fp32 oracle vs float64, device vs float64, device vs fp32 oracle)", rows,
           "differing codes of the inverse roots", trio.root_flips)
     assert all(dev <= 2 * ref + 2e-3 and direct <= 1e-2 for ref, dev, direct in rows)
+
+
+@pytest.mark.parametrize("mode", [1, 0])
+def test_vanishing_gradients_end_where_the_oracle_ends(mods, code_maps, mode, tmp_path, monkeypatch):
+    """All-zero gradients: the reference's update keeps the smaller half of the Rayleigh quotients, which is the half
+    the rebuilt statistic (rank n/2) does not reach -- zeros -- so after two updates the statistic is exactly zero and
+    its inverse root is not finite.  The device paths must not invent anything else: same stored quotients, and
+    non-finite roots where the oracle's are."""
+    monkeypatch.chdir(tmp_path)
+    code = code_maps[("linear-2", 4)]
+    shapes = [(128, 192), (256, 128)]
+    trio = Trio(mods, code, shapes, mode, KW)
+    grads = [torch.zeros(s) for s in shapes]
+    for st in range(3):
+        trio.adopt_oracle_state()
+        trio.update(grads)
+    for entry in trio.table:
+        pi, j, side, order, row = entry
+        slot = trio.refs[pi].stats[2 * j + side]
+        assert float(slot.svalue.abs().max()) == 0.0 and float(slot.max_eig) == 0.0
+        for name, c, a, s, k, mx, stat in trio.device_states(*entry):
+            assert float(s.abs().max()) == 0.0 and float(mx) == 0.0, name
+            assert float(stat.abs().max()) == 0.0, name
+    assert trio.bank.qr_fallbacks == 0
+    trio.adopt_oracle_state()
+    want, _, per, bank = trio.roots_and_directions(grads, 5)
+    for w, p_, b in zip(want, per, bank):
+        assert not bool(torch.isfinite(torch.as_tensor(w)).all())
+        assert not bool(torch.isfinite(p_).all()) and not bool(torch.isfinite(b).all())
+
