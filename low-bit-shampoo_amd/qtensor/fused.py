@@ -528,7 +528,8 @@ class CholeskyQR:
         self.ids = np.arange(B)
         self.near = np.zeros(B, dtype=bool)
         self.last = None                              # (pivot flags, near, ids) of the round not yet looked at
-        self.was_far = np.zeros(B, dtype=bool)        # per working-set entry: far at the test before this one
+        self.far_before = np.full(B, np.inf)          # per working-set entry: ||G - I||_F^2 at the test before this one if it was far
+        self.stuck = np.zeros(B, dtype=np.int64)      # per working-set entry: rounds in a row that did not halve that distance
         self.mended = np.zeros(B, dtype=bool)         # per working-set entry: has been through the replacing sweep
         self.stale = False                            # the Gram matrices are those of before a repair: no round on them
         self.swept = sweep
@@ -561,7 +562,8 @@ class CholeskyQR:
         self.Q = self.Q.index_select(0, index)
         if self.gram is not None:
             self.gram = self.gram.index_select(0, index)
-        self.ids, self.near, self.was_far, self.mended = self.ids[keep], self.near[keep], self.was_far[keep], self.mended[keep]
+        self.ids, self.near, self.mended = self.ids[keep], self.near[keep], self.mended[keep]
+        self.far_before, self.stuck = self.far_before[keep], self.stuck[keep]
 
     def check(self):
         if self.swept:
@@ -614,22 +616,26 @@ class CholeskyQR:
         done &= ~failed
         self.redo += self.ids[failed].tolist()
         self._finish(np.nonzero(done)[0], self.Q)
+        distance = far[:, 1][~(done | failed)]
         self._keep(~(done | failed))
         self.finished = self.ids.size == 0
         if not self.finished:
             # A matrix that is far from orthonormal after the sweep usually has a few stand-in columns that are a
-            # little off, and one round mends it.  One that is far again after a round -- or a stack where every
-            # fourth matrix is far (eight at least) -- is of low numerical rank: rounds diverge there, the replacing
-            # sweep does not.
-            far = ~self.near
-            many = far.sum() >= 8 and far.sum() * 4 > self.Y.shape[0]
-            again = far & ~self.mended & (self.was_far | many)
+            # little off, and a round or two mend it (a round may first throw it further off).  One that two rounds
+            # in a row did not bring nearer than half of before -- or a stack where every fourth matrix is far (eight
+            # at least) -- is of low numerical rank: rounds diverge there, the replacing sweep does not.
+            away = ~self.near
+            many = away.sum() >= 8 and away.sum() * 4 > self.Y.shape[0]
+            with np.errstate(invalid="ignore"):
+                no_nearer = away & np.isfinite(self.far_before) & ~(distance < 0.5 * self.far_before)      # (NaN and inf count)
+            self.stuck = np.where(no_nearer, self.stuck + 1, 0)
+            again = away & ~self.mended & ((self.stuck >= 2) | many)
             if again.any():
                 self._repair(np.nonzero(again)[0])
                 self.mended |= again
                 self.stale = True
                 self.rounds_left = min(self.rounds_left, 3)   # what is far after the repair and three rounds goes to the library
-            self.was_far = far
+            self.far_before = np.where(away, distance, np.inf)
         return self.finished
 
     def advance(self):
