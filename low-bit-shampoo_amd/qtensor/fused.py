@@ -489,10 +489,10 @@ class CholeskyQR:
     PIVOT_FLOOR takes its column out of that factorisation (cholesky_upper) instead of failing it.
 
     Once ||G - I||_F < 0.5 one Cholesky QR round makes Q orthonormal to fp32 rounding and the matrix leaves
-    the working set without a further test.  A matrix that is farther than that again after a round (or a
-    stack where every fourth matrix is that far right after the sweep) is of low numerical rank: rounds
-    diverge there, and it is swept again from its original columns with every dependent column replaced by
-    a stand-in (_repair).  Matrices that still are far three rounds after that, or after max_rounds, or whose
+    the working set without a further test.  A matrix that is farther than that and that two rounds in a row
+    did not bring nearer than half of before (or a stack where every fourth matrix is that far right after
+    the sweep) is of low numerical rank: rounds diverge there, and it is swept again from its original
+    columns with every dependent column replaced by a stand-in (_repair).  Matrices that still are far three rounds after that, or after max_rounds, or whose
     factorisation meets a NaN, go through torch.linalg.qr.  Orders that are not a multiple of 64 are padded
     with an identity block (QR of diag(Y, I) is diag(Q, I)).
 
