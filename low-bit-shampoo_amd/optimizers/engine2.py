@@ -23,7 +23,7 @@ finished this way are redone with torch.linalg.qr.
 """
 import torch
 
-from optimizers.engine import ShampooBank, SideJob
+from optimizers.engine import BESIDE_SLOT, EARLY_SLOT, ShampooBank, SideJob, shared_stream
 from optimizers.matrix_functions import ComputePowerBatched
 from qtensor import fused as X
 
@@ -45,18 +45,14 @@ class ShampooBank2(ShampooBank):
         super().__init__(params, name2qmap, code, **kwargs)
 
     def _early_stream(self):
-        if getattr(self, "_early", None) is None:
-            self._early = torch.cuda.Stream(device=self.device)
-        return self._early
+        return shared_stream(self.device, EARLY_SLOT)
 
     def _beside_stream(self):
         # the side stream that no order's chain runs on, if there is one: a stream more would share a hardware queue
         # with one of the chains (23.3 against 24.1 ms per regular step)
         if len(self.streams) > len(self.per_order):
             return self.streams[-1]
-        if getattr(self, "_beside", None) is None:
-            self._beside = torch.cuda.Stream(device=self.device)
-        return self._beside
+        return shared_stream(self.device, BESIDE_SLOT)
 
     def _init_statistics(self):
         """Basis = quantized identity, every kept quotient and the largest one = matrix_eps

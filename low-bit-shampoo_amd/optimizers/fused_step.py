@@ -3,7 +3,7 @@ ShampooBank (no counterpart in the reference, whose step() walks the parameters 
 optimizers/shampoo1.py:371-427, shampoo2.py:412-468), and the checkpointing of that bank."""
 import torch
 
-from optimizers.engine import SideJob as _SideJob
+from optimizers.engine import UNBATCHED_SLOT as _UNBATCHED_SLOT, SideJob as _SideJob, shared_stream as _shared_stream
 from optimizers.shampoo_common import CODE
 
 
@@ -138,7 +138,7 @@ def fused_step(opt, group, update, group_index=0):
     if (bank is not None and unbatched and opt.overlap_unbatched_statistics and step % group['stat_compute_steps'] == 0
             and all('preconditioner' in opt.state[p] for p in unbatched)):
         if entry.get('side_stream') is None:
-            entry['side_stream'] = torch.cuda.Stream(device=unbatched[0].device)
+            entry['side_stream'] = _shared_stream(unbatched[0].device, _UNBATCHED_SLOT)
 
         def update_unbatched():
             for q in unbatched:
@@ -165,7 +165,7 @@ def fused_step(opt, group, update, group_index=0):
             if (unbatched and opt.overlap_unbatched_inverse_roots
                     and all('preconditioner' in opt.state[p] for p in unbatched)):
                 if entry.get('side_stream') is None:
-                    entry['side_stream'] = torch.cuda.Stream(device=unbatched[0].device)
+                    entry['side_stream'] = _shared_stream(unbatched[0].device, _UNBATCHED_SLOT)
                 if side_job is None and step % group['stat_compute_steps'] == 0:
                     for q in unbatched:                               # this step's statistics come before its roots
                         opt.state[q]['preconditioner'].add_statistics(grads[id(q)])
