@@ -42,10 +42,25 @@ class ShampooBank2(ShampooBank):
         self.qr_rounds = 0                        # Cholesky QR rounds so far, summed over the stacks
         self.qr_repairs = 0                       # matrices that went through the replacing sweep so far (low numerical rank)
         self.alongside = None                     # callable that the next add_statistics runs next to its factorisations
+        self.low_rank = {}                        # order -> [most of the stack needed the replacing sweep, updates since the plain one was tried]
         super().__init__(params, name2qmap, code, **kwargs)
 
     def _early_stream(self):
         return shared_stream(self.device, EARLY_SLOT)
+
+    LOOK_AGAIN = 8                                # updates after which a stack of low numerical rank tries the plain sweep again
+
+    def _replace_first(self, order):
+        """Whether this update of the stack starts with the replacing sweep: its last update with the plain sweep
+        needed the replacing one for more than a quarter of the matrices, fewer than LOOK_AGAIN updates ago."""
+        state = self.low_rank.setdefault(order, [False, 0])
+        if not state[0]:
+            return False
+        state[1] += 1
+        if state[1] >= self.LOOK_AGAIN:
+            state[1] = 0
+            return False
+        return True
 
     def _beside_stream(self):
         # the side stream that no order's chain runs on, if there is one: a stream more would share a hardware queue
@@ -113,7 +128,7 @@ class ShampooBank2(ShampooBank):
 
         def project(order):
             def run():
-                solver[order] = X.CholeskyQR(X.gemm(stat[order], basis[order], trans_b=True))     # L Vt^T
+                solver[order] = X.CholeskyQR(X.gemm(stat[order], basis[order], trans_b=True), replace_first=direct[order])     # L Vt^T
             return run
 
         def iterate(order):
@@ -135,6 +150,7 @@ class ShampooBank2(ShampooBank):
         # The Cholesky QR of every order advances on its own stream; the host waits once per round.
         # (_fan_out gives job i the stream i % streams, so an order keeps its stream from call to call.)
         solver, redone = {}, {}
+        direct = {o: self._replace_first(o) for o in orders}
         self._fan_out([project(o) for o in orders])
         # work of the caller that does not depend on the statistics (bank.alongside, consumed here) fills the device
         # next to the factorisations, on a thread and a stream of its own
@@ -178,6 +194,9 @@ class ShampooBank2(ShampooBank):
         self.qr_fallbacks += sum(redone.values())
         self.qr_rounds += sum(solver[o].rounds for o in orders)
         self.qr_repairs += sum(solver[o].repairs for o in orders)
+        for o in orders:
+            if not direct[o]:
+                self.low_rank[o][0] = solver[o].repairs * 4 > self.per_order[o]
 
     @torch.no_grad()
     def compute_preconditioners(self, v0=None):

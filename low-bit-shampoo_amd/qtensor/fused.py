@@ -502,7 +502,7 @@ class CholeskyQR:
     matrices still in the working set, result() returns (Q, number of matrices redone by the
     library).  All calls for one object must be made with the same current stream."""
 
-    def __init__(self, Y, max_rounds=12, pivot_floor=PIVOT_FLOOR, tolerance=2e-5, sweep=True):
+    def __init__(self, Y, max_rounds=12, pivot_floor=PIVOT_FLOOR, tolerance=2e-5, sweep=True, replace_first=False):
         if Y.dim() != 3 or Y.shape[1] != Y.shape[2] or Y.dtype != torch.float32 or not Y.is_cuda:
             raise ValueError("CholeskyQR takes an fp32 GPU stack [B, n, n]")
         B, self.true_n, _ = Y.shape
@@ -537,7 +537,11 @@ class CholeskyQR:
             # One sweep of block Gram-Schmidt with reorthogonalisation.  Where no pivot of a panel factorisation
             # came near the floor and no column had to be replaced (info == 0) the result is orthonormal to
             # fp32 rounding by construction; the rounds below are for the other matrices only.
-            block_gram_schmidt(self.Q, self.info, pivot_floor)
+            # replace_first: the caller knows the stack to be of low numerical rank (its last update needed the
+            # replacing sweep for most matrices) and goes there directly
+            block_gram_schmidt(self.Q, self.info, pivot_floor, replace_dependent=replace_first)
+            if replace_first:
+                self.mended[:] = True
 
     def _index(self, positions):
         return torch.as_tensor(np.ascontiguousarray(positions), dtype=torch.int64).to(self.Q.device)

@@ -245,6 +245,18 @@ def test_stacks_of_low_numerical_rank_are_swept_again_with_replacement(mods, con
     assert int(still.sum()) <= batch // 4 and int(still.sum()) < int(far.sum())
     with pytest.raises(ValueError):
         X.block_gram_schmidt(again, info, complete=False, replace_dependent=True)
+    # a caller that knows the stack goes to the replacing sweep directly: same outcome, no second sweep
+    direct = X.CholeskyQR(Y, replace_first=True)
+    while not direct.finished:
+        direct.check()
+        if not direct.poll():
+            direct.advance()
+    Qd, redone = direct.result()
+    assert redone == 0 and direct.repairs == 0 and direct.rounds <= 3
+    assert float((Qd.transpose(1, 2) @ Qd - eye).abs().max()) < 5e-5
+    lead = Qd[:, :, :k].double().cpu()
+    resid = Qh[:, :, :k] - lead @ (lead.transpose(1, 2) @ Qh[:, :, :k])
+    assert float(resid.norm(dim=1).max()) < 2e-5
 
 
 def test_low_rank_gradients_do_not_reach_the_library_qr(mods, tmp_path, monkeypatch):
@@ -275,6 +287,18 @@ def test_low_rank_gradients_do_not_reach_the_library_qr(mods, tmp_path, monkeypa
     out = bank.preconditioned_grads(grads)
     assert all(bool(torch.isfinite(o).all()) for o in out)
     print("matrices swept again:", bank.qr_repairs, "rounds:", bank.qr_rounds)
+    # A stack that needed the replacing sweep for most of its matrices starts there for the next updates and looks
+    # again after LOOK_AGAIN of them; with gradients of full rank the plain sweep is then enough and stays.
+    order = max(bank.per_order, key=bank.per_order.get)
+    bank.low_rank[order] = [True, 0]
+    fallbacks = bank.qr_fallbacks
+    for i in range(bank.LOOK_AGAIN):
+        full = [0.02 * torch.randn(p.shape, device="cuda", generator=g) for p in params]
+        bank.add_statistics(full)
+        assert bank.low_rank[order] == ([True, i + 1] if i + 1 < bank.LOOK_AGAIN else [False, 0])
+    assert bank.qr_fallbacks == fallbacks
+    vt = X.dequantize_stack(bank.basis[order])
+    assert float((vt @ vt.transpose(1, 2) - torch.eye(order, device="cuda")).abs().max()) < 0.35
 
 
 def test_pivot_floor_takes_a_dependent_column_out_of_the_factorisation(mods):
