@@ -46,6 +46,17 @@ def stress_tensor(torch, order, seed=0):
     return x
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(torch, x_slice, code):
     """The reference's CPU code path (per-segment torch loop) on a bounded sample: 1024 rows of
     the same tensor viewed as a 4096 x 4096 matrix (identical segments)."""
@@ -79,6 +90,7 @@ def cpu_baseline(torch, x_slice, code):
                   "quantize+dequantize with the per-segment torch loop of the reference's CPU path",
         "seconds": dt,
         "host_cpus": os.cpu_count(),
+        "cpu_model": cpu_model(),
         "torch_threads": torch.get_num_threads(),
     }
 
