@@ -180,15 +180,18 @@ class ShampooBank:
             done.record(side)
             main.wait_event(done)
 
-    def _run_on(self, slot, job):
+    def _run_on(self, slot, job, after_current=True):
         """Run one callable on side stream `slot` (the stream _fan_out gives job number `slot`), after what the
-        current stream holds; the current stream then waits for it."""
+        current stream holds; the current stream then waits for it.  after_current=False: only after what that
+        side stream holds itself -- for a job that goes on with the work of an earlier job on the same stream,
+        while the current stream has since been made to wait for other streams as well."""
         if not self.streams:
             job()
             return
         main = torch.cuda.current_stream(self.device)
         side = self.streams[slot % len(self.streams)]
-        side.wait_stream(main)
+        if after_current:
+            side.wait_stream(main)
         with torch.cuda.stream(side):
             job()
         main.wait_stream(side)

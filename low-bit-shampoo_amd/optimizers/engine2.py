@@ -21,9 +21,11 @@ QR; batched launches of libqtensor_hip.so), checked afterwards and polished by a
 where needed, which yields the same factor Q up to column signs.  Matrices that cannot be
 finished this way are redone with torch.linalg.qr.
 """
+import time
+
 import torch
 
-from optimizers.engine import BESIDE_SLOT, EARLY_SLOT, ShampooBank, SideJob, shared_stream
+from optimizers.engine import BESIDE_SLOT, ShampooBank, SideJob, shared_stream
 from optimizers.matrix_functions import ComputePowerBatched
 from qtensor import fused as X
 
@@ -44,9 +46,6 @@ class ShampooBank2(ShampooBank):
         self.alongside = None                     # callable that the next add_statistics runs next to its factorisations
         self.low_rank = {}                        # order -> [most of the stack needed the replacing sweep, updates since the plain one was tried]
         super().__init__(params, name2qmap, code, **kwargs)
-
-    def _early_stream(self):
-        return shared_stream(self.device, EARLY_SLOT)
 
     LOOK_AGAIN = 8                                # updates after which a stack of low numerical rank tries the plain sweep again
 
@@ -129,6 +128,10 @@ class ShampooBank2(ShampooBank):
         def project(order):
             def run():
                 solver[order] = X.CholeskyQR(X.gemm(stat[order], basis[order], trans_b=True), replace_first=direct[order])     # L Vt^T
+                # (the event that tells the host this stack's sweep is through goes right behind it: streams share
+                # hardware queues, and behind the launches of another stack's sweep it would wait for those as well)
+                tick[order] = torch.cuda.Event()
+                tick[order].record(torch.cuda.current_stream(self.device))
             return run
 
         def iterate(order):
@@ -149,46 +152,66 @@ class ShampooBank2(ShampooBank):
         self._fan_out([accumulate(g, side) for g in self.groups for side in (0, 1)])
         # The Cholesky QR of every order advances on its own stream; the host waits once per round.
         # (_fan_out gives job i the stream i % streams, so an order keeps its stream from call to call.)
-        solver, redone = {}, {}
+        solver, redone, tick = {}, {}, {}
         direct = {o: self._replace_first(o) for o in orders}
-        self._fan_out([project(o) for o in orders])
+        # Two lanes for the sweeps and what follows them: a process has four hardware queues, the parameters outside
+        # the bank and the job that applies the stored roots take one each, and streams beyond that share a queue in
+        # the order of their launches -- a third stack on a stream of its own ran behind the second anyway, and held
+        # up what the second had to do after its sweep.  The stacks are dealt out by cost, the cheap ones of a lane first.
+        lanes = [[] for _ in range(min(2, len(orders)))]
+        for o in orders:                                                   # (most expensive first)
+            min(lanes, key=lambda lane: sum(x ** 3 * self.per_order[x] for x in lane)).append(o)
+        lanes = [sorted(lane, key=lambda x: x ** 3 * self.per_order[x]) for lane in lanes]
+        slot = {o: i for i, lane in enumerate(lanes) for o in lane}
+        self._fan_out([(lambda lane=lane: [project(o)() for o in lane]) for lane in lanes])
         # work of the caller that does not depend on the statistics (bank.alongside, consumed here) fills the device
         # next to the factorisations, on a thread and a stream of its own
         beside, self.alongside = self.alongside, None
         if beside is not None:
             beside = SideJob(self.device, self._beside_stream(), beside)
-        # The stacks whose factorisation is complete go on (Rayleigh quotients, requantize) on a thread and a
-        # stream of their own while the others still iterate: the later rounds of a few ill-conditioned
-        # matrices are chains of small launches that leave most of the device, and this thread, waiting.
-        # The test after the sweep needs the host (it reads the sweep's flags, then the deviations of the flagged
-        # matrices), so the stacks are looked at in the order in which their sweeps end, cheapest first, and each
-        # goes through test, reading and polishing round in one go: the polishing of a few matrices of a cheap stack
-        # then runs while the sweep of the most expensive one is still under way.
-        slot = {o: i for i, o in enumerate(orders)}
-        by_finish = sorted(orders, key=lambda o: o ** 3 * self.per_order[o])
+        # Every stack goes on alone from here, on the stream that holds its sweep: the test after the sweep (the host
+        # reads the sweep's flags, then the deviations of the flagged matrices), a polishing round where needed, and
+        # as soon as it is finished its Rayleigh quotients and re-encoding -- none of it waits for the sweep of another
+        # stack (the current stream, which waits for all of them, is left out of it).  The host takes the stacks in the
+        # order in which their streams get there: it polls an event per stack.
+        unfinished = sorted(orders, key=lambda o: o ** 3 * self.per_order[o])
+        on_side = bool(self.streams)
+
+        def tick_of(order):
+            event = torch.cuda.Event()
+            event.record(self.streams[slot[order] % len(self.streams)] if on_side else torch.cuda.current_stream(self.device))
+            return event
+
+        tested = {o: False for o in orders}            # the test of the current iterate is queued, its outcome not read yet
 
         def look_at(order):
+            # one step of the stack's state machine; every read of the host in it finds its data there already,
+            # because the step before it ended with the event that is now through
             def run():
                 s = solver[order]
-                s.check()
-                if not s.finished and not s.poll():
-                    s.advance()
+                if not tested[order]:
+                    s.check()
+                    tested[order] = not s.finished
+                else:
+                    tested[order] = False
+                    if not s.poll():
+                        s.advance()
             return run
 
-        early, waiting = None, list(orders)
-        while not all(solver[o].finished for o in orders):
-            for o in by_finish:
-                if not solver[o].finished:
-                    self._run_on(slot[o], look_at(o))
-            ready = [o for o in waiting if solver[o].finished]
-            if self.streams and early is None and ready and len(ready) < len(waiting):
-                waiting = [o for o in waiting if o not in ready]
-                early = SideJob(self.device, self._early_stream(), lambda done=tuple(ready): [iterate(o)() for o in done])
         try:
-            self._fan_out([iterate(o) for o in waiting])
+            while unfinished:
+                ready = [o for o in unfinished if tick[o].query()]
+                if not ready:
+                    time.sleep(2e-5)
+                    continue
+                for o in sorted(ready, key=lambda x: -x ** 3 * self.per_order[x]):
+                    self._run_on(slot[o], look_at(o), after_current=False)
+                    if solver[o].finished:
+                        unfinished.remove(o)
+                        self._run_on(slot[o], iterate(o), after_current=False)
+                    else:
+                        tick[o] = tick_of(o)
         finally:
-            if early is not None:
-                early.join()
             if beside is not None:
                 beside.join()
         self.qr_fallbacks += sum(redone.values())
