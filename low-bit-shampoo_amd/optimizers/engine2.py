@@ -34,8 +34,9 @@ cholesky_qr = X.cholesky_qr
 
 
 class ShampooBank2(ShampooBank):
-    # One stream more than there are big stacks: measured on the ViT-B/32 shapes (three orders) 24.1 ms per regular step
-    # with four side streams against 25.7 with three, 24.9-25.2 with five or six (four hardware queues per process).
+    # Measured on the ViT-B/32 shapes (three orders, four hardware queues per process): 22.5 ms per regular step with
+    # three or four side streams, 23.7 with two, 26.7 with five (the job that applies the stored roots then shares
+    # a hardware queue with the longest sweep).
     DEFAULT_STREAMS = 4
 
     def __init__(self, params, name2qmap, code, *, rect_t1=1, rect_t2=4, inv_root_mode=0, **kwargs):
