@@ -41,22 +41,109 @@ class _Group:
 
 
 _SHARED_STREAMS = {}
+LANES = 2                                            # chains of launches the eigenbasis bank runs side by side
+BESIDE_SLOT, UNBATCHED_SLOT = 9, 10                  # fixed places in the pool, behind the fan-out streams (at most 8)
+
+
+def _same_queue(a, b, scratch):
+    """Whether work on stream b waits for work on stream a: a spins for a while, b gets one tiny launch.  (Twice: a
+    launch that the host is slow to make -- the first one of a kind -- looks like one that waited.)"""
+    waited = True
+    for _ in range(2):
+        torch.cuda.synchronize(scratch.device)
+        start, end_a, end_b = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+        with torch.cuda.stream(a):
+            start.record()
+            torch.cuda._sleep(1_000_000)
+            end_a.record()
+        with torch.cuda.stream(b):
+            scratch.add_(1)
+            end_b.record()
+        torch.cuda.synchronize(scratch.device)
+        waited = waited and start.elapsed_time(end_b) > 0.5 * start.elapsed_time(end_a)
+    return waited
+
+
+def _build_pool(index):
+    """The side streams of a device, by role.  A process has few hardware queues (four by default) and every stream
+    is bound to one of them when it is first used, in turn; streams on one queue run their launches in the order in
+    which the host made them.  Which of the bank's chains share a queue decides a fifth of the step time (22.3 ms
+    when the two sweep lanes, the parameters outside the bank and the current stream have a queue each, 26.5-27.5
+    when an application that made a stream or three of its own first shifts the turn), so the pool does not take
+    streams as they come: it makes a dozen, lets each one run something once (that binds it), finds out with a
+    spinning kernel which of them wait for each other, and hands them out by queue:
+      slot 0               the current stream's queue        (first lane of the sweeps; first stream of every fan-out)
+      slots 1, 2           a second queue                    (second lane; fan-outs)
+      slot 3, BESIDE_SLOT  a third queue                     (the job that applies the stored roots; fan-outs)
+      UNBATCHED_SLOT       the fourth queue                  (parameters outside the bank, on a thread)
+      every other slot     the current stream's queue"""
+    device = torch.device("cuda", index)
+    with torch.cuda.device(device):
+        current = torch.cuda.current_stream(device)
+        made = [torch.cuda.Stream(device=device) for _ in range(12)]
+        scratch = torch.zeros(64, device=device)
+        groups = [[current]]                                   # streams by hardware queue; the first group is the current stream's
+        if hasattr(torch.cuda, "_sleep"):
+            torch.cuda._sleep(1000)
+            for stream in made:
+                with torch.cuda.stream(stream):
+                    scratch.add_(1)
+            for stream in made:
+                for group in groups:
+                    if _same_queue(group[0], stream, scratch):
+                        group.append(stream)
+                        break
+                else:
+                    groups.append([stream])
+            torch.cuda.synchronize(device)
+        else:
+            groups += [[stream] for stream in made]            # no way to tell: as they come
+    own, others = groups[0][1:], [g for g in groups[1:] if g]
+    # the queues in the order of their turn, starting behind the current stream's: streams are bound in turn, so the
+    # queue of the stream made right after one of the current stream's queue is the next one, whatever else the
+    # process has bound before
+    if len(groups) > 1 and own:
+        turn = []
+        at = made.index(own[0])
+        for stream in made[at + 1:] + made[:at]:
+            group = next(g for g in groups if stream in g)
+            if group is not groups[0] and group not in turn:
+                turn.append(group)
+        others = turn + [g for g in others if g not in turn]
+    # Who may share a queue.  A stream that is told to wait for another one blocks its whole queue until then: the
+    # launches that other streams on that queue make in the meantime wait with it.  So
+    #   the job that applies the stored roots (made early, waits for the end of all sweeps) gets a queue to itself;
+    #   the thread of the parameters outside the bank (a long chain of small launches) gets one to itself: product
+    #     launches of a fan-out behind that chain would hold up a whole phase (22 -> 26.8 ms per step);
+    #   the second lane shares its queue only with a fan-out stream of the phases before the sweeps;
+    #   the first lane shares the current stream's queue: the current stream does little but wait, and what it waits
+    #     for is queued ahead of its barriers.
+    # (This is the arrangement a fresh process happens to get from streams taken in turn, 22.0 ms per step; the
+    # other ways round that were tried cost 1 to 5 ms.)
+    spare = own[1:] + [s for g in others for s in g[2:]]
+    if not spare:
+        spare = own or [g[0] for g in others] or made
+    pick = lambda k, j, fallback: others[k][j] if len(others) > k and len(others[k]) > j else fallback      # noqa: E731
+    pool = {0: own[0] if own else pick(0, 0, made[0])}
+    pool[1] = pick(0, 0, spare[0])
+    pool[2] = pick(0, 1, spare[0])
+    pool[3] = pool[BESIDE_SLOT] = pick(1, 0, spare[-1])
+    pool[UNBATCHED_SLOT] = pick(2, 0, spare[-1])
+    pool["spare"] = spare
+    return pool
 
 
 def shared_stream(device, slot):
-    """Side stream number `slot` of the device, the same object for every bank and optimizer of the process.
-    A device has few hardware queues (four per process by default) and streams are dealt out over them as they
-    are created: every bank bringing streams of its own puts the work chains of the second and third bank of a
-    process on queues they share (measured: 23 -> 26 ms per step for the second optimizer of a process)."""
+    """Side stream number `slot` of the device, the same object for every bank and optimizer of the process
+    (see _build_pool for which slot is what)."""
     device = torch.device(device)
     index = device.index if device.index is not None else torch.cuda.current_device()
-    pool = _SHARED_STREAMS.setdefault(index, [])
-    while len(pool) <= slot:
-        pool.append(torch.cuda.Stream(device=torch.device("cuda", index)))
+    if index not in _SHARED_STREAMS:
+        _SHARED_STREAMS[index] = _build_pool(index)
+    pool = _SHARED_STREAMS[index]
+    if slot not in pool:
+        pool[slot] = pool["spare"][slot % len(pool["spare"])]
     return pool[slot]
-
-
-EARLY_SLOT, BESIDE_SLOT, UNBATCHED_SLOT = 8, 9, 10    # fixed places in the pool, behind the chains' streams (at most 8)
 
 
 class SideJob:
@@ -142,7 +229,7 @@ class ShampooBank:
         # head of the next; biggest first.
         self.groups.sort(key=lambda g: -len(g) * g.bm * g.bn * (g.bm + g.bn))
         streams = self.DEFAULT_STREAMS if streams is None else streams
-        self.streams = [shared_stream(self.device, i) for i in range(min(streams, len(self.groups), EARLY_SLOT))]
+        self.streams = [shared_stream(self.device, i) for i in range(min(streams, len(self.groups), 8))]
 
     def _init_statistics(self):
         """Statistics start as matrix_eps * I, stored quantized with an exact diagonal."""

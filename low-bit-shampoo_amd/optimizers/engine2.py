@@ -25,7 +25,7 @@ import time
 
 import torch
 
-from optimizers.engine import BESIDE_SLOT, ShampooBank, SideJob, shared_stream
+from optimizers.engine import BESIDE_SLOT, LANES, ShampooBank, SideJob, shared_stream
 from optimizers.matrix_functions import ComputePowerBatched
 from qtensor import fused as X
 
@@ -63,11 +63,7 @@ class ShampooBank2(ShampooBank):
         return True
 
     def _beside_stream(self):
-        # the side stream that no order's chain runs on, if there is one: a stream more would share a hardware queue
-        # with one of the chains (23.3 against 24.1 ms per regular step)
-        if len(self.streams) > len(self.per_order):
-            return self.streams[-1]
-        return shared_stream(self.device, BESIDE_SLOT)
+        return shared_stream(self.device, BESIDE_SLOT)       # (the same stream as the fourth of the fan-out streams)
 
     def _init_statistics(self):
         """Basis = quantized identity, every kept quotient and the largest one = matrix_eps
@@ -159,7 +155,7 @@ class ShampooBank2(ShampooBank):
         # the bank and the job that applies the stored roots take one each, and streams beyond that share a queue in
         # the order of their launches -- a third stack on a stream of its own ran behind the second anyway, and held
         # up what the second had to do after its sweep.  The stacks are dealt out by cost, the cheap ones of a lane first.
-        lanes = [[] for _ in range(min(2, len(orders)))]
+        lanes = [[] for _ in range(min(LANES, len(orders)))]
         for o in orders:                                                   # (most expensive first)
             min(lanes, key=lambda lane: sum(x ** 3 * self.per_order[x] for x in lane)).append(o)
         lanes = [sorted(lane, key=lambda x: x ** 3 * self.per_order[x]) for lane in lanes]
