@@ -49,6 +49,7 @@ class ShampooBank2(ShampooBank):
         super().__init__(params, name2qmap, code, **kwargs)
 
     LOOK_AGAIN = 8                                # updates after which a stack of low numerical rank tries the plain sweep again
+    STALL_SECONDS = 300.0                         # the host polls the device while the stacks are factored: not for ever
 
     def _replace_first(self, order):
         """Whether this update of the stack starts with the replacing sweep: its last update with the plain sweep
@@ -195,12 +196,17 @@ class ShampooBank2(ShampooBank):
                         s.advance()
             return run
 
+        waiting_since = time.monotonic()
         try:
             while unfinished:
                 ready = [o for o in unfinished if tick[o].query()]
                 if not ready:
+                    if time.monotonic() - waiting_since > self.STALL_SECONDS:
+                        raise RuntimeError(f"the statistics update of the orders {unfinished} made no progress on the device "
+                                           f"for {self.STALL_SECONDS} s")
                     time.sleep(2e-5)
                     continue
+                waiting_since = time.monotonic()
                 for o in sorted(ready, key=lambda x: -x ** 3 * self.per_order[x]):
                     self._run_on(slot[o], look_at(o), after_current=False)
                     if solver[o].finished:
