@@ -180,18 +180,23 @@ def fused_step(opt, group, update, group_index=0):
                         opt.state[q]['preconditioner'].compute_preconditioners(v0=starts[id(q)])
 
                 roots_job = _SideJob(unbatched[0].device, entry['side_stream'], roots_of_unbatched)
-            try:
+        else:
+            roots_job = None
+        try:
+            if step % group['prec_compute_steps'] == 0:
                 bank.compute_preconditioners()
-            finally:
-                if roots_job is not None:
-                    roots_job.join()
-                    roots_done = True
-        if step >= group['start_prec_step'] and bank.is_active():
-            # the rescaling to each gradient's norm happens inside the fused update
-            if applied is None:
-                applied = bank.preconditioned_grads(bgrads)
-            directions = {id(p): o for p, o in zip(banked, applied)}
-            grafted = set(directions)
+            if step >= group['start_prec_step'] and bank.is_active():
+                # the rescaling to each gradient's norm happens inside the fused update
+                if applied is None:
+                    applied = bank.preconditioned_grads(bgrads)
+                directions = {id(p): o for p, o in zip(banked, applied)}
+                grafted = set(directions)
+        finally:
+            # (joined behind the bank's products with the new roots: the current stream waits for the small launches
+            # of the side job only where the parameters outside the bank need their roots)
+            if roots_job is not None:
+                roots_job.join()
+                roots_done = True
     for p in params:
         if id(p) not in entry['ids']:
             # into a buffer that stays where it is: the fused update keeps a device table of addresses
