@@ -427,6 +427,46 @@ def test_bank_against_unmodified_per_parameter_path(mods, code_maps, mode, monke
         assert float((got - want).norm()) <= 0.1 * max(float(want.norm()), top)
 
 
+def test_steps_issued_from_another_stream_give_the_same_parameters(mods, tmp_path, monkeypatch):
+    """The engines run on side streams of their own and join the stream that is current when step() is called:
+    steps issued from a stream of the application, next to other streams of the application that are busy, end in
+    the same bits as steps issued from the default stream."""
+    S2, _ = mods
+    import optimizers.matrix_functions as MF
+    monkeypatch.chdir(tmp_path)
+    real_rand = torch.rand
+    monkeypatch.setattr(MF.torch, "rand", lambda *size, **kw: torch.full(size, 0.75, **kw))
+    g = torch.Generator().manual_seed(12)
+    shapes = SHAPES + [(64,), (128, 100)]
+    init = [real_rand(s, generator=g) for s in shapes]
+    gs = [[0.02 * torch.randn(s, generator=g) for s in shapes] for _ in range(4)]
+
+    def run(stream):
+        params = [torch.nn.Parameter(t.clone().cuda()) for t in init]
+        opt = S2.ShampooAdamW(params, lr=1e-2, weight_decay=0.05, start_prec_step=2, stat_compute_steps=1, prec_compute_steps=2,
+                              fused=True, inv_root_mode=1, **KW)
+        grads = [[gr.cuda() for gr in step] for step in gs]
+        torch.cuda.synchronize()
+        busy = [torch.cuda.Stream() for _ in range(3)]
+        noise = torch.zeros(1 << 20, device="cuda")
+        with torch.cuda.stream(stream) if stream is not None else torch.cuda.stream(torch.cuda.current_stream()):
+            for step in grads:
+                for other in busy:                                   # the application keeps its own streams busy
+                    with torch.cuda.stream(other):
+                        noise.add_(1.0)
+                for p_, gr in zip(params, step):
+                    p_.grad = gr.clone()
+                opt.step()
+        torch.cuda.synchronize()
+        return [p_.detach().clone() for p_ in params]
+
+    plain = run(None)
+    other = run(torch.cuda.Stream())
+    assert all(bool(torch.isfinite(p_).all()) for p_ in plain)
+    for a, b in zip(plain, other):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("which,mode", [("adamw", 1), ("sgd", 0)])
 def test_fused_shampoo2_optimizer_runs_and_resumes_from_a_checkpoint(mods, which, mode, tmp_path, monkeypatch):
     import io
