@@ -111,10 +111,16 @@ __device__ __forceinline__ float4 gload4(const float *p) {
 }
 // A word or four at `base` (the same for the whole wave) plus a byte offset of 32 bits per lane: the form of the
 // load instruction that takes the base from scalar registers, so that moving the base costs no vector arithmetic.
-// (Buffer loads: the compiler turns a global load of base + offset into one 64-bit address per lane and load, advanced
-// by vector arithmetic from tile to tile.)
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t whole_range(const float *base) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(base), 0, -1, 0x00020000);
+}
+// A pointer that is the same in every lane, as a value the compiler knows to be: without that it wraps every buffer
+// load into a loop over the distinct values of its base.
+__device__ __forceinline__ const float *wave_uniform(const float *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return reinterpret_cast<const float *>(((uint64_t)hi << 32) | lo);
 }
 __device__ __forceinline__ float gload_at(const float *base, uint32_t byte_off) {
     return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(whole_range(base), (int)byte_off, 0, 0));
@@ -364,49 +370,33 @@ __device__ __forceinline__ void commit_split_four(unsigned char *operand, int ro
 // consecutive k (half t & 1) of row t >> 1; 64 rows: 4 consecutive k (quarter t & 3) of row t >> 2.  Rows beyond the
 // matrix are clamped (their products are never stored).  `vec`: rows are 16-byte aligned (the same for the whole
 // workgroup); otherwise word loads.
-// SCALAR_BASE (products of two dense operands): the loads take the tile's base from scalar registers and a byte offset
-// of 32 bits per lane that stays the same from tile to tile, so that moving on to the next tile costs no vector
-// arithmetic (with a pointer per lane the compiler advances one 64-bit address per load and tile).  Not for the
-// kernels that expand a quantized operand beside it: they were measured slower that way (207 -> 233 us).
-template <int ROWS, bool SCALAR_BASE>
+// The loads take the tile's base from scalar registers and a byte offset of 32 bits per lane that stays the same from
+// tile to tile (buffer loads), so that moving on to the next tile costs no vector arithmetic: with a pointer per lane the
+// compiler advances one 64-bit address per load and tile.
+template <int ROWS>
 struct SplitKContig {
     static_assert(ROWS == 128 || ROWS == 64, "tile rows");
     static constexpr int PER = ROWS * BK / 256;
     float v[PER];
-    long long first;                    // SCALAR_BASE: elements from the operand's origin to the tile's first row
-    uint32_t off;                       // from there (else: from the origin) to this lane's first word: bytes (else: elements)
+    long long first;                    // elements from the operand's origin to the tile's first row (the same for all lanes)
+    uint32_t off;                       // bytes from there to this lane's first word (the host keeps 128 rows inside 32 bits)
     bool vec = true;
     __device__ __forceinline__ void prepare(int ld, int row0, int rows) {
         const int row = ROWS == 128 ? threadIdx.x >> 1 : threadIdx.x >> 2, part = ROWS == 128 ? threadIdx.x & 1 : threadIdx.x & 3;
-        if constexpr (SCALAR_BASE) {
-            first = (long long)row0 * ld;
-            off = (uint32_t)((min(row0 + row, rows - 1) - row0) * ld + part * PER) * 4u;       // (the host keeps 128 rows inside 32 bits)
-        } else {
-            off = (uint32_t)(min(row0 + row, rows - 1) * ld + part * PER);
-        }
+        first = (long long)row0 * ld;
+        off = (uint32_t)((min(row0 + row, rows - 1) - row0) * ld + part * PER) * 4u;
     }
     __device__ __forceinline__ void fetch_fast(const float *tile_base) {
-        if constexpr (SCALAR_BASE) {
-            const float *base = tile_base + first;
-            if (vec) {
-#pragma unroll
-                for (int q = 0; q < PER / 4; ++q) {
-                    const float4 x = gload4_at(base, off + 16u * q);
-                    v[4 * q] = x.x; v[4 * q + 1] = x.y; v[4 * q + 2] = x.z; v[4 * q + 3] = x.w;
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < PER; ++j) v[j] = gload_at(base, off + 4u * j);
-            }
-        } else if (vec) {
+        const float *base = tile_base + first;
+        if (vec) {
 #pragma unroll
             for (int q = 0; q < PER / 4; ++q) {
-                const float4 x = gload4(tile_base + (int)off + 4 * q);
+                const float4 x = gload4_at(base, off + 16u * q);
                 v[4 * q] = x.x; v[4 * q + 1] = x.y; v[4 * q + 2] = x.z; v[4 * q + 3] = x.w;
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < PER; ++j) v[j] = gload(tile_base + (int)off + j);
+            for (int j = 0; j < PER; ++j) v[j] = gload_at(base, off + 4u * j);
         }
     }
     __device__ __forceinline__ void commit_split(unsigned char *operand) const {
@@ -417,34 +407,24 @@ struct SplitKContig {
 
 // Dense, row index contiguous in memory (element (row, k) at base[k * ld + row]); whole k tiles.  128 rows: thread t
 // takes row t & 127 and the 8 k of half t >> 7; 64 rows: row t & 63 and the 4 k of quarter t >> 6; one word per load,
-// a wave's load covers 64 consecutive words.
-template <int ROWS, bool SCALAR_BASE>
+// a wave's load covers 64 consecutive words.  Scalar base and per-lane byte offsets as above.
+template <int ROWS>
 struct SplitRowContig {
     static_assert(ROWS == 128 || ROWS == 64, "tile rows");
     static constexpr int PER = ROWS * BK / 256;
     float v[PER];
-    int first, ld_;                     // SCALAR_BASE: the tile's first row
-    uint32_t off[SCALAR_BASE ? PER : 1];    // SCALAR_BASE: bytes from there to each of this lane's words, kept from tile to tile
+    int first;                          // the tile's first row (the same for all lanes)
+    uint32_t off[PER];                  // bytes from there to each of this lane's words
     __device__ __forceinline__ void prepare(int ld, int row0, int rows) {
         const int row = threadIdx.x & (ROWS - 1), part = ROWS == 128 ? threadIdx.x >> 7 : threadIdx.x >> 6;
-        if constexpr (SCALAR_BASE) {
-            first = row0;
+        first = row0;
 #pragma unroll
-            for (int j = 0; j < PER; ++j) off[j] = (uint32_t)((part * PER + j) * ld + (min(row0 + row, rows - 1) - row0)) * 4u;
-        } else {
-            ld_ = ld;
-            off[0] = (uint32_t)(part * PER * ld + min(row0 + row, rows - 1));
-        }
+        for (int j = 0; j < PER; ++j) off[j] = (uint32_t)((part * PER + j) * ld + (min(row0 + row, rows - 1) - row0)) * 4u;
     }
     __device__ __forceinline__ void fetch_fast(const float *tile_base) {
-        if constexpr (SCALAR_BASE) {
-            const float *base = tile_base + first;
+        const float *base = tile_base + first;
 #pragma unroll
-            for (int j = 0; j < PER; ++j) v[j] = gload_at(base, off[j]);
-        } else {
-#pragma unroll
-            for (int j = 0; j < PER; ++j) v[j] = gload(tile_base + (int)off[0] + j * ld_);
-        }
+        for (int j = 0; j < PER; ++j) v[j] = gload_at(base, off[j]);
     }
     __device__ __forceinline__ void commit_split(unsigned char *operand) const {
         if constexpr (ROWS == 128) commit_split_eight<ROWS>(operand, threadIdx.x & 127, threadIdx.x >> 7, v);
@@ -663,7 +643,6 @@ __global__ __launch_bounds__(256, (kWavesPerSimd<BM, BN, KA, KB, PREC>)) void ge
     id /= slices;
     constexpr bool kSplit = PREC == kPipeSplit;
 
-    constexpr bool kBothDense = KA < kQuant4 && KB < kQuant4;
     using PlainA = typename std::conditional<KA == kDense, LoadKContig<BM>,
         typename std::conditional<KA == kDenseT, LoadRowContig<BM>,
             LoadQuant<BM, KA == kQuant4 ? 4 : 8, true>>::type>::type;
@@ -671,10 +650,10 @@ __global__ __launch_bounds__(256, (kWavesPerSimd<BM, BN, KA, KB, PREC>)) void ge
         typename std::conditional<KB == kDenseT, LoadKContig<BN>,
             LoadQuant<BN, KB == kQuant4 ? 4 : 8, false>>::type>::type;
     using LoaderA = typename std::conditional<!kSplit || KA >= kQuant4, PlainA,
-        typename std::conditional<KA == kDense, SplitKContig<BM, kBothDense>, SplitRowContig<BM, kBothDense>>::type>::type;
+        typename std::conditional<KA == kDense, SplitKContig<BM>, SplitRowContig<BM>>::type>::type;
     using LoaderB = typename std::conditional<!kSplit, PlainB,
         typename std::conditional<KB >= kQuant4, LoadQuant<BN, KB == kQuant4 ? 4 : 8, false, true>,
-            typename std::conditional<KB == kDense, SplitRowContig<BN, kBothDense>, SplitKContig<BN, kBothDense>>::type>::type>::type;
+            typename std::conditional<KB == kDense, SplitRowContig<BN>, SplitKContig<BN>>::type>::type>::type;
     // An operand whose k is contiguous at the source sits in LDS as [row][k] (16-byte commits, one
     // 16-byte fragment read per four MFMA steps); the others as [k][row] (16-byte commits, one word
     // per step).  Which k a lane feeds into which step is free as long as both operands agree:
@@ -737,6 +716,10 @@ __global__ __launch_bounds__(256, (kWavesPerSimd<BM, BN, KA, KB, PREC>)) void ge
 
     const float *A = (KA < kQuant4) ? dense_ptr(args.A, b, args.batch_inner, args.inner_a) : nullptr;
     const float *B = (KB < kQuant4) ? dense_ptr(args.B, b, args.batch_inner, args.inner_b) : nullptr;
+    if constexpr (kSplit) {                    // the same for the whole workgroup: say so, the loads take them from scalar registers
+        A = wave_uniform(A);
+        B = wave_uniform(B);
+    }
     const bool a_vec = KA < kQuant4 && (args.lda & 3) == 0 && is_aligned16(A);
     const bool b_vec = KB < kQuant4 && (args.ldb & 3) == 0 && is_aligned16(B);
 
