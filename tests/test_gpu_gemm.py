@@ -398,6 +398,36 @@ def test_random_shapes_strides_and_alignments_all_dense_layouts(mods):
         assert rel_err(got, want) <= TOL, (case, m, n, k, batch, ta, tb, pad_a, pad_b, shift_a, shift_b)
 
 
+@pytest.mark.parametrize("shift", [0, 1])
+def test_operands_inside_very_wide_arrays_are_read_where_they_are(mods, shift):
+    """Dense operands given as views into wide arrays.  The split pipe's loads take a tile's base from scalar registers
+    and a byte offset of 32 bits per lane: with a leading dimension just under 2^22 words the offsets of a tile's last
+    rows lie beyond 2^31 bytes and must still be taken as unsigned; from 2^22 words on the product goes to the fp32
+    pipe.  Results must be those of the same operands stored compactly (bit for bit on the same pipe).  shift 1: rows
+    that are not 16-byte aligned (word loads)."""
+    _, X = mods
+    g = torch.Generator(device="cuda").manual_seed(31 + shift)
+    a = torch.randn(128, 64, device="cuda", generator=g)
+    b = torch.randn(64, 128, device="cuda", generator=g)
+    want = a.double().cpu() @ b.double().cpu()
+    compact = X.gemm(a, b)
+    assert rel_err(compact, want) <= TOL
+    for ld, same_pipe in (((1 << 22) - 4, True), (1 << 22, False)):
+        wide_a = torch.zeros(128, ld, device="cuda")
+        wide_b = torch.zeros(64, ld, device="cuda")
+        A = wide_a[:, 1000 + shift:1064 + shift]
+        B = wide_b[:, 2000 + shift:2128 + shift]
+        A.copy_(a)
+        B.copy_(b)
+        got = X.gemm(A, B)                                   # A: k contiguous, B: row index contiguous
+        assert torch.equal(got, compact) if same_pipe else rel_err(got, want) <= TOL
+        for got_t, compact_t in ((X.gemm(B, b, trans_a=True), X.gemm(b, b, trans_a=True)),        # left operand with its row index contiguous
+                                 (X.gemm(a, A, trans_b=True), X.gemm(a, a, trans_b=True))):       # right operand with k contiguous
+            assert torch.equal(got_t, compact_t) if same_pipe else rel_err(got_t, compact_t.cpu()) <= TOL
+        del wide_a, wide_b, A, B
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("batch,m,n,k", [(64, 256, 384, 64), (40, 512, 512, 1024), (6, 1024, 1024, 2048), (50, 500, 392, 336),
                                          (3, 200, 72, 160), (1, 64, 64, 32)])
 @pytest.mark.parametrize("spread", [0.0, 3.0])
