@@ -91,8 +91,12 @@ void cdequantize_blockwise_diagreal_4bit_bf16_stream(unsigned char *A, float *co
 /* ---- stacks of equally sized matrices in one launch (no counterpart in the reference, which
  * loops over matrices in Python: optimizers/shampoo2.py:184-200, 249-269) --------------------
  * A is batch x order x order, contiguous; absmax, diag and out are the per-matrix buffers of
- * the single-matrix entry points laid end to end.  Needs blocksize to divide order, 16-byte
- * aligned A/out and batch*order*order < 2^31.  diag == NULL selects the plain form. */
+ * the single-matrix entry points laid end to end (order * ceil(order / blocksize) maxima, order
+ * diagonal entries, ceil(order * order * bits / 8) code bytes per matrix: the codes of an odd order are
+ * padded to a whole byte per matrix).  batch*order*order < 2^31.  With blocksize dividing order and
+ * 16-byte aligned A/out the whole stack is one stream of segments (the fast path); any other order goes
+ * through the general path, one matrix per grid row, at most 65535 matrices per launch.  diag == NULL
+ * selects the plain form. */
 void qtensor_hip_quantize_batched(const void *A, int a_is_bf16, const float *code, int bits, int order, int batch,
                                   float *absmax, float *diag, unsigned char *out, int blocksize, qtensor_stream_t stream);
 void qtensor_hip_dequantize_batched(const unsigned char *q, const float *code, int bits, int order, int batch,
@@ -189,6 +193,9 @@ typedef struct {
         int triangular;         /* bit 0: A is upper triangular (A[m][k] = 0 for k < m), bit 1: B is upper triangular
                                  * (B[k][n] = 0 for k > n), square in their k index: the zero part of the k range is
                                  * skipped (dense operands only, not with `symmetric`)                           */
+        int pipe;               /* which matrix pipe multiplies this product: 0 = the process-wide choice
+                                 * (qtensor_hip_gemm_pipe), 1 = the fp32 pipe, 2 = the split bf16 pipe (where its
+                                 * conditions hold, see qtensor_hip_gemm_pipe; the fp32 pipe otherwise)          */
     } args;
 } qtensor_gemm_desc;
 
@@ -205,10 +212,13 @@ void qtensor_hip_gemm(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
  * epilogue without the symmetric / triangular / two-level batch options (the only products that are ever cut);
  * anything else, and any product with 2 * batch * M * N > QTENSOR_STATIC_SCRATCH_FLOATS, is refused with an
  * error and nothing is launched.  Results are bit-identical to qtensor_hip_gemm with a caller workspace of
- * that size.  All calls on one GPU share the array: calls that overlap in time on one GPU (several streams or
- * threads) race; nothing in the array needs clearing between calls (every partial product is written in full
- * before it is read).  The first call on a GPU looks the array's address up (hipGetSymbolAddress): make it
- * before a graph capture begins. */
+ * that size.  All calls on one GPU share the array, so calls that overlap in time on one GPU would race: calls on
+ * one stream are ordered by the stream; a call on another stream than the last one is refused with an error
+ * (nothing launched) while the last call's work is still running on the GPU -- wait for it first.  A stream under
+ * graph capture is not checked (nothing runs at capture time): keeping replays of such graphs apart is the
+ * caller's business.  Nothing in the array needs clearing between calls (every partial product is written in
+ * full before it is read).  The first call on a GPU looks the array's address up (hipGetSymbolAddress) and makes
+ * the event that the check uses: make it before a graph capture begins. */
 #define QTENSOR_STATIC_SCRATCH_FLOATS (1 << 24)
 void qtensor_hip_gemm_static(const qtensor_gemm_desc *desc, qtensor_stream_t stream);
 
@@ -221,14 +231,21 @@ void qtensor_hip_gemm_static(const qtensor_gemm_desc *desc, qtensor_stream_t str
  *      in fp32 by v_mfma_f32_32x32x16_bf16.  What is left out is below 2^-24 |a b| per product, so a dot product
  *      carries the error of fp32 arithmetic (tests/test_gpu_gemm.py measures both pipes against float64), while the
  *      bf16 pipe does sixteen multiply-adds per cycle for every one of the fp32 pipe.  Differences: an infinite
- *      operand element gives NaN where the fp32 pipe gives infinity; elements below 2^-110 lose their low pieces.
+ *      operand element gives NaN where the fp32 pipe gives infinity, and so does a finite one of magnitude
+ *      >= 0x7f7f8000 as bits (about 3.3962e38, the top 2^-9 of the fp32 range), whose leading piece rounds to the
+ *      bf16 infinity; elements below 2^-110 lose their low pieces.
  *      Taken for K a multiple of 16 and at least 32 (dense operands within 31-bit offsets; quantized operands are
  *      expanded to fp32 and split the same way), under every tile shape, so that the bits of a product do not
  *      depend on how it is tiled; every other product runs on the fp32 pipe whatever the mode.  In a symmetric
  *      product every element below the diagonal takes the value of its partner above (a b and b a add their
  *      pieces in different orders): the result is exactly symmetric.
  * mode < 0 only queries.  Returns the mode in force before the call.  The initial mode is 1 unless the environment
- * variable QT_GEMM_PIPE is "f32". */
+ * variable QT_GEMM_PIPE is "f32".  Every product that leaves args.pipe at 0 reads the mode when it is launched,
+ * including the products inside the Cholesky / Gram-Schmidt entry points below: change it only while no other
+ * host thread is launching products (before an optimizer's first step, say), or choose per product with args.pipe.
+ * (QT_GEMM_PIPE is the only environment variable a release build reads; builds made with -DQT_TUNING_KNOBS also
+ * read QT_GEMM_TILE, QT_GEMM_SPLIT, QT_GEMM_STREAM_WGS, QT_GEMM_STREAM_MIN, QT_BGS_PANEL and QT_SOLVE_PANEL, which
+ * force tile shapes, k cuts and panel widths for experiments and thereby change summation orders.) */
 int qtensor_hip_gemm_pipe(int mode);
 
 /* Yardstick for the product kernels (no counterpart in the reference): one launch in which every wave of
@@ -329,6 +346,12 @@ int qtensor_hip_tail_chunk(void);
 void qtensor_hip_adamw_tail(const qtensor_tail_tensor *table, const int *chunk_tensor, int n_chunks, float *partial, int graft,
                             double lr, double beta1, double beta2, double eps, double weight_decay, long long step,
                             qtensor_stream_t stream);
+/* qtensor_hip_adamw_tail for parameters whose step counts differ (the reference counts steps per parameter,
+ * optimizers/shampoo2.py:335-342, and skips a parameter without a gradient, :415): row_corrections (device,
+ * 2 floats per table row) holds {sqrt(1 - beta2^t), -lr / (1 - beta1^t)} for that row's own step count t. */
+void qtensor_hip_adamw_tail_rows(const qtensor_tail_tensor *table, const int *chunk_tensor, int n_chunks, float *partial,
+                                 int graft, double lr, double beta1, double beta2, double eps, double weight_decay,
+                                 const float *row_corrections, qtensor_stream_t stream);
 void qtensor_hip_sgd_tail(const qtensor_tail_tensor *table, const int *chunk_tensor, int n_chunks, float *partial, int graft,
                           double lr, double momentum, double weight_decay, int nesterov, qtensor_stream_t stream);
 

@@ -507,9 +507,14 @@ struct Sweep {
 }  // namespace qt
 
 extern "C" int qtensor_hip_block_gram_schmidt_width(void) {
-    // QT_BGS_PANEL (a tuning knob): another width of the outer panels, a multiple of 64
+    // QT_BGS_PANEL (a tuning knob, only in builds made with -DQT_TUNING_KNOBS): another width of the outer panels,
+    // a multiple of 64
     static const int width = [] {
+#ifdef QT_TUNING_KNOBS
         const char *env = getenv("QT_BGS_PANEL");
+#else
+        const char *env = nullptr;
+#endif
         const int asked = env != nullptr ? atoi(env) : 0;
         return asked >= qt::NB && asked % qt::NB == 0 && asked <= 1024 ? asked : 128;
     }();
@@ -574,9 +579,14 @@ extern "C" void qtensor_hip_solve_upper_right_batched(const float *q, const floa
     if (rows < 1) { set_error(kBadArgument, "solve_upper_right_batched: rows must be positive"); return; }
     hipStream_t stream = (hipStream_t)stream_v;
     const long long mat = (long long)n * n, tall = (long long)rows * n;
-    // QT_SOLVE_PANEL (a tuning knob): another panel width, 64 times a power of two
+    // QT_SOLVE_PANEL (a tuning knob, only in builds made with -DQT_TUNING_KNOBS): another panel width, 64 times a
+    // power of two
     static const int top = [] {
+#ifdef QT_TUNING_KNOBS
         const char *env = getenv("QT_SOLVE_PANEL");
+#else
+        const char *env = nullptr;
+#endif
         const int asked = env != nullptr ? atoi(env) : 0;
         const bool usable = asked >= NB && asked % NB == 0 && ((asked / NB) & (asked / NB - 1)) == 0;
         return usable ? asked : kSolvePanel;

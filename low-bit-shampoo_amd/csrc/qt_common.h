@@ -9,6 +9,7 @@ namespace qt {
 // ---- host side: per-thread error slot and launch helpers --------------------------
 void clear_error();
 void set_error(int code, const char *fmt, ...);
+int error_code();          // this host thread's slot (0: the last call went through)
 // Records a failed launch (hipGetLastError) under `what`; returns true when all is well.
 bool launch_ok(const char *what);
 // Compute units of the current device (cached per device ordinal).

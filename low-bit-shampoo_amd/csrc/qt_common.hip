@@ -18,6 +18,8 @@ void clear_error() {
     t_error_text[0] = '\0';
 }
 
+int error_code() { return t_error_code; }
+
 void set_error(int code, const char *fmt, ...) {
     t_error_code = code;
     va_list ap;

@@ -157,6 +157,11 @@ __global__ __launch_bounds__(kThreads) void dequantize_general_kernel(
     for (int i = threadIdx.x; i < NCODE; i += kThreads) s_code[i] = code[i];
     __syncthreads();
     const uint32_t n_bytes = (total + EPB - 1) / EPB;
+    // blockIdx.y = matrix of a stack (its own run of code bytes, maxima and diagonal entries)
+    q += (size_t)blockIdx.y * n_bytes;
+    absmax += (size_t)blockIdx.y * order * nb;
+    if (DIAG) diag += (size_t)blockIdx.y * order;
+    out += (size_t)blockIdx.y * total;
     for (uint32_t j = blockIdx.x * kThreads + threadIdx.x; j < n_bytes; j += gridDim.x * kThreads) {
         const uint32_t byte = q[j];
 #pragma unroll
@@ -206,8 +211,9 @@ void dequantize_dispatch(const uint8_t *q, const float *code, int order_i, const
     const uint32_t order = (uint32_t)order_i, bs = (uint32_t)blocksize;
     const uint32_t total = order * order * (uint32_t)batch;
     const bool flat = order % bs == 0 && is_aligned(out, 4 * sizeof(T)) && is_aligned(q, 16) && is_aligned(absmax, 4);
-    if (batch > 1 && !flat) {
-        set_error(kBadArgument, "dequantize_blockwise: a stack of matrices needs blocksize to divide the order and aligned buffers");
+    if (batch > 65535 && !flat) {
+        set_error(kBadArgument, "dequantize_blockwise: a stack whose order the blocksize does not divide (or with unaligned buffers) "
+                                "takes at most 65535 matrices per launch");
         return;
     }
     if (flat) {
@@ -225,9 +231,10 @@ void dequantize_dispatch(const uint8_t *q, const float *code, int order_i, const
         }
     } else {
         const uint32_t nb = (order + bs - 1) / bs;
-        const uint32_t n_bytes = (total * BITS + 7) / 8;
-        hipLaunchKernelGGL((dequantize_general_kernel<T, BITS, DIAG>), dim3(capped_grid((n_bytes + kThreads - 1) / kThreads, 16)),
-                           dim3(kThreads), 0, stream, q, code, order, bs, nb, total, absmax, diag, out);
+        const uint32_t one = order * order;
+        const uint32_t n_bytes = (one * BITS + 7) / 8;
+        hipLaunchKernelGGL((dequantize_general_kernel<T, BITS, DIAG>), dim3(capped_grid((n_bytes + kThreads - 1) / kThreads, 16), batch),
+                           dim3(kThreads), 0, stream, q, code, order, bs, nb, one, absmax, diag, out);
     }
     launch_ok("dequantize_blockwise");
 }

@@ -35,6 +35,14 @@
 #ifndef QT_STREAMK
 #define QT_STREAMK 1
 #endif
+// Tuning knobs of the tile / k-cut choice (environment variables QT_GEMM_TILE, QT_GEMM_SPLIT, QT_GEMM_STREAM_WGS,
+// QT_GEMM_STREAM_MIN) exist only in builds made with -DQT_TUNING_KNOBS: they change the summation order of a
+// product, which a release build promises not to depend on anything but the operands' shapes.
+#ifdef QT_TUNING_KNOBS
+#define QT_KNOB(name) getenv(name)
+#else
+#define QT_KNOB(name) (static_cast<const char *>(nullptr))
+#endif
 
 namespace qt {
 
@@ -83,6 +91,7 @@ struct GemmArgs {
     long long inner_a, inner_b, inner_c, inner_e;   // base + (b / batch_inner) * stride + (b % batch_inner) * inner_x
     int triangular;               // bit 0: A is upper triangular (A[m][k] = 0 for k < m): k starts at the tile's first row;
                                   // bit 1: B is upper triangular (B[k][n] = 0 for k > n): k ends with the tile's last column
+    int pipe;                     // 0: the process-wide choice (qtensor_hip_gemm_pipe); 1: the fp32 pipe; 2: the split bf16 pipe
 };
 
 namespace {
@@ -1370,27 +1379,43 @@ struct qtensor_gemm_desc {
 static __device__ __align__(256) float scratch[QTENSOR_STATIC_SCRATCH_FLOATS];
 
 namespace {
-// Device address of `scratch` on the current device, looked up once per device.
-float *static_scratch() {
-    constexpr int kMaxDevices = 64;
-    static std::mutex guard;
-    static float *address[kMaxDevices] = {};
+// Per GPU: the device address of `scratch` (looked up once, with that device current) and who used it last.
+// All calls on a GPU share the one array, so a call on another stream than the last one is only let through when
+// that last call's work has finished on the device (an event recorded behind it says so); calls on one stream are
+// ordered by the stream.
+struct StaticScratch {
+    float *address = nullptr;
+    hipEvent_t last_done = nullptr;       // recorded behind the last call's launches
+    hipStream_t last_stream = nullptr;
+    bool pending = false;                 // last_done has been recorded and not yet been seen complete
+};
+constexpr int kMaxDevices = 64;
+std::mutex static_guard;
+StaticScratch static_slots[kMaxDevices];
+
+// The current device's slot, set up on first use (nullptr and the error slot on failure).  Caller holds static_guard.
+StaticScratch *static_scratch() {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         qt::set_error(qt::kBadArgument, "gemm_static: no current device");
         return nullptr;
     }
-    std::lock_guard<std::mutex> lock(guard);
-    if (address[dev] == nullptr) {
+    StaticScratch &slot = static_slots[dev];
+    if (slot.address == nullptr) {
         void *p = nullptr;
-        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess || p == nullptr) {
             qt::set_error(qt::kLaunchFailed, "gemm_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
             return nullptr;
         }
-        address[dev] = static_cast<float *>(p);
+        e = hipEventCreateWithFlags(&slot.last_done, hipEventDisableTiming);
+        if (e != hipSuccess) {
+            qt::set_error(qt::kLaunchFailed, "gemm_static: hipEventCreateWithFlags failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        slot.address = static_cast<float *>(p);
     }
-    return address[dev];
+    return &slot;
 }
 
 void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream);
@@ -1455,12 +1480,31 @@ extern "C" void qtensor_hip_gemm_static(const qtensor_gemm_desc *d, void *stream
                   need, QTENSOR_STATIC_SCRATCH_FLOATS);
         return;
     }
-    float *ptr = static_scratch();
-    if (ptr == nullptr) return;
+    hipStream_t stream = (hipStream_t)stream_v;
+    std::lock_guard<std::mutex> lock(static_guard);
+    StaticScratch *slot = static_scratch();
+    if (slot == nullptr) return;
+    // A stream under graph capture launches nothing now: there is nothing to order against, and an event recorded
+    // into a capture cannot be queried.  Such calls are the caller's to keep apart.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(stream, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone;
+    if (!capturing && slot->pending && slot->last_stream != stream) {
+        const hipError_t state = hipEventQuery(slot->last_done);
+        if (state == hipErrorNotReady) {
+            set_error(kBadArgument, "gemm_static: the static scratch of this GPU is still in use by a call on another stream; "
+                                    "calls on different streams must not overlap (wait for the earlier one, or use one stream)");
+            return;
+        }
+        if (state != hipSuccess) { set_error(kLaunchFailed, "gemm_static: hipEventQuery: %s", hipGetErrorString(state)); return; }
+        slot->pending = false;
+    }
     qtensor_gemm_desc with_scratch = *d;
-    with_scratch.args.workspace = ptr;
+    with_scratch.args.workspace = slot->address;
     with_scratch.args.workspace_floats = QTENSOR_STATIC_SCRATCH_FLOATS;
-    gemm_dispatch(&with_scratch, (hipStream_t)stream_v);
+    gemm_dispatch(&with_scratch, stream);
+    if (!capturing && error_code() == 0) {
+        if (hipEventRecord(slot->last_done, stream) == hipSuccess) { slot->pending = true; slot->last_stream = stream; }
+    }
 }
 
 namespace {
@@ -1518,14 +1562,15 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
 
     // Tile shape: the one with the smallest estimated makespan.  Workgroups that share a compute unit
     // share its matrix pipes, so the time is (most tiles on one unit) x (tile area) / (efficiency of
-    // that shape: smaller tiles read more LDS words per multiply).  Quantized operands keep a
-    // 128-wide tile on their side unless QT_GEMM_TILE=MxN (a tuning knob) says otherwise.
+    // that shape: smaller tiles read more LDS words per multiply).
     struct Shape { int bm, bn; double eff; };
     static const Shape shapes[4] = {{128, 128, 1.0}, {128, 64, 0.92}, {64, 128, 0.92}, {64, 64, 0.82}};
     // The split pipe: for whole k tiles, where the offsets of the dense operands' loads fit 31 bits -- whatever the tile
     // shape, so that the bits of a product do not depend on how it is tiled.
     bool split_pipe = false;
-    if (gemm_pipe_mode() == kPipeSplit && d->K % BK == 0 && d->K >= 2 * BK) {
+    if (a.pipe < 0 || a.pipe > 2) { set_error(kBadArgument, "gemm: pipe must be 0 (process default), 1 (fp32) or 2 (split bf16), got %d", a.pipe); return; }
+    const int pipe_mode = a.pipe == 0 ? gemm_pipe_mode() : a.pipe == 1 ? kPipeF32 : kPipeSplit;
+    if (pipe_mode == kPipeSplit && d->K % BK == 0 && d->K >= 2 * BK) {
         const long long reach_a = ka >= kQuant4 ? 0 : ka == kDense ? (long long)d->M * a.lda : (long long)BK * a.lda + d->M;
         const long long reach_b = kb >= kQuant4 ? 0 : kb == kDenseT ? (long long)d->N * a.ldb : (long long)BK * a.ldb + d->N;
         // (and a tile's rows, 128 at most, inside 32 bits of bytes from its first one)
@@ -1533,7 +1578,7 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         split_pipe = reach_a < 0x7fffffffLL && reach_b < 0x7fffffffLL && near_a && near_b;
     }
     int pick = 0;
-    static const char *forced = getenv("QT_GEMM_TILE");
+    static const char *forced = QT_KNOB("QT_GEMM_TILE");
     if (forced != nullptr) {
         int fm = 0, fn = 0;
         if (sscanf(forced, "%dx%d", &fm, &fn) == 2)
@@ -1582,7 +1627,7 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         const double whole = cost_of(1);
         double best = whole;
         int best_split = 1;
-        static const char *forced_split = getenv("QT_GEMM_SPLIT");
+        static const char *forced_split = QT_KNOB("QT_GEMM_SPLIT");
         for (int sp = 2; sp <= 8; ++sp) {
             if (k_tiles % sp != 0 || k_tiles / sp < 8) continue;
             if ((long long)sp * d->batch * d->M * d->N > a.workspace_floats) continue;
@@ -1596,14 +1641,14 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         // the arithmetic whatever the number of output tiles, so the big, efficient tile shape can be kept
         // where it alone would leave half of the units idle (144 tiles of 128 x 128 on 256 units for a
         // 768 x 3072 result).  Taken when the output tiles of that shape would not fill the units twice over.
-        static const int stream_wgs = getenv("QT_GEMM_STREAM_WGS") != nullptr ? atoi(getenv("QT_GEMM_STREAM_WGS")) : 2;
+        static const int stream_wgs = QT_KNOB("QT_GEMM_STREAM_WGS") != nullptr ? atoi(QT_KNOB("QT_GEMM_STREAM_WGS")) : 2;
         const int big = d->M >= 96 && d->N >= 96 ? 0 : pick;
         const Shape &bs = shapes[big];
         const long long btm = (d->M + bs.bm - 1) / bs.bm, btn = (d->N + bs.bn - 1) / bs.bn;
         const long long big_tiles = btm * btn * d->batch, runs = big_tiles * k_tiles;
         if (stream_wgs > 0 && (ka >= kQuant4 || kb >= kQuant4) && a.skip == nullptr && k_tiles >= 16 && big_tiles < 2 * (long long)units) {
             long long groups = (long long)units * stream_wgs;
-            static const int min_run = getenv("QT_GEMM_STREAM_MIN") != nullptr ? atoi(getenv("QT_GEMM_STREAM_MIN")) : 24;
+            static const int min_run = QT_KNOB("QT_GEMM_STREAM_MIN") != nullptr ? atoi(QT_KNOB("QT_GEMM_STREAM_MIN")) : 24;
             if (groups > runs / min_run) {                                // at least that many k tiles per workgroup,
                 groups = runs / min_run;                                  // and no unit with one workgroup more than another
                 if (groups > (long long)units) groups -= groups % (long long)units;

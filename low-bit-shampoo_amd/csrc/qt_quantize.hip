@@ -213,11 +213,16 @@ __global__ __launch_bounds__(kFlatThreads) void quantize_flat_kernel(
 }
 
 // ---- general path ----------------------------------------------------------------------
+// (blockIdx.y = matrix of a stack: every matrix has its own run of maxima, diagonal entries and code bytes, the
+// codes of an odd order padded to a whole byte per matrix as the single-matrix format has them)
 // One wave per segment; writes absmax (and diag).
 template <typename T, bool DIAG>
 __global__ __launch_bounds__(kThreads) void segment_max_kernel(
     const T *__restrict__ A, uint32_t order, uint32_t bs, uint32_t nb, uint32_t n_segments,
     float *__restrict__ absmax, float *__restrict__ diag) {
+    A += (size_t)blockIdx.y * order * order;
+    absmax += (size_t)blockIdx.y * n_segments;
+    if (DIAG) diag += (size_t)blockIdx.y * order;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
     const uint32_t n_waves = gridDim.x * (kThreads / 64);
@@ -247,6 +252,9 @@ __global__ __launch_bounds__(kThreads) void encode_kernel(
     __shared__ CodeTables<NCODE> tab;
     build_code_tables<NCODE>(code, tab, nullptr);
     const uint32_t n_bytes = (total + EPB - 1) / EPB;
+    A += (size_t)blockIdx.y * total;
+    absmax += (size_t)blockIdx.y * order * nb;
+    out += (size_t)blockIdx.y * n_bytes;
     for (uint32_t j = blockIdx.x * kThreads + threadIdx.x; j < n_bytes; j += gridDim.x * kThreads) {
         uint32_t byte = 0;
 #pragma unroll
@@ -367,15 +375,16 @@ void launch_flat(const T *A, const float *code, uint32_t order, uint32_t batch, 
 }
 
 template <typename T, int BITS, bool DIAG>
-void launch_general(const T *A, const float *code, uint32_t order, uint32_t bs, float *absmax, float *diag, uint8_t *out, hipStream_t stream) {
+void launch_general(const T *A, const float *code, uint32_t order, uint32_t bs, uint32_t batch, float *absmax, float *diag, uint8_t *out,
+                    hipStream_t stream) {
     const uint32_t nb = (order + bs - 1) / bs;
     const uint32_t n_segments = order * nb;
     const uint32_t total = order * order;
-    hipLaunchKernelGGL((segment_max_kernel<T, DIAG>), dim3(grid_for((n_segments + 3) / 4, 8)), dim3(kThreads), 0, stream,
+    hipLaunchKernelGGL((segment_max_kernel<T, DIAG>), dim3(grid_for((n_segments + 3) / 4, 8), batch), dim3(kThreads), 0, stream,
                        A, order, bs, nb, n_segments, absmax, diag);
     if (!launch_ok("segment_max_kernel")) return;
     const uint32_t n_bytes = (total * BITS + 7) / 8;
-    hipLaunchKernelGGL((encode_kernel<T, BITS, DIAG>), dim3(grid_for((n_bytes + kThreads - 1) / kThreads, 8)), dim3(kThreads), 0, stream,
+    hipLaunchKernelGGL((encode_kernel<T, BITS, DIAG>), dim3(grid_for((n_bytes + kThreads - 1) / kThreads, 8), batch), dim3(kThreads), 0, stream,
                        A, code, order, bs, nb, total, absmax, out);
 }
 
@@ -398,8 +407,9 @@ void quantize_dispatch(const T *A, const float *code, int order_i, float *absmax
     }
     const uint32_t order = (uint32_t)order_i, bs = (uint32_t)blocksize;
     const bool flat = order % bs == 0 && is_aligned(A, 4 * sizeof(T)) && is_aligned(out, 16) && is_aligned(absmax, 4);
-    if (batch > 1 && !flat) {
-        set_error(kBadArgument, "quantize_blockwise: a stack of matrices needs blocksize to divide the order and aligned buffers");
+    if (batch > 65535 && !flat) {
+        set_error(kBadArgument, "quantize_blockwise: a stack whose order the blocksize does not divide (or with unaligned buffers) "
+                                "takes at most 65535 matrices per launch");
         return;
     }
     if (flat) {
@@ -412,7 +422,7 @@ void quantize_dispatch(const T *A, const float *code, int order_i, float *absmax
             default: launch_flat<T, BITS, 2048, DIAG>(A, code, order, (uint32_t)batch, absmax, diag, out, stream); break;
         }
     } else {
-        launch_general<T, BITS, DIAG>(A, code, order, bs, absmax, diag, out, stream);
+        launch_general<T, BITS, DIAG>(A, code, order, bs, (uint32_t)batch, absmax, diag, out, stream);
     }
     launch_ok("quantize_blockwise");
 }

@@ -102,6 +102,10 @@ __device__ __forceinline__ float graft_scale(const TailTensor &t, const float *p
 
 struct AdamW {
     float decay, beta1, alpha1, beta2, alpha2, sqrt_c2, eps, neg_step;
+    const float *row_corrections;      // optional: {sqrt(1 - beta2^t), -lr / (1 - beta1^t)} per table row (its own step count t)
+    __device__ __forceinline__ void bind(int row) {
+        if (row_corrections != nullptr) { sqrt_c2 = g1(row_corrections + 2 * row); neg_step = g1(row_corrections + 2 * row + 1); }
+    }
     __device__ __forceinline__ void operator()(float &p, float &m, float &v, float d) const {
         p = p * decay;
         m = m * beta1 + alpha1 * d;
@@ -114,6 +118,7 @@ struct AdamW {
 struct Sgd {
     float momentum, weight_decay, neg_lr;
     int nesterov;
+    __device__ __forceinline__ void bind(int) {}
     __device__ __forceinline__ void operator()(float &p, float &m, float &v, float d) const {
         (void)v;
         if (weight_decay != 0.0f) d = d + weight_decay * p;
@@ -125,10 +130,12 @@ struct Sgd {
 
 template <typename RULE, bool HAS_V>
 __global__ __launch_bounds__(kThreads) void tail_update_kernel(const TailTensor *table, const int *chunk_tensor,
-                                                               const float *partial, const RULE rule) {
+                                                               const float *partial, const RULE launch_rule) {
     __shared__ float s_scale;
     const int c = blockIdx.x;
     const TailTensor t = table[chunk_tensor[c]];
+    RULE rule = launch_rule;
+    rule.bind(chunk_tensor[c]);
     const float scale = graft_scale(t, partial, &s_scale);
     const bool graft = (t.flags & 1) != 0;
     const long long start = ((long long)c - t.first_chunk) * kChunk;
@@ -181,13 +188,13 @@ bool tail_args_ok(const void *table, const void *chunk_tensor, int n_chunks, con
 
 extern "C" int qtensor_hip_tail_chunk(void) { return qt::kChunk; }
 
-extern "C" void qtensor_hip_adamw_tail(const void *table, const int *chunk_tensor, int n_chunks, float *partial, int graft,
-                                       double lr, double beta1, double beta2, double eps, double weight_decay,
-                                       long long step, void *stream) {
-    using namespace qt;
+namespace qt {
+namespace {
+void adamw_tail(const void *table, const int *chunk_tensor, int n_chunks, float *partial, int graft, double lr, double beta1,
+                double beta2, double eps, double weight_decay, long long step, const float *row_corrections, void *stream) {
     clear_error();
     if (!tail_args_ok(table, chunk_tensor, n_chunks, partial, graft, "adamw_tail")) return;
-    if (step < 1) { set_error(kBadArgument, "adamw_tail: step counts from 1"); return; }
+    if (row_corrections == nullptr && step < 1) { set_error(kBadArgument, "adamw_tail: step counts from 1"); return; }
     if (n_chunks == 0) return;
     const TailTensor *tab = static_cast<const TailTensor *>(table);
     if (graft) {
@@ -200,12 +207,32 @@ extern "C" void qtensor_hip_adamw_tail(const void *table, const int *chunk_tenso
     rule.alpha1 = (float)(1.0 - beta1);
     rule.beta2 = (float)beta2;
     rule.alpha2 = (float)(1.0 - beta2);
-    rule.sqrt_c2 = (float)sqrt(1.0 - pow(beta2, (double)step));
+    rule.sqrt_c2 = row_corrections != nullptr ? 1.0f : (float)sqrt(1.0 - pow(beta2, (double)step));
     rule.eps = (float)eps;
-    rule.neg_step = (float)(-lr / (1.0 - pow(beta1, (double)step)));
+    rule.neg_step = row_corrections != nullptr ? 0.0f : (float)(-lr / (1.0 - pow(beta1, (double)step)));
+    rule.row_corrections = row_corrections;
     hipLaunchKernelGGL((tail_update_kernel<AdamW, true>), dim3(n_chunks), dim3(kThreads), 0, (hipStream_t)stream, tab,
                        chunk_tensor, partial, rule);
     launch_ok("adamw_tail");
+}
+}  // namespace
+}  // namespace qt
+
+extern "C" void qtensor_hip_adamw_tail(const void *table, const int *chunk_tensor, int n_chunks, float *partial, int graft,
+                                       double lr, double beta1, double beta2, double eps, double weight_decay,
+                                       long long step, void *stream) {
+    qt::adamw_tail(table, chunk_tensor, n_chunks, partial, graft, lr, beta1, beta2, eps, weight_decay, step, nullptr, stream);
+}
+
+extern "C" void qtensor_hip_adamw_tail_rows(const void *table, const int *chunk_tensor, int n_chunks, float *partial, int graft,
+                                            double lr, double beta1, double beta2, double eps, double weight_decay,
+                                            const float *row_corrections, void *stream) {
+    if (row_corrections == nullptr) {
+        qt::clear_error();
+        qt::set_error(qt::kNullPointer, "adamw_tail_rows: null row_corrections");
+        return;
+    }
+    qt::adamw_tail(table, chunk_tensor, n_chunks, partial, graft, lr, beta1, beta2, eps, weight_decay, 0, row_corrections, stream);
 }
 
 extern "C" void qtensor_hip_sgd_tail(const void *table, const int *chunk_tensor, int n_chunks, float *partial, int graft,

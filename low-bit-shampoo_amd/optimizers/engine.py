@@ -12,10 +12,16 @@ same arithmetic is done here with one launch per group of equally shaped blocks:
   P_L G P_R    two fused products per block shape, the quantized factors expanded on the fly
 
 The quantized state of all blocks of one order lives in one stacked allocation
-(codes [B, n*n/2], maxima [B, n*n/bs], diagonals [B, n]); entry b is bit-for-bit what
-quantize_blockwise_diagreal writes for that matrix.  Parameters with a block the fused kernels
-cannot take (an order that the blocksize does not divide, or too small to quantize) keep a
-per-parameter `Preconditioner`.
+(codes [B, n*n/2], maxima [B, n*ceil(n/bs)], diagonals [B, n]); entry b is bit-for-bit what
+quantize_blockwise_diagreal writes for that matrix.  An order that the blocksize does not divide
+(the 100 of a 768 x 100 head) is stored in the same format but cannot be read by the products
+directly: its stack is dequantized, updated by dense products and quantized again.  An order
+with fewer than min_lowbit_size elements, and every order with prec_bits = 32, is a plain fp32
+stack, as the reference's holders keep such matrices (qtensor/utils.py:11-17).
+
+Every operation takes an optional set of parameters to work on (`only`): the reference counts
+steps per parameter and skips a parameter without a gradient (optimizers/shampoo1.py:371-377),
+so the parameters of a bank may be due for different things at one call.
 """
 import threading
 from collections import defaultdict
@@ -62,6 +68,19 @@ def _same_queue(a, b, scratch):
         torch.cuda.synchronize(scratch.device)
         waited = waited and start.elapsed_time(end_b) > 0.5 * start.elapsed_time(end_a)
     return waited
+
+
+PROBE_QUEUES = False                                 # True: _build_pool sorts the streams by hardware queue (see there)
+
+
+def _plain_pool(index):
+    """A dozen side streams of the device as they come."""
+    device = torch.device("cuda", index)
+    with torch.cuda.device(device):
+        made = [torch.cuda.Stream(device=device) for _ in range(12)]
+    pool = {i: made[i] for i in range(12)}
+    pool["spare"] = made
+    return pool
 
 
 def _build_pool(index):
@@ -139,7 +158,7 @@ def shared_stream(device, slot):
     device = torch.device(device)
     index = device.index if device.index is not None else torch.cuda.current_device()
     if index not in _SHARED_STREAMS:
-        _SHARED_STREAMS[index] = _build_pool(index)
+        _SHARED_STREAMS[index] = _build_pool(index) if PROBE_QUEUES else _plain_pool(index)
     pool = _SHARED_STREAMS[index]
     if slot not in pool:
         pool[slot] = pool["spare"][slot % len(pool["spare"])]
@@ -178,11 +197,14 @@ class ShampooBank:
     def __init__(self, params, name2qmap, code, stat_decay=0.95, matrix_eps=1e-6, prec_maxorder=1200,
                  prec_bits=4, min_lowbit_size=4096, quan_blocksize=64, streams=None):
         self.stat_decay, self.matrix_eps = stat_decay, matrix_eps
-        self.bits, self.blocksize = prec_bits, quan_blocksize
+        self.bits, self.blocksize, self.min_lowbit_size = prec_bits, quan_blocksize, min_lowbit_size
         self.params = list(params)
         self.device = self.params[0].device
-        self.code = name2qmap[code].to(self.device)
-        name2qmap[code] = self.code
+        if prec_bits in (4, 8):
+            self.code = name2qmap[code].to(self.device)
+            name2qmap[code] = self.code
+        else:
+            self.code = None
         self.shapes = []                              # matrix view (m, n) of every parameter
         groups = {}
         for pi, p in enumerate(self.params):
@@ -212,37 +234,40 @@ class ShampooBank:
         if too_many:
             raise ValueError(f"the batched engine takes at most 65535 blocks per order in one launch, got {too_many}; "
                              "use a larger prec_maxorder or the per-parameter path (fused=False)")
-        self.precs = {}
-        for order, count in per_order.items():
-            eye = torch.eye(order, device=self.device).expand(count, order, order)
-            self.precs[order] = X.quantize_stack(eye.contiguous(),
-                                                 X.empty_quantized(count, order, quan_blocksize, prec_bits, self.code, True))
+        self.precs = {order: self._new_store(order, count, 1.0, True) for order, count in per_order.items()}
         self._init_statistics()
-        for g in self.groups:       # fp32 landing area of P_L G, per group
-            g.half = torch.empty(len(g), g.bm, g.bn, device=self.device)
-        self.outputs = [torch.empty(m, n, device=self.device) for m, n in self.shapes]
-        for g in self.groups:
-            g.out_ptrs = torch.tensor([self.outputs[pi].data_ptr() + 4 * off for pi, off in zip(g.param_index, g.offset)],
-                                      dtype=torch.int64, device=self.device)
-        self._active = False
+        self.active = [False] * len(self.params)      # per parameter: its inverse roots have been computed at least once
+        self._rows_cache, self._skip_cache = {}, {}
         # Independent groups run on a few side streams so that the tail of one launch overlaps the
         # head of the next; biggest first.
         self.groups.sort(key=lambda g: -len(g) * g.bm * g.bn * (g.bm + g.bn))
         streams = self.DEFAULT_STREAMS if streams is None else streams
         self.streams = [shared_stream(self.device, i) for i in range(min(streams, len(self.groups), 8))]
 
+    # ---- storage ---------------------------------------------------------------------------------
+    def lowbit(self, order):
+        """Whether the matrices of this order are stored quantized (the rule of the reference's holders)."""
+        return self.bits in (4, 8) and order * order >= self.min_lowbit_size
+
+    def _new_store(self, order, count, scale, diagreal):
+        """A stack of `count` matrices scale * I of this order in the bank's storage format."""
+        eye = torch.zeros(count, order, order, device=self.device)
+        eye.diagonal(dim1=1, dim2=2).fill_(scale)
+        if not self.lowbit(order):
+            return X.DenseStack(eye)
+        return X.quantize_stack(eye, X.empty_quantized(count, order, self.blocksize, self.bits, self.code, diagreal))
+
     def _init_statistics(self):
         """Statistics start as matrix_eps * I, stored quantized with an exact diagonal."""
-        self.stats = {}
-        for order, count in self.per_order.items():
-            eye = torch.eye(order, device=self.device).expand(count, order, order)
-            self.stats[order] = X.quantize_stack((self.matrix_eps * eye).contiguous(),
-                                                 X.empty_quantized(count, order, self.blocksize, self.bits, self.code, True))
+        self.stats = {order: self._new_store(order, count, self.matrix_eps, True) for order, count in self.per_order.items()}
 
     def _landing(self, g, side):
         """fp32 landing area of an updated statistic stack (only for blocksizes the requantizing product does not take)."""
         if getattr(g, "scratch", None) is None:
-            g.scratch = [torch.empty(len(g), o, o, device=self.device) for o in (g.bm, g.bn)]
+            g.scratch = [None, None]
+        if g.scratch[side] is None:
+            order = (g.bm, g.bn)[side]
+            g.scratch[side] = torch.empty(len(g), order, order, device=self.device)
         return g.scratch[side]
 
     def _fan_out(self, jobs, inline=False):
@@ -301,50 +326,96 @@ class ShampooBank:
 
     @classmethod
     def accepts(cls, p, prec_maxorder, prec_bits, min_lowbit_size, quan_blocksize):
-        """A parameter can live in the bank when it is an fp32 GPU matrix all of whose block orders are
-        quantized in the layout the fused kernels read (blocksize divides the order)."""
-        if not p.is_cuda or p.dtype != torch.float32 or prec_bits not in (4, 8):
+        """A parameter can live in the bank when it is an fp32 GPU tensor with a matrix view (two or more
+        dimensions that are not 1) and the bit width is one the bank stores (4, 8: quantized; 32: fp32)."""
+        if not p.is_cuda or p.dtype != torch.float32 or prec_bits not in (4, 8, 32):
             return False
-        shape = cls.matrix_shape(p)
-        if shape is None:
-            return False
-        orders = set(cls._pieces(shape[0], prec_maxorder) + cls._pieces(shape[1], prec_maxorder))
-        return all(o % quan_blocksize == 0 and o * o >= min_lowbit_size for o in orders)
+        return cls.matrix_shape(p) is not None
 
     # ---- per-step plumbing -----------------------------------------------------------------------
     def _segment(self, table, g, side):
         order, first = g.slot[side]
-        q = table[order]
-        n = len(g)
-        return X.Quantized(q.codes[first:first + n], q.absmax[first:first + n], q.diag[first:first + n], order,
-                           q.blocksize, q.bits, q.code)
+        return table[order].rows(first, len(g))
 
     def _grad_list(self, g, grads):
-        key = tuple(grads[pi].data_ptr() for pi in g.param_index)
+        # (a parameter that is left out of this call has no gradient: its own storage stands in, never read)
+        key = tuple((self.params[pi] if grads[pi] is None else grads[pi]).data_ptr() for pi in g.param_index)
         if key != g.grad_key:
             g.grad_ptrs = torch.tensor([base + 4 * off for base, off in zip(key, g.offset)], dtype=torch.int64,
                                        device=self.device)
             g.grad_key = key
         return X.PtrList(g.grad_ptrs, (len(g), g.bm, g.bn), ld=g.ld)
 
-    def _check(self, grads):
+    def _out_list(self, g):
+        if g.out_ptrs is None:
+            g.out_ptrs = torch.tensor([self.outputs[pi].data_ptr() + 4 * off for pi, off in zip(g.param_index, g.offset)],
+                                      dtype=torch.int64, device=self.device)
+        return X.PtrList(g.out_ptrs, (len(g), g.bm, g.bn), ld=g.ld)
+
+    def _check(self, grads, only=None):
         if len(grads) != len(self.params):
             raise ValueError("one gradient per parameter, in the order given at construction")
-        for grad, (m, n) in zip(grads, self.shapes):
+        for pi, (grad, (m, n)) in enumerate(zip(grads, self.shapes)):
+            if only is not None and pi not in only:
+                continue
+            if grad is None:
+                raise ValueError("a parameter that takes part in this call needs a gradient")
             if grad.numel() != m * n or not grad.is_contiguous() or grad.dtype != torch.float32 or not grad.is_cuda:
                 raise ValueError("gradients must be contiguous fp32 GPU tensors of the parameters' shapes")
 
-    def prepare(self, grads):
+    @staticmethod
+    def _only(only, count):
+        """None when every parameter takes part, else the frozenset of those that do."""
+        if only is None:
+            return None
+        only = frozenset(only)
+        return None if len(only) == count and all(0 <= i < count for i in only) else only
+
+    def _skip(self, g, only):
+        """int32 [len(g)] with 1 for the blocks of parameters that are left out (None: none is)."""
+        if only is None:
+            return None
+        key = (id(g), only)
+        if key not in self._skip_cache:
+            if len(self._skip_cache) > 64:
+                self._skip_cache.clear()
+            flags = [0 if pi in only else 1 for pi in g.param_index]
+            self._skip_cache[key] = torch.tensor(flags, dtype=torch.int32, device=self.device) if any(flags) else None
+        return self._skip_cache[key]
+
+    def _rows(self, order, only):
+        """int64 vector of the rows of this order's stacks that belong to the parameters in `only` (None: all rows)."""
+        if only is None:
+            return None
+        key = (order, only)
+        if key not in self._rows_cache:
+            if len(self._rows_cache) > 64:
+                self._rows_cache.clear()
+            rows = [first + i for g in self.groups for (o, first) in g.slot if o == order
+                    for i, pi in enumerate(g.param_index) if pi in only]
+            full = len(rows) == self.per_order[order]
+            self._rows_cache[key] = None if full else torch.tensor(sorted(rows), dtype=torch.int64, device=self.device)
+        return self._rows_cache[key]
+
+    def _touched(self, order, only):
+        """Whether any row of this order belongs to a parameter in `only`."""
+        rows = self._rows(order, only)
+        return rows is None or rows.numel() > 0
+
+    def prepare(self, grads, only=None):
         """Checks the gradients and writes the device tables of their block addresses, so that operations
         started afterwards from several threads only read them."""
-        self._check(grads)
+        only = self._only(only, len(self.params))
+        self._check(grads, only)
         for g in self.groups:
             self._grad_list(g, grads)
 
     # ---- the three operations of the reference's Preconditioner, for all parameters at once ------
     @torch.no_grad()
-    def add_statistics(self, grads):
-        self._check(grads)
+    def add_statistics(self, grads, only=None):
+        """only: the indices of the parameters whose statistics are updated (default: all)."""
+        only = self._only(only, len(self.params))
+        self._check(grads, only)
         w1 = self.stat_decay
         w2 = 1.0 if w1 == 1.0 else 1.0 - w1
 
@@ -352,56 +423,102 @@ class ShampooBank:
             def run():
                 G = self._grad_list(g, grads)
                 seg = self._segment(self.stats, g, side)
-                if self.blocksize == 64:
+                skip = self._skip(g, only)
+                kw = dict(trans_a=side == 1, trans_b=side == 0, alpha=w2, beta=w1, symmetric=True)
+                if seg.flat and self.blocksize == 64:
                     # dequantize, update and requantize in one launch: the fp32 statistic never reaches memory
-                    X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, symmetric=True,
-                           requantize=True)
+                    X.gemm(G, G, addend=seg, requantize=True, skip=skip, **kw)
                     return
-                out = self._landing(g, side)
-                X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, out=out,
-                       symmetric=True)
-                X.quantize_stack(out, seg)
+                if skip is None:
+                    if seg.flat:
+                        out = self._landing(g, side)
+                        X.gemm(G, G, addend=seg, out=out, **kw)
+                    else:                               # dense products on the dequantized (or fp32) stack
+                        out = X.load_stack(seg)
+                        X.gemm(G, G, addend=out, out=out, **kw)
+                    X.store_stack(out, seg)
+                    return
+                # some blocks are left out: the others are gathered, updated and put back
+                take = torch.nonzero(skip == 0).squeeze(1)
+                sub = seg.select(take)
+                dense = X.load_stack(sub)
+                X.gemm(X.PtrList(G.ptrs.index_select(0, take), (take.numel(), g.bm, g.bn), ld=g.ld),
+                       X.PtrList(G.ptrs.index_select(0, take), (take.numel(), g.bm, g.bn), ld=g.ld),
+                       addend=dense, out=dense, **kw)
+                seg.put(take, X.store_stack(dense, sub))
             return run
 
         for g in self.groups:           # address tables are written on the current stream, before the fan-out
             self._grad_list(g, grads)
-        self._fan_out([job(g, side) for g in self.groups for side in (0, 1)])
+        self._fan_out([job(g, side) for g in self.groups for side in (0, 1)
+                       if only is None or any(pi in only for pi in g.param_index)])
 
     @torch.no_grad()
-    def compute_preconditioners(self, v0=None):
-        """v0: optional dict order -> [count, order] start vectors of the power iteration."""
+    def compute_preconditioners(self, v0=None, only=None):
+        """v0: optional dict order -> [count, order] start vectors of the power iteration.
+        only: the indices of the parameters whose inverse roots are computed (default: all)."""
+        only = self._only(only, len(self.params))
+
         def job(order):
             def run():
-                dense = X.dequantize_stack(self.stats[order])
-                roots = ComputePowerBatched(dense, 4, ridge_epsilon=self.matrix_eps, v0=starts[order])
-                X.quantize_stack(roots.contiguous(), self.precs[order])
+                rows = self._rows(order, only)
+                stat = self.stats[order] if rows is None else self.stats[order].select(rows)
+                start = starts[order] if rows is None else starts[order].index_select(0, rows)
+                # (an fp32 statistic is handed over as it is and keeps the ridge that the iteration adds in
+                # place, as in the reference: optimizers/shampoo1.py:198)
+                dense = X.load_stack(stat)
+                roots = ComputePowerBatched(dense, 4, ridge_epsilon=self.matrix_eps, v0=start)
+                if rows is None:
+                    X.store_stack(roots, self.precs[order])
+                else:
+                    if isinstance(stat, X.DenseStack):
+                        self.stats[order].put(rows, stat)
+                    self.precs[order].put(rows, X.store_stack(roots, self.precs[order].select(rows)))
             return run
 
         # start vectors come from the global generator in a fixed order, whatever the streams do
         starts = {order: (torch.rand(stat.batch, order, device=self.device) * 2 - 1) if v0 is None else v0[order]
                   for order, stat in self.stats.items()}
-        self._fan_out([job(order) for order in sorted(self.stats, key=lambda o: -o ** 3 * self.stats[o].batch)])
-        self._active = True
+        orders = [o for o in sorted(self.stats, key=lambda o: -o ** 3 * self.stats[o].batch) if self._touched(o, only)]
+        self._fan_out([job(order) for order in orders])
+        for pi in range(len(self.params)):
+            if only is None or pi in only:
+                self.active[pi] = True
+
+    def _ensure_outputs(self):
+        if getattr(self, "outputs", None) is None:
+            self.outputs = [torch.empty(m, n, device=self.device) for m, n in self.shapes]
+            for g in self.groups:
+                g.out_ptrs = None
 
     @torch.no_grad()
-    def preconditioned_grads(self, grads, inline=False):
-        """List of P_L G P_R per parameter (buffers owned by the bank, overwritten by the next call).
-        inline: every launch on the current stream."""
-        self._check(grads)
+    def preconditioned_grads(self, grads, inline=False, only=None):
+        """List of P_L G P_R per parameter (buffers owned by the bank, overwritten by the next call; None for a
+        parameter that `only` leaves out).  inline: every launch on the current stream."""
+        only = self._only(only, len(self.params))
+        self._check(grads, only)
+        self._ensure_outputs()
 
         def job(g):
             def run():
-                X.gemm(self._segment(self.precs, g, 0), self._grad_list(g, grads), out=g.half)
-                X.gemm(g.half, self._segment(self.precs, g, 1), out=X.PtrList(g.out_ptrs, (len(g), g.bm, g.bn), ld=g.ld))
+                skip = self._skip(g, only)
+                left, right = self._segment(self.precs, g, 0), self._segment(self.precs, g, 1)
+                left = left if left.flat else X.load_stack(left)         # read inside the product, or dequantized first
+                right = right if right.flat else X.load_stack(right)
+                half = torch.empty(len(g), g.bm, g.bn, device=self.device)
+                X.gemm(left, self._grad_list(g, grads), out=half, skip=skip)
+                X.gemm(half, right, out=self._out_list(g), skip=skip)
             return run
 
         for g in self.groups:
             self._grad_list(g, grads)
-        self._fan_out([job(g) for g in self.groups], inline=inline)
-        return [out.view(p.shape) for out, p in zip(self.outputs, self.params)]
+            self._out_list(g)
+        self._fan_out([job(g) for g in self.groups if only is None or any(pi in only for pi in g.param_index)], inline=inline)
+        return [out.view(p.shape) if only is None or pi in only else None
+                for pi, (out, p) in enumerate(zip(self.outputs, self.params))]
 
     def is_active(self):
-        return self._active
+        return all(self.active)
 
     # ---- inspection (tests, checkpoints) ---------------------------------------------------------
     def block_table(self):
@@ -421,20 +538,31 @@ class ShampooBank:
                     rows.append((pi, j, side, order, first + i))
         return rows
 
+    @staticmethod
+    def _store_tensors(prefix, store, out):
+        if isinstance(store, X.DenseStack):
+            out[prefix + ".dense"] = store.data
+            return
+        out[prefix + ".codes"], out[prefix + ".absmax"] = store.codes, store.absmax
+        if store.diag is not None:
+            out[prefix + ".diag"] = store.diag
+
     def _tensors(self):
         """name -> tensor of everything a checkpoint has to hold."""
         out = {}
         for name, table in (("stats", self.stats), ("precs", self.precs)):
             for order, q in table.items():
-                out[f"{name}.{order}.codes"] = q.codes
-                out[f"{name}.{order}.absmax"] = q.absmax
-                out[f"{name}.{order}.diag"] = q.diag
+                self._store_tensors(f"{name}.{order}", q, out)
         return out
 
     def state_dict(self):
-        return {"active": self._active, **self._tensors()}
+        return {"active": torch.tensor(self.active), **self._tensors()}
 
     def load_state_dict(self, sd):
-        self._active = bool(sd["active"])
+        active = sd["active"]
+        if torch.is_tensor(active) and active.dim() == 1:
+            self.active = [bool(a) for a in active.tolist()]
+        else:                                                       # one flag for the whole bank
+            self.active = [bool(active)] * len(self.params)
         for name, t in self._tensors().items():
             t.copy_(sd[name])

@@ -71,38 +71,59 @@ class ShampooBank2(ShampooBank):
         (reference: utils.py:134-153 with var = matrix_eps * I)."""
         self.basis, self.svalue, self.keep, self.max_eig = {}, {}, {}, {}
         for order, count in self.per_order.items():
-            eye = torch.eye(order, device=self.device).expand(count, order, order).contiguous()
-            self.basis[order] = X.quantize_stack(eye, X.empty_quantized(count, order, self.blocksize, self.bits, self.code, False))
+            self.basis[order] = self._new_store(order, count, 1.0, False)
             half = max(1, order // 2)
             self.keep[order] = torch.arange(half, device=self.device).expand(count, half).contiguous()
             self.svalue[order] = torch.full((count, half), self.matrix_eps, device=self.device)
             self.max_eig[order] = torch.full((count,), self.matrix_eps, device=self.device)
 
     # ---- pieces of QTensorSVDFast, for a whole stack ---------------------------------------------
-    def _rectified_basis(self, order):
-        """Dequantized Vt after rect_t1 Bjorck steps (utils.py:194-198)."""
-        vt = X.dequantize_stack(self.basis[order])
+    def _pick(self, order, rows):
+        """(basis, kept row indices, kept quotients, largest quotient) of the whole stack (rows None) or of a copy
+        of the given rows of it."""
+        if rows is None:
+            return self.basis[order], self.keep[order], self.svalue[order], self.max_eig[order]
+        return (self.basis[order].select(rows), self.keep[order].index_select(0, rows),
+                self.svalue[order].index_select(0, rows), self.max_eig[order].index_select(0, rows))
+
+    def _rectified_basis(self, order, rows=None):
+        """Dequantized Vt after rect_t1 Bjorck steps (utils.py:194-198; a basis held in fp32 is used as it is)."""
+        basis = self._pick(order, rows)[0]
+        vt = X.load_stack(basis)
+        if isinstance(basis, X.DenseStack):
+            return vt
         for _ in range(self.rect_t1):
             vvt = X.gemm(vt, vt, trans_b=True, symmetric=True)
             vt = X.gemm(vvt, vt, addend=vt, alpha=-0.5, beta=1.5)
         return vt
 
-    def _kept_rows(self, order, vt):
+    @staticmethod
+    def _gather_rows(vt, keep):
         n = vt.shape[2]
-        return torch.gather(vt, 1, self.keep[order].unsqueeze(2).expand(-1, -1, n))
+        return torch.gather(vt, 1, keep.unsqueeze(2).expand(-1, -1, n))
 
-    def _statistic(self, order, vt, out=None):
+    def _kept_rows(self, order, vt, rows=None):
+        return self._gather_rows(vt, self._pick(order, rows)[1])
+
+    def _statistic(self, order, vt, out=None, rows=None):
         """Vt[keep]^T diag(S) Vt[keep] (utils.py:200-203)."""
-        rows = self._kept_rows(order, vt)
-        return X.gemm(rows * self.svalue[order].unsqueeze(2), rows, trans_a=True, symmetric=True, out=out)
+        _, keep, svalue, _ = self._pick(order, rows)
+        kept = self._gather_rows(vt, keep)
+        return X.gemm(kept * svalue.unsqueeze(2), kept, trans_a=True, symmetric=True, out=out)
 
     # ---- the operations of the reference's Preconditioner ----------------------------------------
     @torch.no_grad()
-    def add_statistics(self, grads):
-        self._check(grads)
+    def add_statistics(self, grads, only=None):
+        """only: the indices of the parameters whose statistics are updated (default: all).  The stacks that hold
+        a block of one of them are updated whole -- the other matrices of such a stack go through the same update
+        without a gradient term -- and only the rows of the chosen parameters are written back."""
+        only = self._only(only, len(self.params))
+        self._check(grads, only)
         w1 = self.stat_decay
         w2 = 1.0 if w1 == 1.0 else 1.0 - w1
-        orders = sorted(self.per_order, key=lambda o: -o ** 3 * self.per_order[o])
+        orders = [o for o in sorted(self.per_order, key=lambda o: -o ** 3 * self.per_order[o]) if self._touched(o, only)]
+        if not orders:
+            return
         # buffers that cross the phases below belong to the current stream
         stat = {o: torch.empty(self.per_order[o], o, o, device=self.device) for o in orders}
         basis = {}
@@ -120,7 +141,8 @@ class ShampooBank2(ShampooBank):
                 order, first = g.slot[side]
                 seg = stat[order][first:first + len(g)]
                 G = self._grad_list(g, grads)
-                X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, out=seg, symmetric=True)
+                X.gemm(G, G, trans_a=side == 1, trans_b=side == 0, addend=seg, alpha=w2, beta=w1, out=seg, symmetric=True,
+                       skip=self._skip(g, only))
             return run
 
         def project(order):
@@ -140,14 +162,23 @@ class ShampooBank2(ShampooBank):
                 quotients = X.column_dots(Q, LQ) if Q.shape[1] % 64 == 0 else (Q * LQ).sum(dim=1)      # diag(Q^T L Q)
                 ascending, where = torch.sort(quotients, dim=1)
                 half = self.keep[order].shape[1]
-                self.keep[order] = where[:, :half].contiguous()
-                self.svalue[order] = ascending[:, :half].contiguous()
-                self.max_eig[order] = quotients.amax(dim=1)
-                X.quantize_stack(Q, self.basis[order], transposed=True)                # rows of the stored matrix = columns of Q
+                rows = self._rows(order, only)
+                if rows is None:
+                    self.keep[order] = where[:, :half].contiguous()
+                    self.svalue[order] = ascending[:, :half].contiguous()
+                    self.max_eig[order] = quotients.amax(dim=1)
+                    X.store_stack(Q, self.basis[order], transposed=True)               # rows of the stored matrix = columns of Q
+                else:                                                                  # only the chosen parameters' rows change
+                    self.keep[order].index_copy_(0, rows, where[:, :half].index_select(0, rows))
+                    self.svalue[order].index_copy_(0, rows, ascending[:, :half].index_select(0, rows))
+                    self.max_eig[order].index_copy_(0, rows, quotients.amax(dim=1).index_select(0, rows))
+                    chosen = Q.index_select(0, rows)
+                    self.basis[order].put(rows, X.store_stack(chosen, self.basis[order].select(rows), transposed=True))
             return run
 
         self._fan_out([rebuild(o) for o in orders])
-        self._fan_out([accumulate(g, side) for g in self.groups for side in (0, 1)])
+        self._fan_out([accumulate(g, side) for g in self.groups for side in (0, 1)
+                       if only is None or any(pi in only for pi in g.param_index)])
         # The Cholesky QR of every order advances on its own stream; the host waits once per round.
         # (_fan_out gives job i the stream i % streams, so an order keeps its stream from call to call.)
         solver, redone, tick = {}, {}, {}
@@ -225,10 +256,11 @@ class ShampooBank2(ShampooBank):
                 self.low_rank[o][0] = solver[o].repairs * 4 > self.per_order[o]
 
     @torch.no_grad()
-    def compute_preconditioners(self, v0=None):
+    def compute_preconditioners(self, v0=None, only=None):
         """inv_root_mode 0: inverse 4th root from the stored eigenpairs (functional.py:749-762 through
-        utils.py:205-227); 1: coupled Newton on the rebuilt statistic.  v0 as in ShampooBank."""
-        orders = sorted(self.per_order, key=lambda o: -o ** 3 * self.per_order[o])
+        utils.py:205-227); 1: coupled Newton on the rebuilt statistic.  v0, only as in ShampooBank."""
+        only = self._only(only, len(self.params))
+        orders = [o for o in sorted(self.per_order, key=lambda o: -o ** 3 * self.per_order[o]) if self._touched(o, only)]
         starts = {}
         if self.inv_root_mode != 0:
             starts = {o: (torch.rand(self.per_order[o], o, device=self.device) * 2 - 1) if v0 is None else v0[o]
@@ -236,32 +268,51 @@ class ShampooBank2(ShampooBank):
 
         def job(order):
             def run():
+                rows = self._rows(order, only)
+                basis, keep, svalue, max_eig = self._pick(order, rows)
                 if self.inv_root_mode == 0:
-                    rows = self._kept_rows(order, X.dequantize_stack(self.basis[order]))
-                    for _ in range(self.rect_t2):
-                        vvt = X.gemm(rows, rows, trans_b=True, symmetric=True)
-                        rows = X.gemm(vvt, rows, addend=rows, alpha=-0.5, beta=1.5)
-                    ridge = self.matrix_eps * self.max_eig[order]
-                    weights = 1 / (self.svalue[order] + ridge.unsqueeze(1)).pow(1 / 4)
-                    roots = X.gemm(rows * weights.unsqueeze(2), rows, trans_a=True, symmetric=True)
+                    kept = self._gather_rows(X.load_stack(basis), keep)
+                    if not isinstance(basis, X.DenseStack):              # (a basis held in fp32 is not rectified: utils.py:205-227)
+                        for _ in range(self.rect_t2):
+                            vvt = X.gemm(kept, kept, trans_b=True, symmetric=True)
+                            kept = X.gemm(vvt, kept, addend=kept, alpha=-0.5, beta=1.5)
+                    ridge = self.matrix_eps * max_eig
+                    weights = 1 / (svalue + ridge.unsqueeze(1)).pow(1 / 4)
+                    roots = X.gemm(kept * weights.unsqueeze(2), kept, trans_a=True, symmetric=True)
                 else:
-                    L = self._statistic(order, self._rectified_basis(order))
+                    L = self._statistic(order, self._rectified_basis(order, rows), rows=rows)
+                    start = starts[order] if rows is None else starts[order].index_select(0, rows)
                     # L is symmetric up to the rounding inside its diagonal tiles: half products are fine
-                    roots = ComputePowerBatched(L, 4, ridge_epsilon=self.matrix_eps, v0=starts[order], symmetric=True)
-                X.quantize_stack(roots.contiguous(), self.precs[order])
+                    roots = ComputePowerBatched(L, 4, ridge_epsilon=self.matrix_eps, v0=start, symmetric=True)
+                if rows is None:
+                    X.store_stack(roots, self.precs[order])
+                else:
+                    self.precs[order].put(rows, X.store_stack(roots, self.precs[order].select(rows)))
             return run
 
         self._fan_out([job(o) for o in orders])
-        self._active = True
+        for pi in range(len(self.params)):
+            if only is None or pi in only:
+                self.active[pi] = True
 
     # ---- checkpoints -----------------------------------------------------------------------------
     def _tensors(self):
         out = {}
         for order in self.per_order:
-            q = self.basis[order]
-            out[f"basis.{order}.codes"], out[f"basis.{order}.absmax"] = q.codes, q.absmax
+            self._store_tensors(f"basis.{order}", self.basis[order], out)
             out[f"basis.{order}.svalue"], out[f"basis.{order}.keep"] = self.svalue[order], self.keep[order]
             out[f"basis.{order}.max_eigenvalue"] = self.max_eig[order]
-            p = self.precs[order]
-            out[f"precs.{order}.codes"], out[f"precs.{order}.absmax"], out[f"precs.{order}.diag"] = p.codes, p.absmax, p.diag
+            self._store_tensors(f"precs.{order}", self.precs[order], out)
         return out
+
+    def state_dict(self):
+        # (which sweep a stack starts with is part of the state: a resumed run then takes the same sweeps and ends in
+        # the same codes as an uninterrupted one)
+        low_rank = torch.tensor([[o, int(state[0]), int(state[1])] for o, state in sorted(self.low_rank.items())],
+                                dtype=torch.int64).reshape(-1, 3)
+        return {**super().state_dict(), "low_rank": low_rank}
+
+    def load_state_dict(self, sd):
+        super().load_state_dict(sd)
+        if "low_rank" in sd:
+            self.low_rank = {int(o): [bool(flag), int(count)] for o, flag, count in sd["low_rank"].tolist()}

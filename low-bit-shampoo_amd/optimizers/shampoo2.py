@@ -98,8 +98,8 @@ class ShampooAdamW(_Fused2, ShampooAdamWBase):
 
 
 _MORE = """
-        rect_t1 (int): number of iterations t1 for rectification
-        rect_t2 (int): number of iterations t2 for rectification
-        inv_root_mode(int): "0" for SVD computation and "1" for Schur-Newton iteration"""
+        rect_t1: Bjorck steps V <- 1.5 V - 0.5 V V^T V on the dequantized basis before a statistic is rebuilt
+        rect_t2: the same before an inverse root is taken from the stored eigenpairs
+        inv_root_mode: 0 = inverse root from the stored eigenpairs, 1 = coupled Newton iteration on the rebuilt statistic"""
 ShampooSGD.__doc__ = _DOC.format(base="SGD", more=_MORE) + _FusedStep.__doc__
 ShampooAdamW.__doc__ = _DOC.format(base="AdamW", more=_MORE) + _FusedStep.__doc__

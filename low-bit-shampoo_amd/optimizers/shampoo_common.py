@@ -175,6 +175,24 @@ class PreconditionerBase:
     def is_active(self) -> bool:
         return self._active
 
+    # ---- flat checkpoint form (the reference pickles this object: optimizers/shampoo2.py:311-317) ----
+    def state_dict(self):
+        """Plain tensors, numbers and lists only (readable with torch.load(weights_only=True)): 'active' and,
+        per block and side in the order of BlockPartitioner.shapes_for_preconditioners(), the holders'
+        own state_dict()s under 'statistics' and 'preconditioners'."""
+        return {"active": bool(self._active),
+                "statistics": [h.state_dict() for h in self.statistics],
+                "preconditioners": [h.state_dict() for h in self.preconditioners]}
+
+    def load_state_dict(self, sd):
+        if len(sd["statistics"]) != len(self.statistics) or len(sd["preconditioners"]) != len(self.preconditioners):
+            raise ValueError("checkpoint was written for another parameter shape or block size")
+        self._active = bool(sd["active"])
+        for holder, one in zip(self.statistics, sd["statistics"]):
+            holder.load_state_dict(one)
+        for holder, one in zip(self.preconditioners, sd["preconditioners"]):
+            holder.load_state_dict(one)
+
 
 def dense_gram(block, axis):
     return block.T @ block if axis == 1 else block @ block.T
@@ -210,12 +228,42 @@ class _ShampooOptimizer(optim.Optimizer):
     def _init_shampoo(self, prec_bits):
         self.name2qmap = build_code_maps(prec_bits)
 
+    def state_dict(self):
+        """torch's layout, except that no Python object is pickled: the per-parameter preconditioners leave the
+        'state' entries and go, in their flat form (PreconditionerBase.state_dict: tensors, numbers, lists), to
+        'shampoo_preconditioners' = {parameter id as in 'state': flat dict}.  (The reference leaves the
+        Preconditioner objects in the state and thus in the pickle: optimizers/shampoo2.py:311-317.)"""
+        sd = super().state_dict()
+        flat, state = {}, {}
+        for pid, one in sd['state'].items():
+            prec = one.get('preconditioner') if isinstance(one, dict) else None
+            if isinstance(prec, PreconditionerBase):
+                flat[pid] = prec.state_dict()
+                one = {k: v for k, v in one.items() if k != 'preconditioner'}
+            state[pid] = one
+        sd['state'] = state
+        sd['shampoo_preconditioners'] = flat
+        return sd
+
     def load_state_dict(self, state_dict):
+        """Reads what state_dict() writes; a checkpoint whose 'state' entries still hold Preconditioner objects
+        (the reference's form) is taken as well."""
+        state_dict = dict(state_dict)
+        flat = state_dict.pop('shampoo_preconditioners', None) or {}
         super().load_state_dict(state_dict)
+        by_id = {}
+        for group, saved in zip(self.param_groups, state_dict['param_groups']):
+            for p, pid in zip(group['params'], saved['params']):
+                by_id[pid] = (p, group)
+        for pid, one in flat.items():
+            p, group = by_id[pid]
+            prec = self._make_preconditioner(p, group)
+            prec.load_state_dict(one)
+            self.state[p]['preconditioner'] = prec
         for group in self.param_groups:
             for p in group['params']:
                 state = self.state[p]
-                if len(state) != 0 and 'preconditioner' in state:     # absent for parameters held by a ShampooBank
+                if len(state) != 0 and isinstance(state.get('preconditioner'), PreconditionerBase):
                     state['preconditioner'].set_device(p.device)
 
     def _make_preconditioner(self, p, group):
@@ -313,16 +361,16 @@ class ShampooAdamWBase(_ShampooOptimizer):
 
 
 _DOC = r"""
-    Implements {base}+Shampoo.
+    {base} with Shampoo preconditioning of every parameter that has a matrix view.
 
-    Args:
-        start_prec_step (int): the step starting preconditioning
-        stat_compute_steps (int): interval of updating preconditioners (T_1)
-        prec_compute_steps (int): interval of updating inverse roots of preconditioners (T_2)
-        stat_decay (float): exponential decay rate for preconditioners (beta)
-        matrix_eps (float): dampening term (epsilon)
-        prec_maxorder (int): maximum order for preconditioners
-        prec_bits (int): bitwidth of a preconditioner
-        min_lowbit_size (int): minimum tensor size required for quantization
-        quan_blocksize (int): block size for block-wise quantization{more}
+    Arguments beyond those of {base} (names and defaults as in the reference's optimizers):
+        start_prec_step: first step at which the preconditioned direction is used
+        stat_compute_steps: T_1, the statistics L, R take in a gradient every T_1-th step
+        prec_compute_steps: T_2, the inverse 4th roots are recomputed every T_2-th step
+        stat_decay: beta of L <- beta L + (1 - beta) G G^T (1.0: plain sum)
+        matrix_eps: epsilon, the initial statistic is epsilon I and the ridge is epsilon times the largest eigenvalue
+        prec_maxorder: sides longer than this are cut into blocks of at most this order
+        prec_bits: 32, 16, 8 or 4, the storage width of statistics and preconditioners
+        min_lowbit_size: matrices with fewer elements stay in fp32 whatever prec_bits says
+        quan_blocksize: elements per quantization segment (64 ... 2048){more}
     """

@@ -5,6 +5,7 @@ Arithmetic of the reference's step(): optimizers/shampoo1.py:310-331 (SGD), :405
 and the same lines of shampoo2.py.
 """
 import ctypes as ct
+import math
 
 import torch
 
@@ -16,6 +17,9 @@ if F.lib is not None:
     F.lib.qtensor_hip_adamw_tail.restype = None
     F.lib.qtensor_hip_adamw_tail.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_void_p, ct.c_int, ct.c_double, ct.c_double,
                                              ct.c_double, ct.c_double, ct.c_double, ct.c_longlong, ct.c_void_p]
+    F.lib.qtensor_hip_adamw_tail_rows.restype = None
+    F.lib.qtensor_hip_adamw_tail_rows.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_void_p, ct.c_int, ct.c_double, ct.c_double,
+                                                  ct.c_double, ct.c_double, ct.c_double, ct.c_void_p, ct.c_void_p]
     F.lib.qtensor_hip_sgd_tail.restype = None
     F.lib.qtensor_hip_sgd_tail.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_void_p, ct.c_int, ct.c_double, ct.c_double,
                                            ct.c_double, ct.c_int, ct.c_void_p]
@@ -67,9 +71,19 @@ class TailPlan:
         self.keep = (list(params), list(m), list(v))
 
     def adamw(self, params, dirs, grads, exp_avg, exp_avg_sq, graft, lr, betas, eps, weight_decay, step):
+        """step: one count for all parameters, or a list with one count per parameter (the reference counts per
+        parameter: optimizers/shampoo2.py:335-342); counts that differ go up as per-row bias corrections."""
         self._prepare(params, dirs, grads, exp_avg, exp_avg_sq, graft)
-        F._call(F.lib.qtensor_hip_adamw_tail, params[0].device, self.table.data_ptr(), self.owner.data_ptr(), self.n_chunks,
-                self.partial.data_ptr(), int(self.any_graft), lr, betas[0], betas[1], eps, weight_decay, step)
+        steps = [step] * len(params) if isinstance(step, int) else list(step)
+        if all(s == steps[0] for s in steps):
+            F._call(F.lib.qtensor_hip_adamw_tail, params[0].device, self.table.data_ptr(), self.owner.data_ptr(), self.n_chunks,
+                    self.partial.data_ptr(), int(self.any_graft), lr, betas[0], betas[1], eps, weight_decay, steps[0])
+            return
+        rows = [[math.sqrt(1.0 - betas[1] ** s), -lr / (1.0 - betas[0] ** s)] for s in steps]
+        corrections = torch.tensor(rows, dtype=torch.float32).pin_memory().to(params[0].device, non_blocking=True)
+        F._call(F.lib.qtensor_hip_adamw_tail_rows, params[0].device, self.table.data_ptr(), self.owner.data_ptr(), self.n_chunks,
+                self.partial.data_ptr(), int(self.any_graft), lr, betas[0], betas[1], eps, weight_decay, corrections.data_ptr())
+        self.corrections = corrections          # kept until the next call: the launch reads it asynchronously
 
     def sgd(self, params, dirs, grads, momentum_bufs, graft, lr, momentum, weight_decay, nesterov):
         self._prepare(params, dirs, grads, momentum_bufs, [None] * len(params), graft)

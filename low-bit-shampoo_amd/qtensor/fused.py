@@ -42,7 +42,7 @@ class GemmArgs(ct.Structure):
                 ("workspace", ct.c_void_p), ("workspace_floats", ct.c_longlong), ("split_k_", ct.c_int),
                 ("batch_count_", ct.c_int), ("stream_per_", ct.c_int), ("stream_lcm_", ct.c_int),
                 ("batch_inner", ct.c_int), ("inner_a", ct.c_longlong), ("inner_b", ct.c_longlong),
-                ("inner_c", ct.c_longlong), ("inner_e", ct.c_longlong), ("triangular", ct.c_int)]
+                ("inner_c", ct.c_longlong), ("inner_e", ct.c_longlong), ("triangular", ct.c_int), ("pipe", ct.c_int)]
 
 
 class GemmDesc(ct.Structure):
@@ -60,17 +60,37 @@ if F.lib is not None:
 class Quantized:
     """A batch of equally sized quantized square matrices held in stacked buffers.
 
-    codes [batch, order*order*bits/8] uint8, absmax [batch, order*order/blocksize] fp32,
+    codes [batch, ceil(order*order*bits/8)] uint8, absmax [batch, order*ceil(order/blocksize)] fp32,
     diag [batch, order] fp32 or None, all contiguous on one GPU.  Entry b is exactly what
-    quantize_blockwise(_diagreal) writes for one matrix."""
+    quantize_blockwise(_diagreal) writes for one matrix.  `flat`: the blocksize divides the order, so a
+    matrix is one stream of whole segments -- the layout the products read directly (as an operand or an
+    addend); stacks of any other order go through quantize_stack / dequantize_stack only."""
 
     def __init__(self, codes: Tensor, absmax: Tensor, diag: Optional[Tensor], order: int, blocksize: int,
                  bits: int, code: Tensor):
-        if order % blocksize:
-            raise ValueError("fused kernels need blocksize to divide the order")
         self.codes, self.absmax, self.diag = codes, absmax, diag
         self.order, self.blocksize, self.bits, self.code = order, blocksize, bits, code
         self.batch = codes.shape[0] if codes.dim() == 2 else 1
+        self.flat = order % blocksize == 0
+
+    def rows(self, first: int, count: int) -> "Quantized":
+        """The entries first .. first + count - 1 of the stack, as views."""
+        return Quantized(self.codes[first:first + count], self.absmax[first:first + count],
+                         None if self.diag is None else self.diag[first:first + count], self.order, self.blocksize,
+                         self.bits, self.code)
+
+    def select(self, index: Tensor) -> "Quantized":
+        """A copy of the entries index (int64 GPU vector)."""
+        return Quantized(self.codes.index_select(0, index), self.absmax.index_select(0, index),
+                         None if self.diag is None else self.diag.index_select(0, index), self.order, self.blocksize,
+                         self.bits, self.code)
+
+    def put(self, index: Tensor, other: "Quantized") -> None:
+        """Entries index of this stack = the entries of other, in order."""
+        self.codes.index_copy_(0, index, other.codes)
+        self.absmax.index_copy_(0, index, other.absmax)
+        if self.diag is not None:
+            self.diag.index_copy_(0, index, other.diag)
 
     @classmethod
     def from_holder(cls, h) -> "Quantized":
@@ -79,6 +99,8 @@ class Quantized:
                    h.var_order, h.blocksize, h.bits, h.name2qmap[h.code])
 
     def ref(self) -> QuantRef:
+        if not self.flat:
+            raise ValueError("the products read quantized matrices whose order the blocksize divides; dequantize this stack first")
         q = QuantRef()
         q.codes = BatchPtr(self.codes.data_ptr(), None, self.codes.stride(0) if self.codes.dim() == 2 else 0)
         q.absmax = BatchPtr(self.absmax.data_ptr(), None, self.absmax.stride(0) if self.absmax.dim() == 2 else 0)
@@ -151,9 +173,12 @@ def gemm_pipe(mode: Optional[str] = None) -> str:
     return names[F.lib.qtensor_hip_gemm_pipe(-1 if mode is None else names.index(mode))]
 
 
+_PIPES = {None: 0, "f32": 1, "split": 2}
+
+
 def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, alpha=1.0, beta=0.0,
          addend=None, newton=None, skip: Optional[Tensor] = None, symmetric: bool = False,
-         upper_a: bool = False, upper_b: bool = False, requantize: bool = False):
+         upper_a: bool = False, upper_b: bool = False, requantize: bool = False, pipe: Optional[str] = None):
     """out[b] = epilogue(op(A[b]) @ op(B[b])).
 
     A, B: fp32 tensors ([m,k] / [batch,m,k]; with trans_x the stored matrix is the transpose) or a
@@ -169,9 +194,13 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
     into E's buffers (codes, maxima, exact diagonal) -- bit-identical to writing it out and quantizing it, but
     the fp32 matrix never reaches memory; returns E.
     upper_a / upper_b: op(A) / op(B) is upper triangular (zero below the diagonal, square in its k
-    index, dense): the part of the k range where it is zero is skipped."""
+    index, dense): the part of the k range where it is zero is skipped.
+    pipe: None (the process-wide choice, gemm_pipe), "f32" or "split" for this product alone."""
     d = GemmDesc()
     a = d.args
+    if pipe not in _PIPES:
+        raise ValueError('pipe must be None, "f32" or "split"')
+    a.pipe = _PIPES[pipe]
     dev = None
     code = None
     if isinstance(A, Quantized):
@@ -289,10 +318,12 @@ if F.lib is not None:
 
 
 def empty_quantized(batch: int, order: int, blocksize: int, bits: int, code: Tensor, diagreal: bool) -> Quantized:
-    """Uninitialised stacked buffers for `batch` matrices of the given order."""
+    """Uninitialised stacked buffers for `batch` matrices of the given order (any order: a last segment of a
+    row may be shorter, and the codes of an odd order are padded to a whole byte per matrix, as in the
+    single-matrix format)."""
     dev = code.device
-    codes = torch.empty(batch, order * order * bits // 8, dtype=torch.uint8, device=dev)
-    absmax = torch.empty(batch, order * order // blocksize, dtype=torch.float32, device=dev)
+    codes = torch.empty(batch, -(-(order * order * bits) // 8), dtype=torch.uint8, device=dev)
+    absmax = torch.empty(batch, order * (-(-order // blocksize)), dtype=torch.float32, device=dev)
     diag = torch.empty(batch, order, dtype=torch.float32, device=dev) if diagreal else None
     return Quantized(codes, absmax, diag, order, blocksize, bits, code)
 
@@ -311,6 +342,10 @@ def quantize_stack(mats: Tensor, q: Quantized, transposed: bool = False) -> Quan
     for t in (q.codes, q.absmax) + ((q.diag,) if q.diag is not None else ()):
         if not t.is_contiguous():
             raise ValueError("stacked quantized buffers must be contiguous")
+    if q.batch > 65535 and not q.flat:
+        for first in range(0, q.batch, 65535):
+            quantize_stack(mats[first:first + 65535], q.rows(first, min(65535, q.batch - first)), transposed)
+        return q
     if transposed:
         if (q.diag is None and mats.dtype == torch.float32 and q.blocksize in (64, 128, 256)
                 and q.order % q.blocksize == 0 and q.order % 64 == 0):
@@ -332,9 +367,52 @@ def dequantize_stack(q: Quantized, out: Optional[Tensor] = None, outdtype=torch.
     if not out.is_contiguous() or out.shape != (q.batch, q.order, q.order):
         raise ValueError(f"out must be a contiguous stack of shape {(q.batch, q.order, q.order)}")
     slot = F._dtype_slot(out.dtype, "out")
+    if q.batch > 65535 and not q.flat:
+        for first in range(0, q.batch, 65535):
+            dequantize_stack(q.rows(first, min(65535, q.batch - first)), out[first:first + 65535])
+        return out
     F._call(F.lib.qtensor_hip_dequantize_batched, out.device, q.codes.data_ptr(), q.code.data_ptr(), q.bits, q.order,
             q.batch, q.absmax.data_ptr(), None if q.diag is None else q.diag.data_ptr(), out.data_ptr(), slot, q.blocksize)
     return out
+
+
+class DenseStack:
+    """A stack of square matrices [batch, order, order] kept as it is (fp32), with the surface of `Quantized`
+    that the batched step drivers use -- for orders with fewer than min_lowbit_size elements and for
+    prec_bits = 32, where the reference's holders keep the matrix itself (qtensor/utils.py:11-17, 68-74)."""
+    flat = False
+    bits = 32
+    diag = None
+
+    def __init__(self, data: Tensor):
+        if data.dim() != 3 or data.shape[1] != data.shape[2] or data.dtype != torch.float32:
+            raise ValueError("DenseStack takes an fp32 stack [batch, order, order]")
+        self.data = data
+        self.batch, self.order = data.shape[0], data.shape[1]
+
+    def rows(self, first: int, count: int) -> "DenseStack":
+        return DenseStack(self.data[first:first + count])
+
+    def select(self, index: Tensor) -> "DenseStack":
+        return DenseStack(self.data.index_select(0, index))
+
+    def put(self, index: Tensor, other: "DenseStack") -> None:
+        self.data.index_copy_(0, index, other.data)
+
+
+def load_stack(q) -> Tensor:
+    """fp32 [batch, order, order] of a `Quantized` (a new tensor) or a `DenseStack` (its own tensor, no copy)."""
+    return q.data if isinstance(q, DenseStack) else dequantize_stack(q)
+
+
+def store_stack(mats: Tensor, q, transposed: bool = False):
+    """Inverse of load_stack: mats (their transposes with transposed=True) into q's buffers."""
+    if isinstance(q, DenseStack):
+        src = mats.transpose(1, 2) if transposed else mats
+        if transposed or src.data_ptr() != q.data.data_ptr():
+            q.data.copy_(src.contiguous() if transposed else src)
+        return q
+    return quantize_stack(mats.contiguous(), q, transposed)
 
 
 # --------------------------------------------------------------------------- Cholesky QR pieces

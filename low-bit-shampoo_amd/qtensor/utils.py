@@ -59,8 +59,40 @@ class _LowBitState:
                 setattr(self, n, getattr(self, n).to(device))
         self.var = self.var.to(device)
 
+    # ---- flat checkpoint form (no counterpart in the reference, which pickles the holder objects:
+    # optimizers/shampoo2.py:311-317 with qtensor/utils.py:57-61) ---------------------------------
+    _lowbit_tensors = ()                            # side buffers of the low-bit form, per holder class
+
+    def state_dict(self):
+        """Plain tensors and numbers only: 'bits', 'var' (uint8 codes, first element of a pair in the high
+        nibble, or the matrix itself for bits 16 / 32) and, when low-bit, 'order', 'dtype' and the side buffers
+        ('absmax' fp32 [order * ceil(order / blocksize)], 'diag' fp32 [order] for the exact-diagonal form)."""
+        out = {"bits": int(self.bits), "var": self.var}
+        if self.bits < 16:
+            out["order"] = int(self.var_order)
+            out["dtype"] = str(self.var_dtype).replace("torch.", "")
+            for name in self._lowbit_tensors:
+                out[name] = getattr(self, name)
+        return out
+
+    def load_state_dict(self, sd):
+        """Takes what state_dict() wrote into a holder constructed with the same arguments."""
+        if int(sd["bits"]) != int(self.bits):
+            raise ValueError(f"checkpointed holder has {int(sd['bits'])} bits, this one {self.bits}")
+        device = self.var.device
+        if self.bits >= 16:
+            self.var = sd["var"].to(device=device, dtype=self.var.dtype).clone()
+            return
+        self.var_order = int(sd["order"])
+        self.var_dtype = getattr(torch, sd["dtype"])
+        self.var = sd["var"].to(device).clone()
+        for name in self._lowbit_tensors:
+            setattr(self, name, sd[name].to(device).clone())
+
 
 class QTensor(_LowBitState):
+    _lowbit_tensors = ("absmax",)
+
     def __init__(self, var, bits=32, name2qmap={}, code='', blocksize=2048, min_lowbit_size=4096):
         if self._adopt_format(var, bits, name2qmap, code, blocksize, min_lowbit_size):
             self.var_dtype = var.dtype
@@ -87,6 +119,8 @@ class QTensor(_LowBitState):
 
 
 class QTensorDiagReal(_LowBitState):
+    _lowbit_tensors = ("absmax", "diag")
+
     def __init__(self, var, bits=32, name2qmap={}, code='', blocksize=2048, min_lowbit_size=4096):
         if self._adopt_format(var, bits, name2qmap, code, blocksize, min_lowbit_size):
             self.var_dtype = var.dtype
@@ -131,6 +165,23 @@ class QTensorSVDFast(_LowBitState):
     Svalue / keep_indices are the smaller half of the Rayleigh quotients and the rows they
     belong to; max_eigenvalue is the largest quotient (used to scale the ridge term).
     rect_t1 / rect_t2 Bjorck steps re-orthonormalise Vt after dequantization."""
+    _lowbit_tensors = ("absmax",)
+
+    def state_dict(self):
+        """As the other holders ('var' = the basis Vt), plus 'Svalue' fp32 [n/2], 'keep_indices' int64 [n/2]
+        and 'max_eigenvalue' (fp32 scalar)."""
+        out = super().state_dict()
+        out.update(Svalue=self.Svalue, keep_indices=self.keep_indices, max_eigenvalue=self.max_eigenvalue,
+                   log_written=bool(self._log_written))
+        return out
+
+    def load_state_dict(self, sd):
+        super().load_state_dict(sd)
+        device = self.var.device
+        self.Svalue = sd["Svalue"].to(device).clone()
+        self.keep_indices = sd["keep_indices"].to(device=device, dtype=torch.int64).clone()
+        self.max_eigenvalue = sd["max_eigenvalue"].to(device).clone()
+        self._log_written = bool(sd.get("log_written", False))
 
     def __init__(self, var, bits=32, name2qmap={}, code='', blocksize=2048, min_lowbit_size=4096,
                  rect_t1=1, rect_t2=4, log_prefix=None):

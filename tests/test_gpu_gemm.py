@@ -75,22 +75,17 @@ def test_quantized_factor_times_dense(mods, code_maps, bits, bs, name, diag):
     F, X = mods
     g = torch.Generator().manual_seed(bits + bs)
     # (few and many matrices, narrow and wide partners: between them the cases take every tile shape)
-    before = X.gemm_pipe()
-    try:
-        for n, other, batch in ((256, 100, 2), (768, 320, 1), (1024, 64, 1), (256, 200, 40), (512, 128, 24), (128, 64, 60), (64, 256, 30)):
-            if n % bs:
-                continue
-            mats = torch.randn(batch, n, n, generator=g)
-            mats[:, 3, :64] = 0.0                                  # a zero-maximum segment
-            q, deq = make_quantized(F, X, mats, code_maps[(name, bits)], bits, bs, diag)
-            G_left = torch.randn(batch, n, other, generator=g)
-            G_right = torch.randn(batch, other, n, generator=g)
-            for pipe in ("split", "f32"):
-                X.gemm_pipe(pipe)
-                assert rel_err(X.gemm(q, G_left.cuda()), deq @ G_left.double()) <= TOL, (pipe, n, other, batch)
-                assert rel_err(X.gemm(G_right.cuda(), q), G_right.double() @ deq) <= TOL, (pipe, n, other, batch)
-    finally:
-        X.gemm_pipe(before)
+    for n, other, batch in ((256, 100, 2), (768, 320, 1), (1024, 64, 1), (256, 200, 40), (512, 128, 24), (128, 64, 60), (64, 256, 30)):
+        if n % bs:
+            continue
+        mats = torch.randn(batch, n, n, generator=g)
+        mats[:, 3, :64] = 0.0                                  # a zero-maximum segment
+        q, deq = make_quantized(F, X, mats, code_maps[(name, bits)], bits, bs, diag)
+        G_left = torch.randn(batch, n, other, generator=g)
+        G_right = torch.randn(batch, other, n, generator=g)
+        for pipe in ("split", "f32"):                          # chosen per product: the process-wide mode stays as it is
+            assert rel_err(X.gemm(q, G_left.cuda(), pipe=pipe), deq @ G_left.double()) <= TOL, (pipe, n, other, batch)
+            assert rel_err(X.gemm(G_right.cuda(), q, pipe=pipe), G_right.double() @ deq) <= TOL, (pipe, n, other, batch)
 
 
 def test_config3_preconditioned_gradient(mods, code_maps):
@@ -440,27 +435,20 @@ def test_split_pipe_is_as_accurate_as_the_fp32_pipe(mods, batch, m, n, k, spread
     it), well scaled entries and entries spread over e^(+-9)."""
     _, X = mods
     g = torch.Generator().manual_seed(batch * 7 + k)
-    before = X.gemm_pipe()
-    try:
-        for trans_a, trans_b in ((False, False), (False, True), (True, False)):
-            A = torch.randn((batch, k, m) if trans_a else (batch, m, k), generator=g)
-            B = torch.randn((batch, n, k) if trans_b else (batch, k, n), generator=g)
-            A = (A * torch.exp(spread * torch.randn(A.shape, generator=g))).cuda()
-            B = (B * torch.exp(spread * torch.randn(B.shape, generator=g))).cuda()
-            a64 = (A.transpose(1, 2) if trans_a else A).double()
-            b64 = (B.transpose(1, 2) if trans_b else B).double()
-            want, scale = a64 @ b64, a64.abs() @ b64.abs()
-            out = {}
-            for pipe in ("f32", "split"):
-                X.gemm_pipe(pipe)
-                out[pipe] = X.gemm(A, B, trans_a=trans_a, trans_b=trans_b)
-            assert not torch.equal(out["f32"], out["split"])                     # the split pipe was taken
-            err = {p: ((o.double() - want).abs() / scale) for p, o in out.items()}
-            assert float(err["split"].max()) <= 1.05 * float(err["f32"].max()) + 1e-8, (trans_a, trans_b)
-            assert float(err["split"].mean()) <= 1.02 * float(err["f32"].mean()), (trans_a, trans_b)
-            assert float(err["split"].max()) <= 2e-5 and float(err["f32"].max()) <= 2e-5
-    finally:
-        X.gemm_pipe(before)
+    for trans_a, trans_b in ((False, False), (False, True), (True, False)):
+        A = torch.randn((batch, k, m) if trans_a else (batch, m, k), generator=g)
+        B = torch.randn((batch, n, k) if trans_b else (batch, k, n), generator=g)
+        A = (A * torch.exp(spread * torch.randn(A.shape, generator=g))).cuda()
+        B = (B * torch.exp(spread * torch.randn(B.shape, generator=g))).cuda()
+        a64 = (A.transpose(1, 2) if trans_a else A).double()
+        b64 = (B.transpose(1, 2) if trans_b else B).double()
+        want, scale = a64 @ b64, a64.abs() @ b64.abs()
+        out = {pipe: X.gemm(A, B, trans_a=trans_a, trans_b=trans_b, pipe=pipe) for pipe in ("f32", "split")}
+        assert not torch.equal(out["f32"], out["split"])                     # the split pipe was taken
+        err = {p: ((o.double() - want).abs() / scale) for p, o in out.items()}
+        assert float(err["split"].max()) <= 1.05 * float(err["f32"].max()) + 1e-8, (trans_a, trans_b)
+        assert float(err["split"].mean()) <= 1.02 * float(err["f32"].mean()), (trans_a, trans_b)
+        assert float(err["split"].max()) <= 2e-5 and float(err["f32"].max()) <= 2e-5
 
 
 def test_split_pipe_switch_epilogues_and_special_values(mods):
@@ -495,5 +483,33 @@ def test_split_pipe_switch_epilogues_and_special_values(mods):
         bad[3, 7, 9] = float("inf")
         out = X.gemm(bad, Bm)
         assert bool(out[3, 7].isnan().all()) and bool(torch.isfinite(out[3, 8]).all()) and bool(torch.isfinite(out[2]).all())
+        # the per-product choice overrides the process-wide mode, in both directions, and leaves it alone
+        assert torch.equal(X.gemm(A, Bm, pipe="f32"), [X.gemm_pipe("f32"), X.gemm(A, Bm), X.gemm_pipe("split")][1])
+        assert torch.equal(X.gemm(A, Bm, pipe="split"), X.gemm(A, Bm)) and X.gemm_pipe() == "split"
+        with pytest.raises(ValueError):
+            X.gemm(A, Bm, pipe="bf16")
     finally:
         X.gemm_pipe(before)
+
+
+def test_split_pipe_at_the_top_of_the_fp32_range(mods):
+    """The leading bf16 piece of an element rounds to infinity from 0x7f7f8000 (about 3.3962e38) on: such an element
+    behaves like an infinite one on the split pipe (NaN in its row of the result), as the header says; just below
+    that the product is as accurate as anywhere else, and the fp32 pipe takes the whole range."""
+    _, X = mods
+    g = torch.Generator().manual_seed(9)
+    n = 128
+    A = torch.randn(1, n, n, generator=g).cuda()
+    Bm = torch.zeros(1, n, n, device="cuda")
+    Bm[0].fill_diagonal_(2.0 ** -20)                          # results stay finite: each is one scaled element of A
+    below = torch.tensor(0x7f7f7fff, dtype=torch.int32).view(torch.float32).item()      # the largest element that still splits
+    at = torch.tensor(0x7f7f8000, dtype=torch.int32).view(torch.float32).item()
+    A[0, 5, 17], A[0, 9, 3] = below, -below
+    for pipe in ("split", "f32"):
+        out = X.gemm(A, Bm, pipe=pipe)
+        assert bool(torch.isfinite(out).all())
+        assert rel_err(out, (A.double() @ Bm.double()).cpu()) <= TOL
+    A[0, 5, 17] = at
+    out = X.gemm(A, Bm, pipe="split")
+    assert bool(out[0, 5].isnan().all()) and bool(torch.isfinite(out[0, 4]).all()) and bool(torch.isfinite(out[0, 9]).all())
+    assert bool(torch.isfinite(X.gemm(A, Bm, pipe="f32")).all())

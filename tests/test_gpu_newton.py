@@ -1,11 +1,21 @@
-"""GPU parity of the batched coupled-Newton inverse root against the single-matrix form run on
-the CPU with the same start vectors (the reference's algorithm, optimizers/matrix_functions.py)."""
+"""GPU parity of the batched coupled-Newton inverse root against the CPU restatement of the reference's
+algorithm (oracle/shampoo_ref.py: power_iteration, newton_root; reference optimizers/matrix_functions.py:21-141,
+pinned to the reference's own seeded runs in tests/test_shampoo_oracle.py) with the same start vectors."""
 import pytest
 import torch
 
-from optimizers.matrix_functions import ComputePower, ComputePowerBatched, PowerIterBatched, PowerIter
+from optimizers.matrix_functions import ComputePowerBatched, PowerIterBatched
+from oracle.shampoo_ref import newton_root, power_iteration
 
 pytestmark = pytest.mark.gpu
+
+
+def ComputePower(mat, p, ridge_epsilon, v0):
+    return newton_root(mat, p, ridge_epsilon, v0)
+
+
+def PowerIter(mat, v0):
+    return power_iteration(mat, v0), None, None
 
 
 def psd_stack(batch, n, cond, seed):

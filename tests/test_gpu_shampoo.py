@@ -80,9 +80,11 @@ def test_bank_equals_per_parameter_path(setup, code_maps, bits):
     params = [torch.zeros(s, device="cuda") for s in mats]
     kw = {k: v for k, v in KW.items() if k in ("prec_maxorder", "prec_bits", "min_lowbit_size", "quan_blocksize")}
     assert all(ShampooBank.accepts(p, **kw) for p in params)
-    assert not ShampooBank.accepts(torch.zeros(64, device="cuda"), **kw)
-    assert not ShampooBank.accepts(torch.zeros(128, 100, device="cuda"), **kw)       # 100 is not a multiple of 64
+    assert not ShampooBank.accepts(torch.zeros(64, device="cuda"), **kw)             # a vector has no statistics
+    assert ShampooBank.accepts(torch.zeros(128, 100, device="cuda"), **kw)           # 100 is not a multiple of 64: general layout
+    assert ShampooBank.accepts(torch.zeros(96, 40, device="cuda"), **kw)             # 40 x 40 is below min_lowbit_size: kept in fp32
     assert not ShampooBank.accepts(torch.zeros(128, 128), **kw)                      # CPU
+    assert not ShampooBank.accepts(torch.zeros(128, 128, device="cuda", dtype=torch.bfloat16), **kw)
     qmap = {"linear-2": torch.from_numpy(code)}
     bank = ShampooBank(params, qmap, "linear-2", **KW)
     pres = [S1.Preconditioner(p, qmap, **KW) for p in params]
@@ -136,7 +138,7 @@ def test_fused_optimizer_matches_per_parameter_optimizer(setup, which, monkeypat
     real_rand = torch.rand
     # identical, deterministic power-iteration start vectors on both paths
     monkeypatch.setattr(MF.torch, "rand", lambda *size, **kw: torch.full(size, 0.75, **kw))
-    shapes = SHAPES + [(128, 100)]                     # the last one cannot enter the bank
+    shapes = SHAPES + [(128, 100), (96, 40)]           # orders the blocksize does not divide / too small to quantize
     g = torch.Generator().manual_seed(5)
     init = [real_rand(s, generator=g) for s in shapes]
     gs = [[0.02 * torch.randn(s, generator=g) for s in shapes] for _ in range(4)]
@@ -248,12 +250,14 @@ def test_fused_optimizer_checkpoint_round_trip(setup, which, monkeypatch):
     run(opt, first, range(3))
     sd = opt.state_dict()
     bank = sd["shampoo_bank"]
-    assert len(bank) == 1 and int(bank[0]["step"]) == 3 and bank[0]["block_table"].shape[1] == 5
-    assert all(isinstance(v, (torch.Tensor, bool)) for v in bank[0].values())
+    assert len(bank) == 1 and bank[0]["block_table"].shape[1] == 5
+    assert all(isinstance(v, torch.Tensor) for v in bank[0].values())
+    assert all(opt.state[p]["step"] == 3 for p in first)
+    assert not any("preconditioner" in opt.state[p] for p in first if p.dim() > 1)      # every matrix lives in the bank
     buf = io.BytesIO()
-    torch.save(bank, buf)
+    torch.save(sd, buf)                                   # the WHOLE state: nothing in it is a pickled object
     buf.seek(0)
-    sd["shampoo_bank"] = torch.load(buf, weights_only=True, map_location="cpu")
+    sd = torch.load(buf, weights_only=True, map_location="cpu")
     resumed = [torch.nn.Parameter(p.detach().clone()) for p in first]
     opt2 = make(resumed)
     opt2.load_state_dict(sd)
@@ -271,8 +275,41 @@ def test_fused_optimizer_checkpoint_round_trip(setup, which, monkeypatch):
         opt3.step()
 
 
-def test_fused_step_error_paths_that_differ_from_the_per_parameter_step(setup):
-    """What fused=True does where the reference's step() would skip a parameter, and what it refuses to load."""
+@pytest.mark.parametrize("which", ["adamw", "sgd"])
+def test_fused_step_skips_and_counts_per_parameter_like_the_reference(setup, which, monkeypatch):
+    """A parameter without a gradient is skipped and every parameter counts its own steps (reference:
+    optimizers/shampoo1.py:371-377, 394-396): the fused step with gradients missing on some steps against the
+    per-parameter optimizer on the same gradients."""
+    S1 = setup[0]
+    import optimizers.matrix_functions as MF
+    real_rand = torch.rand
+    monkeypatch.setattr(MF.torch, "rand", lambda *size, **kw: torch.full(size, 0.75, **kw))
+    shapes = SHAPES + [(128, 100)]
+    g = torch.Generator().manual_seed(15)
+    init = [real_rand(s, generator=g) for s in shapes]
+    gs = [[0.02 * torch.randn(s, generator=g) for s in shapes] for _ in range(7)]
+    # which parameters have a gradient at which step: the second one joins late, the first one pauses twice,
+    # the vector pauses once, the last one is there every other step
+    present = [[st not in (2, 3), st >= 2, st != 4, True, st % 2 == 0] for st in range(7)]
+    finals, counts = [], []
+    for fused in (False, True):
+        params = [torch.nn.Parameter(t.clone().cuda()) for t in init]
+        common = dict(start_prec_step=2, stat_compute_steps=1, prec_compute_steps=2, fused=fused, **KW)
+        opt = (S1.ShampooAdamW(params, lr=1e-2, weight_decay=0.05, **common) if which == "adamw"
+               else S1.ShampooSGD(params, lr=1e-2, momentum=0.9, weight_decay=1e-3, **common))
+        for st in range(7):
+            for p, gr, there in zip(params, gs[st], present[st]):
+                p.grad = gr.clone().cuda() if there else None
+            opt.step()
+        finals.append([p.detach().cpu() for p in params])
+        counts.append([opt.state[p]["step"] for p in params])
+    assert counts[0] == counts[1] == [sum(row[k] for row in present) for k in range(len(shapes))]
+    for a, b in zip(*finals):
+        assert rel(a, b) <= 2e-4
+
+
+def test_fused_step_error_paths(setup):
+    """What the fused optimizer refuses."""
     S1 = setup[0]
     g = torch.Generator().manual_seed(8)
     params = [torch.nn.Parameter(torch.rand(s, generator=g).cuda()) for s in SHAPES]
@@ -281,14 +318,7 @@ def test_fused_step_error_paths_that_differ_from_the_per_parameter_step(setup):
         p.grad = 0.02 * torch.randn(p.shape, generator=g).cuda()
     opt.step()
     assert all(opt.state[p]["step"] == 1 for p in params)
-    # a banked parameter without a gradient on a later step: refused, nothing is skipped silently
-    before = [p.detach().clone() for p in params]
-    params[0].grad = None
-    with pytest.raises(RuntimeError, match="needs a gradient at every later step"):
-        opt.step()
-    assert all(torch.equal(a, p.detach()) for a, p in zip(before, params))           # and nothing was updated
     # a checkpoint of the fused optimizer does not load into the per-parameter one
-    params[0].grad = 0.02 * torch.randn(params[0].shape, generator=g).cuda()
     sd = opt.state_dict()
     plain = S1.ShampooAdamW([torch.nn.Parameter(p.detach().clone()) for p in params], lr=1e-2, start_prec_step=2,
                             stat_compute_steps=1, prec_compute_steps=2, fused=False, **KW)
@@ -301,3 +331,48 @@ def test_fused_step_error_paths_that_differ_from_the_per_parameter_step(setup):
     with pytest.raises((ValueError, NotImplementedError, RuntimeError)):
         ShampooBank(many, {"code": F.create_linear_map(True, 4, 2)}, "code", prec_maxorder=64, prec_bits=4, min_lowbit_size=4096,
                     quan_blocksize=64)
+
+
+def test_per_parameter_optimizer_checkpoint_is_flat(setup, monkeypatch):
+    """fused=False: state_dict() moves the Preconditioner objects out of the per-parameter state into their flat form
+    (tensors, numbers, lists), so the whole checkpoint loads with weights_only=True, and a resumed run continues
+    bit for bit."""
+    import io
+    S1 = setup[0]
+    import optimizers.matrix_functions as MF
+    real_rand = torch.rand
+    monkeypatch.setattr(MF.torch, "rand", lambda *size, **kw: torch.full(size, 0.75, **kw))
+    shapes = SHAPES + [(128, 100), (96, 40)]
+    g = torch.Generator().manual_seed(16)
+    init = [real_rand(s, generator=g) for s in shapes]
+    gs = [[0.02 * torch.randn(s, generator=g) for s in shapes] for _ in range(5)]
+
+    def make(params):
+        return S1.ShampooAdamW(params, lr=1e-2, weight_decay=0.05, start_prec_step=2, stat_compute_steps=1, prec_compute_steps=2,
+                               fused=False, **KW)
+
+    def run(opt, params, steps):
+        for st in steps:
+            for p, gr in zip(params, gs[st]):
+                p.grad = gr.clone().cuda()
+            opt.step()
+
+    straight = [torch.nn.Parameter(t.clone().cuda()) for t in init]
+    run(make(straight), straight, range(5))
+    first = [torch.nn.Parameter(t.clone().cuda()) for t in init]
+    opt = make(first)
+    run(opt, first, range(3))
+    sd = opt.state_dict()
+    assert len(sd["shampoo_preconditioners"]) == len(shapes)
+    assert not any("preconditioner" in one for one in sd["state"].values())
+    assert all("preconditioner" in opt.state[p] for p in first)                      # the live state is untouched
+    buf = io.BytesIO()
+    torch.save(sd, buf)
+    buf.seek(0)
+    sd = torch.load(buf, weights_only=True, map_location="cpu")
+    resumed = [torch.nn.Parameter(p.detach().clone()) for p in first]
+    opt2 = make(resumed)
+    opt2.load_state_dict(sd)
+    run(opt2, resumed, range(3, 5))
+    for a, b in zip(straight, resumed):
+        assert torch.equal(a.detach(), b.detach())

@@ -116,3 +116,61 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit(api, capfd):
     torch.cuda.synchronize()
     assert bool((C == 7.0).all())                            # nothing was launched
     capfd.readouterr()
+
+
+def test_static_scratch_entry_point_allocates_nothing_and_refuses_overlapping_calls(api, capfd):
+    """The property the entry point exists for: a call (after the first one on the device, which looks the static
+    array up) takes no device memory -- the free memory of the device is the same before and after, with torch's
+    caching allocator left out of it -- and a call on another stream while the last call's work is still running is
+    refused instead of racing on the one shared array."""
+    lib, X = api
+    g = torch.Generator().manual_seed(4)
+    m, n, k = 768, 1024, 3072
+    A, B = torch.randn(m, k, generator=g).cuda(), torch.randn(k, n, generator=g).cuda()
+    C, C2 = torch.empty(m, n, device="cuda"), torch.empty(m, n, device="cuda")
+    main = torch.cuda.current_stream()
+    other = torch.cuda.Stream()
+    desc, desc2 = dense_desc(X, A, B, C), dense_desc(X, A, B, C2)
+    lib.qtensor_hip_gemm_static(ct.byref(desc), main.cuda_stream)                    # warm: symbol looked up, kernels loaded
+    assert lib.qtensor_hip_last_error() == 0
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    reserved_before = torch.cuda.memory_reserved()
+    for _ in range(3):
+        lib.qtensor_hip_gemm_static(ct.byref(desc), main.cuda_stream)
+        assert lib.qtensor_hip_last_error() == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_reserved() == reserved_before
+    want = C.clone()
+    # the same stream again and again: ordered by the stream, never refused
+    for _ in range(3):
+        lib.qtensor_hip_gemm_static(ct.byref(desc), main.cuda_stream)
+        assert lib.qtensor_hip_last_error() == 0
+    # another stream while the first one is still busy: refused, nothing launched.  (The first stream is kept busy by
+    # work queued ahead of the product: a long elementwise chain.)
+    busy = torch.zeros(1 << 26, device="cuda")
+    torch.cuda.synchronize()
+    for _ in range(40):
+        busy.add_(1.0)
+    lib.qtensor_hip_gemm_static(ct.byref(desc), main.cuda_stream)
+    assert lib.qtensor_hip_last_error() == 0
+    with torch.cuda.stream(other):
+        C2.fill_(7.0)
+    # (no ordering between the two streams: that is the point)
+    with torch.cuda.stream(other):
+        lib.qtensor_hip_gemm_static(ct.byref(desc2), other.cuda_stream)
+        refused = lib.qtensor_hip_last_error() != 0
+        message = lib.qtensor_hip_last_error_string()
+    torch.cuda.synchronize()
+    if refused:
+        assert b"still in use" in message
+    else:
+        # the first stream had already drained when the second call came (a very fast device): then the call is legal
+        assert torch.equal(C2, want)
+    # once the earlier work is done, the other stream is welcome
+    with torch.cuda.stream(other):
+        lib.qtensor_hip_gemm_static(ct.byref(desc2), other.cuda_stream)
+        assert lib.qtensor_hip_last_error() == 0, lib.qtensor_hip_last_error_string()
+    torch.cuda.synchronize()
+    assert torch.equal(C2, want) and torch.equal(C, want)
+    capfd.readouterr()
