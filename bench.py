@@ -419,6 +419,7 @@ def main():
                          "keeps per-kernel durations in a profile free of overlap)")
     ap.add_argument("--gemm-pipe", choices=["f32", "split"], default=None,
                     help="matrix pipe of the products of dense operands (default: the library's, the split bf16 pipe)")
+    ap.add_argument("--probe-queues", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-step", action="store_true", help="skip the fused-product, other-format and Shampoo-step measurements")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -437,13 +438,15 @@ def main():
     if args.gemm_pipe is not None:
         import qtensor.fused as X
         X.gemm_pipe(args.gemm_pipe)
+    if args.probe_queues:
+        import optimizers.engine as E
+        E.PROBE_QUEUES = True
     if args.bank_streams is not None:
         from optimizers.engine import ShampooBank
         from optimizers.engine2 import ShampooBank2
         ShampooBank.DEFAULT_STREAMS = ShampooBank2.DEFAULT_STREAMS = args.bank_streams
         if args.bank_streams == 0:           # profiling: nothing may overlap, the side thread of shampoo2 neither
             from optimizers import shampoo2
-            shampoo2.ShampooAdamW.overlap_unbatched_statistics = False
             shampoo2.ShampooAdamW.overlap_precondition = False
     if args.section in ("gemm", "step", "step2", "product"):
         if args.section == "gemm":

@@ -46,6 +46,7 @@ class ShampooBank2(ShampooBank):
         self.qr_repairs = 0                       # matrices that went through the replacing sweep so far (low numerical rank)
         self.alongside = None                     # callable that the next add_statistics runs next to its factorisations
         self.low_rank = {}                        # order -> [most of the stack needed the replacing sweep, updates since the plain one was tried]
+        self.low_rank_rows = {}                   # order -> {row: [updates between two looks at the plain sweep, updates until the next look]}
         super().__init__(params, name2qmap, code, **kwargs)
 
     LOOK_AGAIN = 8                                # updates after which a stack of low numerical rank tries the plain sweep again
@@ -62,6 +63,25 @@ class ShampooBank2(ShampooBank):
             state[1] = 0
             return False
         return True
+
+    REPAIR_SLOT = 5                               # side stream of the replacing sweeps that start next to a stack's own sweep
+
+    def _presweep_rows(self, order):
+        """The matrices of this stack whose replacing sweep starts right away: those whose recent updates ended in it.
+        Every `period` updates such a matrix gets the plain sweep alone again; a period doubles (8, 16, ... 256) each
+        time that look ends in the replacing sweep once more."""
+        rows = []
+        for row, state in self.low_rank_rows.setdefault(order, {}).items():
+            if state[1] > 0:
+                state[1] -= 1
+                rows.append(row)
+        return rows
+
+    def _note_repairs(self, order, repaired):
+        table = self.low_rank_rows.setdefault(order, {})
+        for row in repaired:
+            period = min(2 * table[row][0], 256) if row in table else 8
+            table[row] = [period, period]
 
     def _beside_stream(self):
         return shared_stream(self.device, BESIDE_SLOT)       # (the same stream as the fourth of the fan-out streams)
@@ -147,7 +167,8 @@ class ShampooBank2(ShampooBank):
 
         def project(order):
             def run():
-                solver[order] = X.CholeskyQR(X.gemm(stat[order], basis[order], trans_b=True), replace_first=direct[order])     # L Vt^T
+                solver[order] = X.CholeskyQR(X.gemm(stat[order], basis[order], trans_b=True), replace_first=direct[order],
+                                             replace_rows=early[order], side_stream=shared_stream(self.device, self.REPAIR_SLOT))     # L Vt^T
                 # (the event that tells the host this stack's sweep is through goes right behind it: streams share
                 # hardware queues, and behind the launches of another stack's sweep it would wait for those as well)
                 tick[order] = torch.cuda.Event()
@@ -183,14 +204,20 @@ class ShampooBank2(ShampooBank):
         # (_fan_out gives job i the stream i % streams, so an order keeps its stream from call to call.)
         solver, redone, tick = {}, {}, {}
         direct = {o: self._replace_first(o) for o in orders}
+        early = {o: self._presweep_rows(o) for o in orders}
         # Two lanes for the sweeps and what follows them: a process has four hardware queues, the parameters outside
         # the bank and the job that applies the stored roots take one each, and streams beyond that share a queue in
         # the order of their launches -- a third stack on a stream of its own ran behind the second anyway, and held
         # up what the second had to do after its sweep.  The stacks are dealt out by cost, the cheap ones of a lane first.
-        lanes = [[] for _ in range(min(LANES, len(orders)))]
-        for o in orders:                                                   # (most expensive first)
-            min(lanes, key=lambda lane: sum(x ** 3 * self.per_order[x] for x in lane)).append(o)
-        lanes = [sorted(lane, key=lambda x: x ** 3 * self.per_order[x]) for lane in lanes]
+        cost = {o: o ** 3 * self.per_order[o] for o in orders}
+        small = [o for o in orders if cost[o] * 50 < max(cost.values())]          # a matrix or two of a small order: a chain of tiny launches
+        big = [o for o in orders if o not in small]
+        lanes = [[] for _ in range(min(LANES, len(big)))]
+        for o in big:                                                      # (most expensive first)
+            min(lanes, key=lambda lane: sum(cost[x] for x in lane)).append(o)
+        lanes = [sorted(lane, key=lambda x: cost[x]) for lane in lanes]
+        if small:                                                          # (they get a lane of their own: nothing big waits behind them)
+            lanes.append(sorted(small, key=lambda x: cost[x]))
         slot = {o: i for i, lane in enumerate(lanes) for o in lane}
         self._fan_out([(lambda lane=lane: [project(o)() for o in lane]) for lane in lanes])
         # work of the caller that does not depend on the statistics (bank.alongside, consumed here) fills the device
@@ -254,6 +281,7 @@ class ShampooBank2(ShampooBank):
         for o in orders:
             if not direct[o]:
                 self.low_rank[o][0] = solver[o].repairs * 4 > self.per_order[o]
+                self._note_repairs(o, solver[o].repaired_ids)
 
     @torch.no_grad()
     def compute_preconditioners(self, v0=None, only=None):
@@ -310,9 +338,15 @@ class ShampooBank2(ShampooBank):
         # the same codes as an uninterrupted one)
         low_rank = torch.tensor([[o, int(state[0]), int(state[1])] for o, state in sorted(self.low_rank.items())],
                                 dtype=torch.int64).reshape(-1, 3)
-        return {**super().state_dict(), "low_rank": low_rank}
+        rows = torch.tensor([[o, row, state[0], state[1]] for o, table in sorted(self.low_rank_rows.items())
+                             for row, state in sorted(table.items())], dtype=torch.int64).reshape(-1, 4)
+        return {**super().state_dict(), "low_rank": low_rank, "low_rank_rows": rows}
 
     def load_state_dict(self, sd):
         super().load_state_dict(sd)
         if "low_rank" in sd:
             self.low_rank = {int(o): [bool(flag), int(count)] for o, flag, count in sd["low_rank"].tolist()}
+        if "low_rank_rows" in sd:
+            self.low_rank_rows = {}
+            for o, row, period, left in sd["low_rank_rows"].tolist():
+                self.low_rank_rows.setdefault(int(o), {})[int(row)] = [int(period), int(left)]

@@ -580,7 +580,8 @@ class CholeskyQR:
     matrices still in the working set, result() returns (Q, number of matrices redone by the
     library).  All calls for one object must be made with the same current stream."""
 
-    def __init__(self, Y, max_rounds=12, pivot_floor=PIVOT_FLOOR, tolerance=2e-5, sweep=True, replace_first=False):
+    def __init__(self, Y, max_rounds=12, pivot_floor=PIVOT_FLOOR, tolerance=2e-5, sweep=True, replace_first=False,
+                 replace_rows=None, side_stream=None):
         if Y.dim() != 3 or Y.shape[1] != Y.shape[2] or Y.dtype != torch.float32 or not Y.is_cuda:
             raise ValueError("CholeskyQR takes an fp32 GPU stack [B, n, n]")
         B, self.true_n, _ = Y.shape
@@ -600,6 +601,8 @@ class CholeskyQR:
         self.finished = False
         self.rounds = 0                               # factorisation rounds enqueued so far
         self.repairs = 0                              # matrices swept a second time (see _repair)
+        self.repaired_ids = []                        # which matrices of the stack those were
+        self.presweep = None                          # (rows, their replacing sweep's result, event): see replace_rows below
         self.gram = self.far = None
         # The bookkeeping lives on the host (it waits once per round anyway), per working-set entry:
         # which matrix of the stack it is and whether it is within ||G - I||_F < 0.5.
@@ -617,6 +620,24 @@ class CholeskyQR:
             # fp32 rounding by construction; the rounds below are for the other matrices only.
             # replace_first: the caller knows the stack to be of low numerical rank (its last update needed the
             # replacing sweep for most matrices) and goes there directly
+            # replace_rows (list of matrix numbers): the caller knows these matrices to be of low numerical rank (their
+            # last updates ended in the replacing sweep).  Their replacing sweep -- a chain of some three hundred small
+            # launches whatever the number of matrices -- starts now, on side_stream, next to the sweep of the whole
+            # stack, instead of after the test and two stuck rounds; check() puts its result in their place.
+            if replace_rows and not replace_first:
+                rows = torch.as_tensor(sorted(set(int(r) for r in replace_rows)), dtype=torch.int64).to(Y.device)
+                sub = self.Q.index_select(0, rows)
+                sub_info = torch.zeros(rows.numel(), dtype=torch.int32, device=Y.device)
+                done = None
+                if side_stream is not None:
+                    side_stream.wait_stream(torch.cuda.current_stream(Y.device))
+                    with torch.cuda.stream(side_stream):
+                        block_gram_schmidt(sub, sub_info, pivot_floor, replace_dependent=True)
+                        done = torch.cuda.Event()
+                        done.record(side_stream)
+                else:
+                    block_gram_schmidt(sub, sub_info, pivot_floor, replace_dependent=True)
+                self.presweep = (rows, sub, done, sub_info)
             block_gram_schmidt(self.Q, self.info, pivot_floor, replace_dependent=replace_first)
             if replace_first:
                 self.mended[:] = True
@@ -650,6 +671,14 @@ class CholeskyQR:
     def check(self):
         if self.swept:
             self.swept = False
+            if self.presweep is not None:
+                rows, sub, done, _ = self.presweep
+                if done is not None:
+                    torch.cuda.current_stream(self.Q.device).wait_event(done)
+                self.Q.index_copy_(0, rows, sub)
+                self.info.index_fill_(0, rows, 4)                               # (stand-in columns: tested and polished like the others)
+                self.mended[rows.cpu().numpy()] = True
+                self.presweep = None
             clean = self.info.cpu().numpy() == 0                                # (a host synchronisation)
             # the clean matrices are final where they are; only the flagged ones are copied out into a working
             # set of their own and written back when they are done
@@ -674,6 +703,7 @@ class CholeskyQR:
         block_gram_schmidt(again, info, self.pivot_floor, replace_dependent=True)
         self.Q.index_copy_(0, self._index(where), again)
         self.repairs += int(where.size)
+        self.repaired_ids += [int(i) for i in self.ids[where]]
 
     def _failures(self):
         """Host mask over the entries of the last round: the factorisation met a NaN."""
