@@ -186,6 +186,33 @@ def precond_step_gpu(torch, variant="shampoo1"):
     }
 
 
+def per_parameter_layer_gpu(torch, variant="shampoo2", steps=12):
+    """The literal drop-in (fused=False: one Preconditioner object per parameter, the reference's own control flow)
+    over ONE transformer layer of the ViT-B/32 (qkv, proj, fc1, fc2), same settings as the full step: ms per step.
+    Every product of it runs on the library's matrix-core kernels; profile this section to see which kernels it uses."""
+    import importlib
+    S = importlib.import_module("optimizers." + variant)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    params = [torch.nn.Parameter(0.02 * torch.randn(s, device="cuda", generator=g)) for s in LAYER_SHAPES]
+    grads = [0.02 * torch.randn(p.shape, device="cuda", generator=g) for p in params]
+    extra = dict(inv_root_mode=1) if variant == "shampoo2" else {}
+    opt = S.ShampooAdamW(params, lr=1e-3, weight_decay=0.05, start_prec_step=1, stat_compute_steps=1,
+                         prec_compute_steps=10, fused=False, **STEP_KW, **extra)
+    times = []
+    for i in range(1, steps + 1):
+        for p, gr in zip(params, grads):
+            p.grad = gr.clone()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        opt.step()
+        torch.cuda.synchronize()
+        times.append((i, (time.perf_counter() - t0) * 1e3))
+    regular = [t for i, t in times if i % 10 != 0 and i > 2]
+    return {"workload": "optimizers.%s.ShampooAdamW(fused=False) over one ViT-B/32 layer (4 parameters, 10 blocks, 20 statistics)" % variant,
+            "ms_per_step_regular": round(sum(regular) / len(regular), 3),
+            "ms_per_step_with_inverse_roots": round(sum(t for i, t in times if i % 10 == 0) / max(1, sum(1 for i, _ in times if i % 10 == 0)), 3)}
+
+
 FP32_MATRIX_PEAK_TFLOPS = 157.3
 BF16_MATRIX_PEAK_TFLOPS = 2500.0
 SPLIT_PRODUCTS = 6            # bf16 products that make one fp32 product on the split pipe
@@ -412,7 +439,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--section", choices=["all", "quant", "gemm", "step", "step2", "product"], default="all",
+    ap.add_argument("--section", choices=["all", "quant", "gemm", "step", "step2", "product", "layer"], default="all",
                     help="run only one part (for profiling one kernel family); the JSON line then lacks the others")
     ap.add_argument("--bank-streams", type=int, default=None,
                     help="side streams of the batched preconditioner engine (0 serialises its launches, which "
@@ -448,8 +475,10 @@ def main():
         if args.bank_streams == 0:           # profiling: nothing may overlap, the side thread of shampoo2 neither
             from optimizers import shampoo2
             shampoo2.ShampooAdamW.overlap_precondition = False
-    if args.section in ("gemm", "step", "step2", "product"):
-        if args.section == "gemm":
+    if args.section in ("gemm", "step", "step2", "product", "layer"):
+        if args.section == "layer":
+            part = {"per_parameter_layer": per_parameter_layer_gpu(torch)}
+        elif args.section == "gemm":
             part = {"fused_gemm": fused_gemm_gpu(torch, code)}
         elif args.section == "step":
             part = {"precond_step_naive": precond_step_gpu(torch)}

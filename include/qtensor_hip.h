@@ -322,6 +322,11 @@ void qtensor_hip_copy_flagged_batched(float *dst, const float *src, const int *f
 void qtensor_hip_solve_upper_right_batched(const float *q, const float *u, float *x, float *work, float *out,
                                            int rows, int n, int batch, qtensor_stream_t stream);
 
+/* out[b] = a[b] v[b] for a stack a [batch, n, n] of fp32 matrices and vectors v, out [batch, n], in one launch and a
+ * fixed summation order: the matrix-vector product of the power iteration that scales the ridge term of the inverse
+ * roots (torch.mv per matrix and round in the reference: optimizers/matrix_functions.py:42). */
+void qtensor_hip_matvec_batched(const float *a, const float *v, float *out, int n, int batch, qtensor_stream_t stream);
+
 /* ---- the elementwise end of an optimizer step for all parameters at once -------------------------
  * Replaces the per-parameter torch calls of the reference's step():
  *   grafting   direction.mul_(grad.norm() / (direction.norm() + 1e-12))   optimizers/shampoo1.py:421, shampoo2.py:453

@@ -96,6 +96,7 @@ def PowerIterBatched(mats, error_tolerance=1e-6, num_iters=10, v0=None):
     """PowerIter for a stack [B, n, n]; every matrix follows its own stopping rule (entries that
     have converged are frozen).  v0: optional [B, n] or [n] start vectors.  Returns the [B]
     eigenvalue estimates.  No host synchronisation."""
+    from qtensor import fused as X
     B, n, _ = mats.shape
     if v0 is None:
         v = torch.rand(B, n, device=mats.device) * 2 - 1
@@ -103,10 +104,11 @@ def PowerIterBatched(mats, error_tolerance=1e-6, num_iters=10, v0=None):
         v = v0.to(mats.device).expand(B, n).clone()
     value = torch.zeros(B, device=mats.device)
     change = torch.ones(B, device=mats.device)
+    own = X.on_matrix_cores(mats) and mats.is_contiguous()          # the stack-wide matrix-vector kernel of the library
     for _ in range(num_iters):
         active = change > error_tolerance
         u = v / torch.linalg.vector_norm(v, dim=1, keepdim=True)
-        w = torch.bmm(mats, u.unsqueeze(2)).squeeze(2)
+        w = X.matvec(mats, u.contiguous()) if own else torch.bmm(mats, u.unsqueeze(2)).squeeze(2)
         quotient = (u * w).sum(dim=1)
         change = torch.where(active, (quotient - value).abs(), change)
         value = torch.where(active, quotient, value)

@@ -7,7 +7,7 @@ Preconditioner, ShampooSGD, ShampooAdamW, CODE.
 import torch
 
 from optimizers.shampoo_common import (CODE, BlockPartitioner, PreconditionerBase, ShampooAdamWBase, ShampooSGDBase,
-                                       _DOC, _fusable, dense_gram, newton_inverse_root)
+                                       _DOC, _fusable, decay_and_add_gram, newton_inverse_root)
 from optimizers.fused_step import _FusedStep, _adamw_update, _sgd_update
 from qtensor.utils import QTensorDiagReal
 
@@ -32,7 +32,7 @@ class Preconditioner(PreconditionerBase):
             holder.quantize(X.gram(block, axis, stat=X.Quantized.from_holder(holder), beta=w1, alpha=w2))
             return
         stat = holder.dequantize()          # a dense holder hands out its own tensor: updated in place
-        stat.mul_(w1).add_(dense_gram(block, axis), alpha=w2)
+        decay_and_add_gram(stat, block, axis, w1, w2)
         holder.quantize(stat)
 
     def _inverse_root(self, holder, exp, eps):

@@ -10,7 +10,7 @@ import itertools
 import torch
 
 from optimizers.shampoo_common import (CODE, BlockPartitioner, PreconditionerBase, ShampooAdamWBase, ShampooSGDBase,
-                                       _DOC, dense_gram, newton_inverse_root)
+                                       _DOC, decay_and_add_gram, newton_inverse_root)
 from optimizers.fused_step import _FusedStep, _adamw_update, _sgd_update
 from qtensor.utils import QTensorSVDFast
 
@@ -42,7 +42,7 @@ class Preconditioner(PreconditionerBase):
         # rebuild L from the kept eigenpairs, decay, add the Gram matrix, re-diagonalise
         # (reference: shampoo2.py:185-200)
         stat, basis = holder.dequantize()
-        stat.mul_(w1).add_(dense_gram(block, axis), alpha=w2)
+        decay_and_add_gram(stat, block, axis, w1, w2)
         holder.quantize(stat, basis)
 
     def _inverse_root(self, holder, exp, eps):

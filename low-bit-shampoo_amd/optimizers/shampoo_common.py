@@ -168,7 +168,11 @@ class PreconditionerBase:
             out = block
             for j in range(block.dim()):
                 P = factors[j].dequantize().to(block.dtype)
-                out = out @ P if j == 1 else P @ out
+                if block.dim() == 2 and _own_products(P, out):
+                    from qtensor import fused as X
+                    out = X.gemm(out, P) if j == 1 else X.gemm(P, out)
+                else:
+                    out = out @ P if j == 1 else P @ out
             outs.append(out)
         return torch.reshape(self._partitioner.merge_partitions(outs), self._original_shape)
 
@@ -194,8 +198,26 @@ class PreconditionerBase:
             holder.load_state_dict(one)
 
 
+def _own_products(*tensors) -> bool:
+    """fp32 GPU matrices go through the library's matrix-core products instead of torch's."""
+    from qtensor import fused as X
+    return all(t.dim() == 2 for t in tensors) and X.on_matrix_cores(*tensors)
+
+
 def dense_gram(block, axis):
+    if _own_products(block):
+        from qtensor import fused as X
+        return X.gram(block, 0 if axis == 0 else 1)
     return block.T @ block if axis == 1 else block @ block.T
+
+
+def decay_and_add_gram(stat, block, axis, w1, w2):
+    """stat <- w1 * stat + w2 * (block block^T or block^T block), in place (reference: tensor.mul_(w1).add_(gram, alpha=w2),
+    optimizers/shampoo1.py:164-178); one launch on the matrix cores for fp32 GPU matrices."""
+    if _own_products(block, stat):
+        from qtensor import fused as X
+        return X.gram(block, 0 if axis == 0 else 1, stat=stat, beta=w1, alpha=w2, out=stat)
+    return stat.mul_(w1).add_(dense_gram(block, axis), alpha=w2)
 
 
 def newton_inverse_root(mat, exp, eps, v0=None):

@@ -293,8 +293,15 @@ def compute_power(Vt, S, p, iter_count=4, ridge_epsilon=1e-6, indices=None, max_
     Bjorck orthonormalisation steps V <- 1.5 V - 0.5 V V^T V; rho = ridge_epsilon times
     max_eigen (or max S) (reference :749-762)."""
     V = Vt if indices is None else Vt[indices]
-    for _ in range(iter_count):
-        V = 1.5 * V - 0.5 * V @ V.T @ V
     top = S.max() if max_eigen is None else max_eigen
     weights = 1 / (S + ridge_epsilon * top).pow(1 / p)
+    from qtensor import fused as X
+    if X.on_matrix_cores(V) and V.dim() == 2:
+        # the same products on the matrix cores (Gram matrices computed as half products and mirrored)
+        V = V.contiguous()
+        for _ in range(iter_count):
+            V = X.gemm(X.gemm(V, V, trans_b=True, symmetric=True), V, addend=V, alpha=-0.5, beta=1.5)
+        return X.gemm(V * weights.to(V.dtype).unsqueeze(1), V, trans_a=True, symmetric=True)
+    for _ in range(iter_count):
+        V = 1.5 * V - 0.5 * V @ V.T @ V
     return V.T @ weights.diag() @ V

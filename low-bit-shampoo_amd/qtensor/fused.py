@@ -289,6 +289,28 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
     return addend if requantize else out
 
 
+def on_matrix_cores(*tensors) -> bool:
+    """Whether a product of these tensors can go through gemm(): fp32 GPU tensors with a contiguous last dimension
+    (and the library there)."""
+    return F.lib is not None and all(t.is_cuda and t.dtype == torch.float32 and t.dim() in (2, 3) and t.stride(-1) == 1
+                                     and t.numel() > 0 for t in tensors)
+
+
+if F.lib is not None:
+    F.lib.qtensor_hip_matvec_batched.restype = None
+    F.lib.qtensor_hip_matvec_batched.argtypes = [ct.c_void_p, ct.c_void_p, ct.c_void_p, ct.c_int, ct.c_int, ct.c_void_p]
+
+
+def matvec(mats: Tensor, v: Tensor) -> Tensor:
+    """[B, n]: mats[b] @ v[b] for a contiguous fp32 GPU stack [B, n, n] and vectors [B, n], one launch, fixed
+    summation order (the reference: torch.mv per matrix, optimizers/matrix_functions.py:42)."""
+    B, n, _ = mats.shape
+    _stack(mats, "mats", (B, n, n)), _stack(v, "v", (B, n))
+    out = torch.empty(B, n, device=mats.device)
+    F._call(F.lib.qtensor_hip_matvec_batched, mats.device, mats.data_ptr(), v.data_ptr(), out.data_ptr(), n, B)
+    return out
+
+
 def precondition(G: Tensor, left, right, out: Optional[Tensor] = None) -> Tensor:
     """deq(left) @ G @ deq(right) with both factors expanded inside the products.
     left / right: `Quantized` or dense fp32 matrices."""

@@ -210,8 +210,14 @@ class QTensorSVDFast(_LowBitState):
         """One subspace-iteration step: orthonormalise L Vt^T by QR, take Rayleigh quotients,
         remember the smaller half, store the new basis (as rows)."""
         L = var.float()
-        V = _orthonormal_basis(L @ Vt.T.float())
-        quotients = (V.T @ L @ V).diag()
+        from qtensor import fused
+        if fused.on_matrix_cores(L, Vt) and L.dim() == 2:
+            # the same products on the matrix cores; the Rayleigh quotients diag(V^T (L V)) without the product
+            V = _orthonormal_basis(fused.gemm(L, Vt, trans_b=True))
+            quotients = (V * fused.gemm(L, V.contiguous())).sum(dim=0)
+        else:
+            V = _orthonormal_basis(L @ Vt.T.float())
+            quotients = (V.T @ L @ V).diag()
 
         keep = max(1, quotients.numel() // 2)
         ascending, where = torch.sort(quotients)
@@ -246,14 +252,21 @@ class QTensorSVDFast(_LowBitState):
 
     def dequantize(self):
         """Returns (V_keep^T diag(Svalue) V_keep, Vt)."""
+        from qtensor import fused
         if self.bits < 16:
             Vt = self._basis()
+            own = fused.on_matrix_cores(Vt)
             for _ in range(self.rect_t1):
-                Vt = 1.5 * Vt - 0.5 * Vt @ Vt.T @ Vt
+                if own:
+                    Vt = fused.gemm(fused.gemm(Vt, Vt, trans_b=True, symmetric=True), Vt, addend=Vt, alpha=-0.5, beta=1.5)
+                else:
+                    Vt = 1.5 * Vt - 0.5 * Vt @ Vt.T @ Vt
         else:
             Vt = self.var
         rows = Vt[self.keep_indices.to(device=Vt.device)]
         weights = self.Svalue.to(device=Vt.device, dtype=Vt.dtype)
+        if fused.on_matrix_cores(rows):
+            return fused.gemm(rows * weights.unsqueeze(1), rows, trans_a=True, symmetric=True), Vt
         return rows.T @ weights.diag() @ rows, Vt
 
     def computepower(self, exp, ridge_epsilon=1e-6):

@@ -86,3 +86,20 @@ def test_ill_conditioned_inverse_roots_are_as_good_as_the_cpu_iteration(n, cond)
         print(f"n {n} cond 1e{cond:.0f}: error of the CPU fp32 iteration {e_cpu:.2e}, of the GPU {e_gpu:.2e}, apart {apart:.2e}")
         assert e_gpu <= 2 * e_cpu + 1e-5, (n, cond, b, e_cpu, e_gpu)
         assert apart <= 5e-5, (n, cond, b, apart)
+
+
+@pytest.mark.parametrize("n,batch", [(64, 3), (100, 2), (1024, 5), (1500, 1), (7, 4)])
+def test_stack_matrix_vector_product(n, batch):
+    """The library's matrix-vector product for a whole stack (the power iteration's only product) against float64."""
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(n)
+    mats, v = torch.randn(batch, n, n, generator=g), torch.randn(batch, n, generator=g)
+    got = X.matvec(mats.cuda(), v.cuda())
+    want = torch.bmm(mats.double(), v.double().unsqueeze(2)).squeeze(2)
+    scale = torch.bmm(mats.double().abs(), v.double().abs().unsqueeze(2)).squeeze(2)
+    assert got.shape == (batch, n)
+    assert float(((got.cpu().double() - want).abs() / scale).max()) <= 1e-6
+    assert torch.equal(got, X.matvec(mats.cuda(), v.cuda()))                   # fixed summation order
+    view = torch.zeros(batch, n, n + 4, device="cuda")[:, :, 1:n + 1]            # not contiguous: refused
+    with pytest.raises(ValueError):
+        X.matvec(view, v.cuda())
