@@ -142,11 +142,14 @@ def precond_step_gpu(torch, variant="shampoo1"):
         timed_step()
     torch.cuda.synchronize()
     resident = torch.cuda.memory_allocated()             # parameters, four gradient sets, optimizer state, kept scratch
-    torch.cuda.reset_peak_memory_stats()
     regular, newton = [], []
+    peak = {"regular": 0, "roots": 0}
     for i in range(11, 31):
+        torch.cuda.reset_peak_memory_stats()
         wall, dev = timed_step()
         (newton if i % 10 == 0 else regular).append((wall, dev))
+        kind = "roots" if i % 10 == 0 else "regular"
+        peak[kind] = max(peak[kind], torch.cuda.max_memory_allocated())
     mean = lambda xs, k: sum(x[k] for x in xs) / len(xs)          # noqa: E731
     reg, new = mean(regular, 0), mean(newton, 0)
     blocks = sum(((m - 1) // 1024 + 1) * ((n - 1) // 1024 + 1) for m, n in vit_b32_shapes())
@@ -179,7 +182,9 @@ def precond_step_gpu(torch, variant="shampoo1"):
         "device_ms_regular": round(mean(regular, 1), 3),
         "device_ms_with_inverse_roots": round(mean(newton, 1), 3),
         "device_memory_gib": {"allocated_between_steps": round(resident / 2 ** 30, 2),
-                              "peak_inside_a_step": round(torch.cuda.max_memory_allocated() / 2 ** 30, 2),
+                              "peak_inside_a_step": round(max(peak.values()) / 2 ** 30, 2),
+                              "peak_inside_a_regular_step": round(peak["regular"] / 2 ** 30, 2),
+                              "peak_inside_a_step_with_inverse_roots": round(peak["roots"] / 2 ** 30, 2),
                               "of_which_parameters_and_the_four_gradient_sets": round(5 * sum(p.numel() for p in params) * 4 / 2 ** 30, 2)},
         "product_gflop_per_regular_step": round(2 * gram_flop / 1e9, 1),
         "product_tflops_regular": round(2 * gram_flop / (mean(regular, 1) * 1e-3) / 1e12, 1),
@@ -446,7 +451,6 @@ def main():
                          "keeps per-kernel durations in a profile free of overlap)")
     ap.add_argument("--gemm-pipe", choices=["f32", "split"], default=None,
                     help="matrix pipe of the products of dense operands (default: the library's, the split bf16 pipe)")
-    ap.add_argument("--probe-queues", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--no-step", action="store_true", help="skip the fused-product, other-format and Shampoo-step measurements")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -465,9 +469,6 @@ def main():
     if args.gemm_pipe is not None:
         import qtensor.fused as X
         X.gemm_pipe(args.gemm_pipe)
-    if args.probe_queues:
-        import optimizers.engine as E
-        E.PROBE_QUEUES = True
     if args.bank_streams is not None:
         from optimizers.engine import ShampooBank
         from optimizers.engine2 import ShampooBank2

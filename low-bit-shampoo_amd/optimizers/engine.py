@@ -48,121 +48,20 @@ class _Group:
 
 _SHARED_STREAMS = {}
 LANES = 2                                            # chains of launches the eigenbasis bank runs side by side
-BESIDE_SLOT, UNBATCHED_SLOT = 9, 10                  # fixed places in the pool, behind the fan-out streams (at most 8)
-
-
-def _same_queue(a, b, scratch):
-    """Whether work on stream b waits for work on stream a: a spins for a while, b gets one tiny launch.  (Twice: a
-    launch that the host is slow to make -- the first one of a kind -- looks like one that waited.)"""
-    waited = True
-    for _ in range(2):
-        torch.cuda.synchronize(scratch.device)
-        start, end_a, end_b = (torch.cuda.Event(enable_timing=True) for _ in range(3))
-        with torch.cuda.stream(a):
-            start.record()
-            torch.cuda._sleep(1_000_000)
-            end_a.record()
-        with torch.cuda.stream(b):
-            scratch.add_(1)
-            end_b.record()
-        torch.cuda.synchronize(scratch.device)
-        waited = waited and start.elapsed_time(end_b) > 0.5 * start.elapsed_time(end_a)
-    return waited
-
-
-PROBE_QUEUES = False                                 # True: _build_pool sorts the streams by hardware queue (see there)
-
-
-def _plain_pool(index):
-    """A dozen side streams of the device as they come."""
-    device = torch.device("cuda", index)
-    with torch.cuda.device(device):
-        made = [torch.cuda.Stream(device=device) for _ in range(12)]
-    pool = {i: made[i] for i in range(12)}
-    pool["spare"] = made
-    return pool
-
-
-def _build_pool(index):
-    """The side streams of a device, by role.  A process has few hardware queues (four by default) and every stream
-    is bound to one of them when it is first used, in turn; streams on one queue run their launches in the order in
-    which the host made them.  Which of the bank's chains share a queue decides a fifth of the step time (22.3 ms
-    when the two sweep lanes, the parameters outside the bank and the current stream have a queue each, 26.5-27.5
-    when an application that made a stream or three of its own first shifts the turn), so the pool does not take
-    streams as they come: it makes a dozen, lets each one run something once (that binds it), finds out with a
-    spinning kernel which of them wait for each other, and hands them out by queue:
-      slot 0               the current stream's queue        (first lane of the sweeps; first stream of every fan-out)
-      slots 1, 2           a second queue                    (second lane; fan-outs)
-      slot 3, BESIDE_SLOT  a third queue                     (the job that applies the stored roots; fan-outs)
-      UNBATCHED_SLOT       the fourth queue                  (parameters outside the bank, on a thread)
-      every other slot     the current stream's queue"""
-    device = torch.device("cuda", index)
-    with torch.cuda.device(device):
-        current = torch.cuda.current_stream(device)
-        made = [torch.cuda.Stream(device=device) for _ in range(12)]
-        scratch = torch.zeros(64, device=device)
-        groups = [[current]]                                   # streams by hardware queue; the first group is the current stream's
-        if hasattr(torch.cuda, "_sleep"):
-            torch.cuda._sleep(1000)
-            for stream in made:
-                with torch.cuda.stream(stream):
-                    scratch.add_(1)
-            for stream in made:
-                for group in groups:
-                    if _same_queue(group[0], stream, scratch):
-                        group.append(stream)
-                        break
-                else:
-                    groups.append([stream])
-            torch.cuda.synchronize(device)
-        else:
-            groups += [[stream] for stream in made]            # no way to tell: as they come
-    own, others = groups[0][1:], [g for g in groups[1:] if g]
-    # the queues in the order of their turn, starting behind the current stream's: streams are bound in turn, so the
-    # queue of the stream made right after one of the current stream's queue is the next one, whatever else the
-    # process has bound before
-    if len(groups) > 1 and own:
-        turn = []
-        at = made.index(own[0])
-        for stream in made[at + 1:] + made[:at]:
-            group = next(g for g in groups if stream in g)
-            if group is not groups[0] and group not in turn:
-                turn.append(group)
-        others = turn + [g for g in others if g not in turn]
-    # Who may share a queue.  A stream that is told to wait for another one blocks its whole queue until then: the
-    # launches that other streams on that queue make in the meantime wait with it.  So
-    #   the job that applies the stored roots (made early, waits for the end of all sweeps) gets a queue to itself;
-    #   the thread of the parameters outside the bank (a long chain of small launches) gets one to itself: product
-    #     launches of a fan-out behind that chain would hold up a whole phase (22 -> 26.8 ms per step);
-    #   the second lane shares its queue only with a fan-out stream of the phases before the sweeps;
-    #   the first lane shares the current stream's queue: the current stream does little but wait, and what it waits
-    #     for is queued ahead of its barriers.
-    # (This is the arrangement a fresh process happens to get from streams taken in turn, 22.0 ms per step; the
-    # other ways round that were tried cost 1 to 5 ms.)
-    spare = own[1:] + [s for g in others for s in g[2:]]
-    if not spare:
-        spare = own or [g[0] for g in others] or made
-    pick = lambda k, j, fallback: others[k][j] if len(others) > k and len(others[k]) > j else fallback      # noqa: E731
-    pool = {0: own[0] if own else pick(0, 0, made[0])}
-    pool[1] = pick(0, 0, spare[0])
-    pool[2] = pick(0, 1, spare[0])
-    pool[3] = pool[BESIDE_SLOT] = pick(1, 0, spare[-1])
-    pool[UNBATCHED_SLOT] = pick(2, 0, spare[-1])
-    pool["spare"] = spare
-    return pool
+BESIDE_SLOT = 9                                      # a stream no fan-out uses (at most 8 of those): work next to the sweeps
 
 
 def shared_stream(device, slot):
-    """Side stream number `slot` of the device, the same object for every bank and optimizer of the process
-    (see _build_pool for which slot is what)."""
+    """Side stream number `slot` of the device, the same object for every bank and optimizer of the process (a
+    second optimizer with streams of its own would double the chains that compete for the device's few hardware
+    queues).  A dozen plain streams of default priority per device, made together on first use."""
     device = torch.device(device)
     index = device.index if device.index is not None else torch.cuda.current_device()
     if index not in _SHARED_STREAMS:
-        _SHARED_STREAMS[index] = _build_pool(index) if PROBE_QUEUES else _plain_pool(index)
+        with torch.cuda.device(index):
+            _SHARED_STREAMS[index] = [torch.cuda.Stream(device=index) for _ in range(12)]
     pool = _SHARED_STREAMS[index]
-    if slot not in pool:
-        pool[slot] = pool["spare"][slot % len(pool["spare"])]
-    return pool[slot]
+    return pool[slot % len(pool)]
 
 
 class SideJob:
@@ -410,6 +309,24 @@ class ShampooBank:
         for g in self.groups:
             self._grad_list(g, grads)
 
+    # The coupled Newton iteration holds ten fp32 stacks of what it works on (two copies each of the root, the
+    # iterate and the iteration matrix, two powers, the input, the result): a stack goes through it in parts of
+    # at most this many bytes, one after the other, so that the iteration of a whole model takes ten times this
+    # much scratch and not ten times its largest stack (ViT-B/32: 70.1 ms per step with inverse roots and 1.8 GiB of
+    # scratch, against 68.8 ms and 4.2 GiB with whole stacks).  (A part still is dozens of matrices: every product launch
+    # has thousands of tiles; the bits of a matrix's root do not depend on how its stack is cut.)
+    NEWTON_PART_BYTES = 160 << 20
+    NEWTON_SIDE_BY_SIDE = True                   # the orders' iterations run side by side on the side streams (False: one after the other)
+
+    def _newton_parts(self, order, rows):
+        """The stack of this order in parts for the Newton iteration: (first, count) ranges of the whole stack
+        (rows None), else pieces of the int64 vector of rows."""
+        per = max(1, self.NEWTON_PART_BYTES // (4 * order * order))
+        if rows is None:
+            count = self.per_order[order]
+            return [(first, min(per, count - first)) for first in range(0, count, per)]
+        return list(rows.split(per))
+
     # ---- the three operations of the reference's Preconditioner, for all parameters at once ------
     @torch.no_grad()
     def add_statistics(self, grads, only=None):
@@ -462,25 +379,30 @@ class ShampooBank:
         def job(order):
             def run():
                 rows = self._rows(order, only)
-                stat = self.stats[order] if rows is None else self.stats[order].select(rows)
-                start = starts[order] if rows is None else starts[order].index_select(0, rows)
-                # (an fp32 statistic is handed over as it is and keeps the ridge that the iteration adds in
-                # place, as in the reference: optimizers/shampoo1.py:198)
-                dense = X.load_stack(stat)
-                roots = ComputePowerBatched(dense, 4, ridge_epsilon=self.matrix_eps, v0=start)
-                if rows is None:
-                    X.store_stack(roots, self.precs[order])
-                else:
-                    if isinstance(stat, X.DenseStack):
-                        self.stats[order].put(rows, stat)
-                    self.precs[order].put(rows, X.store_stack(roots, self.precs[order].select(rows)))
+                for part in self._newton_parts(order, rows):
+                    if rows is None:
+                        first, count = part
+                        stat, target = self.stats[order].rows(first, count), self.precs[order].rows(first, count)
+                        start = starts[order][first:first + count]
+                    else:
+                        stat, target = self.stats[order].select(part), self.precs[order].select(part)
+                        start = starts[order].index_select(0, part)
+                    # (an fp32 statistic is handed over as it is and keeps the ridge that the iteration adds in
+                    # place, as in the reference: optimizers/shampoo1.py:198)
+                    dense = X.load_stack(stat)
+                    roots = ComputePowerBatched(dense, 4, ridge_epsilon=self.matrix_eps, v0=start)
+                    X.store_stack(roots, target)
+                    if rows is not None:
+                        if isinstance(stat, X.DenseStack):
+                            self.stats[order].put(part, stat)
+                        self.precs[order].put(part, target)
             return run
 
         # start vectors come from the global generator in a fixed order, whatever the streams do
         starts = {order: (torch.rand(stat.batch, order, device=self.device) * 2 - 1) if v0 is None else v0[order]
                   for order, stat in self.stats.items()}
         orders = [o for o in sorted(self.stats, key=lambda o: -o ** 3 * self.stats[o].batch) if self._touched(o, only)]
-        self._fan_out([job(order) for order in orders])
+        self._fan_out([job(order) for order in orders], inline=not self.NEWTON_SIDE_BY_SIDE)
         for pi in range(len(self.params)):
             if only is None or pi in only:
                 self.active[pi] = True

@@ -49,6 +49,7 @@ class ShampooBank2(ShampooBank):
         self.low_rank_rows = {}                   # order -> {row: [updates between two looks at the plain sweep, updates until the next look]}
         super().__init__(params, name2qmap, code, **kwargs)
 
+    QUOTIENT_PART_BYTES = 128 << 20               # L Q for the Rayleigh quotients is formed this much at a time
     LOOK_AGAIN = 8                                # updates after which a stack of low numerical rank tries the plain sweep again
     STALL_SECONDS = 300.0                         # the host polls the device while the stacks are factored: not for ever
 
@@ -64,18 +65,20 @@ class ShampooBank2(ShampooBank):
             return False
         return True
 
-    REPAIR_SLOT = 5                               # side stream of the replacing sweeps that start next to a stack's own sweep
-
-    def _presweep_rows(self, order):
-        """The matrices of this stack whose replacing sweep starts right away: those whose recent updates ended in it.
-        Every `period` updates such a matrix gets the plain sweep alone again; a period doubles (8, 16, ... 256) each
-        time that look ends in the replacing sweep once more."""
-        rows = []
-        for row, state in self.low_rank_rows.setdefault(order, {}).items():
+    def _known_low_rank(self, order):
+        """How many matrices of this stack are, for this update, taken to be of low numerical rank: those whose recent
+        updates ended in the replacing sweep (the order-768 statistic of a 768 x 100 head: rank 100 plus the kept half).
+        A stack that holds one starts with the replacing sweep -- three passes instead of two for the whole stack, less
+        than the chain of some three hundred small launches that sweeping the one matrix again costs behind two stuck
+        polishing rounds (ViT-B/32: 23.2 ms per regular step, every step alike, against 21.5 to 26.5).  Every `period`
+        updates the stack gets the plain sweep again; the period doubles (8, 16, ... 256) each time that look ends in
+        the replacing sweep once more."""
+        known = 0
+        for state in self.low_rank_rows.setdefault(order, {}).values():
             if state[1] > 0:
                 state[1] -= 1
-                rows.append(row)
-        return rows
+                known += 1
+        return known
 
     def _note_repairs(self, order, repaired):
         table = self.low_rank_rows.setdefault(order, {})
@@ -150,6 +153,10 @@ class ShampooBank2(ShampooBank):
         for g in self.groups:
             self._grad_list(g, grads)
 
+        solver, redone, tick = {}, {}, {}
+        # (a stack starts with the replacing sweep when most of it needed that sweep lately, or when it holds a matrix that did)
+        direct = {o: bool(self._replace_first(o) + self._known_low_rank(o)) for o in orders}
+
         def rebuild(order):
             def run():
                 basis[order] = self._rectified_basis(order)
@@ -167,8 +174,19 @@ class ShampooBank2(ShampooBank):
 
         def project(order):
             def run():
-                solver[order] = X.CholeskyQR(X.gemm(stat[order], basis[order], trans_b=True), replace_first=direct[order],
-                                             replace_rows=early[order], side_stream=shared_stream(self.device, self.REPAIR_SLOT))     # L Vt^T
+                # L Vt^T.  The product is given up to the solver (scaled in place, it becomes Q) and the rectified basis
+                # is let go right here: from now on a stack holds its statistic and Q.  The few matrices whose columns
+                # are needed once more (low numerical rank: swept again from the original columns) are made anew.
+                def remake(ids):
+                    return X.gemm(stat[order].index_select(0, ids), self._rectified_basis(order, ids), trans_b=True)
+
+                product = X.gemm(stat[order], basis[order], trans_b=True)
+                # (the rectified basis came from another stream's job: its memory must not be handed out again on that
+                # stream before this one has read it)
+                basis[order].record_stream(torch.cuda.current_stream(self.device))
+                basis[order] = None
+                solver[order] = X.CholeskyQR(product, replace_first=direct[order], remake=remake)
+                del product
                 # (the event that tells the host this stack's sweep is through goes right behind it: streams share
                 # hardware queues, and behind the launches of another stack's sweep it would wait for those as well)
                 tick[order] = torch.cuda.Event()
@@ -179,8 +197,14 @@ class ShampooBank2(ShampooBank):
             def run():
                 L = stat[order]
                 Q, redone[order] = solver[order].result()
-                LQ = X.gemm(L, Q)
-                quotients = X.column_dots(Q, LQ) if Q.shape[1] % 64 == 0 else (Q * LQ).sum(dim=1)      # diag(Q^T L Q)
+                # Rayleigh quotients diag(Q^T L Q), the product L Q a few dozen matrices at a time
+                quotients = torch.empty(Q.shape[0], Q.shape[1], device=self.device)
+                per = max(1, self.QUOTIENT_PART_BYTES // (4 * order * order))
+                for first in range(0, Q.shape[0], per):
+                    q = Q[first:first + per]
+                    lq = X.gemm(L[first:first + per], q)
+                    quotients[first:first + per] = X.column_dots(q, lq) if order % 64 == 0 else (q * lq).sum(dim=1)
+                del lq
                 ascending, where = torch.sort(quotients, dim=1)
                 half = self.keep[order].shape[1]
                 rows = self._rows(order, only)
@@ -202,9 +226,6 @@ class ShampooBank2(ShampooBank):
                        if only is None or any(pi in only for pi in g.param_index)])
         # The Cholesky QR of every order advances on its own stream; the host waits once per round.
         # (_fan_out gives job i the stream i % streams, so an order keeps its stream from call to call.)
-        solver, redone, tick = {}, {}, {}
-        direct = {o: self._replace_first(o) for o in orders}
-        early = {o: self._presweep_rows(o) for o in orders}
         # Two lanes for the sweeps and what follows them: a process has four hardware queues, the parameters outside
         # the bank and the job that applies the stored roots take one each, and streams beyond that share a queue in
         # the order of their launches -- a third stack on a stream of its own ran behind the second anyway, and held
@@ -297,28 +318,32 @@ class ShampooBank2(ShampooBank):
         def job(order):
             def run():
                 rows = self._rows(order, only)
-                basis, keep, svalue, max_eig = self._pick(order, rows)
-                if self.inv_root_mode == 0:
-                    kept = self._gather_rows(X.load_stack(basis), keep)
-                    if not isinstance(basis, X.DenseStack):              # (a basis held in fp32 is not rectified: utils.py:205-227)
-                        for _ in range(self.rect_t2):
-                            vvt = X.gemm(kept, kept, trans_b=True, symmetric=True)
-                            kept = X.gemm(vvt, kept, addend=kept, alpha=-0.5, beta=1.5)
-                    ridge = self.matrix_eps * max_eig
-                    weights = 1 / (svalue + ridge.unsqueeze(1)).pow(1 / 4)
-                    roots = X.gemm(kept * weights.unsqueeze(2), kept, trans_a=True, symmetric=True)
-                else:
-                    L = self._statistic(order, self._rectified_basis(order, rows), rows=rows)
-                    start = starts[order] if rows is None else starts[order].index_select(0, rows)
-                    # L is symmetric up to the rounding inside its diagonal tiles: half products are fine
-                    roots = ComputePowerBatched(L, 4, ridge_epsilon=self.matrix_eps, v0=start, symmetric=True)
-                if rows is None:
-                    X.store_stack(roots, self.precs[order])
-                else:
-                    self.precs[order].put(rows, X.store_stack(roots, self.precs[order].select(rows)))
+                for part in self._newton_parts(order, rows):
+                    # (a part of the whole stack is gathered like a chosen set of rows: one copy of its 4-bit basis)
+                    index = torch.arange(part[0], part[0] + part[1], device=self.device) if rows is None else part
+                    whole = rows is None and part[1] == self.per_order[order]
+                    basis, keep, svalue, max_eig = self._pick(order, None if whole else index)
+                    if self.inv_root_mode == 0:
+                        kept = self._gather_rows(X.load_stack(basis), keep)
+                        if not isinstance(basis, X.DenseStack):          # (a basis held in fp32 is not rectified: utils.py:205-227)
+                            for _ in range(self.rect_t2):
+                                vvt = X.gemm(kept, kept, trans_b=True, symmetric=True)
+                                kept = X.gemm(vvt, kept, addend=kept, alpha=-0.5, beta=1.5)
+                        ridge = self.matrix_eps * max_eig
+                        weights = 1 / (svalue + ridge.unsqueeze(1)).pow(1 / 4)
+                        roots = X.gemm(kept * weights.unsqueeze(2), kept, trans_a=True, symmetric=True)
+                    else:
+                        L = self._statistic(order, self._rectified_basis(order, None if whole else index), rows=None if whole else index)
+                        start = starts[order] if whole else starts[order].index_select(0, index)
+                        # L is symmetric up to the rounding inside its diagonal tiles: half products are fine
+                        roots = ComputePowerBatched(L, 4, ridge_epsilon=self.matrix_eps, v0=start, symmetric=True)
+                    if rows is None:
+                        X.store_stack(roots, self.precs[order].rows(part[0], part[1]))
+                    else:
+                        self.precs[order].put(index, X.store_stack(roots, self.precs[order].select(index)))
             return run
 
-        self._fan_out([job(o) for o in orders])
+        self._fan_out([job(o) for o in orders], inline=not self.NEWTON_SIDE_BY_SIDE)
         for pi in range(len(self.params)):
             if only is None or pi in only:
                 self.active[pi] = True

@@ -144,15 +144,13 @@ def _dense(t):
     return BatchPtr(t.data_ptr(), None, t.stride(0)), t.stride(1), t.shape[0], t.shape[1], t.shape[2]
 
 
-_WORKSPACE = {}                 # (device index, stream) -> fp32 scratch for products that are split along k
-_WORKSPACE_FLOATS = 1 << 24     # 64 MiB
+_WORKSPACE_FLOATS = 1 << 24     # 64 MiB: the most a product that is cut along k gets for its partial products
 
 
-def _workspace(device: torch.device) -> Tensor:
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
-    if key not in _WORKSPACE:
-        _WORKSPACE[key] = torch.empty(_WORKSPACE_FLOATS, dtype=torch.float32, device=device)
-    return _WORKSPACE[key]
+def _workspace(device: torch.device, floats: int) -> Tensor:
+    """fp32 scratch for one product that may be cut along k: taken from torch's allocator for the call and handed
+    back with it (the allocator keeps it for the stream it was used on), so that nothing is held between steps."""
+    return torch.empty(min(_WORKSPACE_FLOATS, floats), dtype=torch.float32, device=device)
 
 
 def _launch(desc: GemmDesc, device: torch.device) -> None:
@@ -282,9 +280,13 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
             raise ValueError("triangular operands are dense and square, in a product that is not marked symmetric")
         a.triangular = (1 if upper_a else 0) | (2 if upper_b else 0)
     if d.epilogue == EPI_STORE and not symmetric and k >= 256 and batch * m * n <= _WORKSPACE_FLOATS // 2:
-        # few output tiles, long k: the library may cut k into slices (one scratch area per stream)
-        scratch = _workspace(dev)
+        # few output tiles, long k: the library may cut k into up to eight slices per tile, or -- with a quantized
+        # operand -- deal runs of k tiles out over two workgroups per compute unit (a 128 x 128 square per run and tile)
+        tiles = batch * (-(-m // 128)) * (-(-n // 128))
+        quantized = isinstance(A, Quantized) or isinstance(B, Quantized)
+        scratch = _workspace(dev, max(8 * batch * m * n, (tiles + 520) * 128 * 128 if quantized and tiles < 1024 else 0))
         a.workspace, a.workspace_floats = scratch.data_ptr(), scratch.numel()
+        keep.append(scratch)
     _launch(d, dev)
     return addend if requantize else out
 
@@ -603,19 +605,23 @@ class CholeskyQR:
     library).  All calls for one object must be made with the same current stream."""
 
     def __init__(self, Y, max_rounds=12, pivot_floor=PIVOT_FLOOR, tolerance=2e-5, sweep=True, replace_first=False,
-                 replace_rows=None, side_stream=None):
+                 remake=None):
+        """remake: optional callable, int64 GPU vector of matrix numbers -> those matrices of Y again.  With it Y is
+        given up: its columns are scaled in place and it becomes the working set (one stack less held through the
+        sweep); the few matrices whose original columns are needed again (_repair, the library fallback) are made anew."""
         if Y.dim() != 3 or Y.shape[1] != Y.shape[2] or Y.dtype != torch.float32 or not Y.is_cuda:
             raise ValueError("CholeskyQR takes an fp32 GPU stack [B, n, n]")
         B, self.true_n, _ = Y.shape
         n = -(-self.true_n // 64) * 64
+        self.batch, self.n, self.device, self.remake = B, n, Y.device, remake
         if n != self.true_n:
-            padded = torch.zeros(B, n, n, device=Y.device)
-            padded[:, :self.true_n, :self.true_n] = Y
-            padded.diagonal(dim1=1, dim2=2)[:, self.true_n:] = 1.0
-            Y = padded
-        self.Y, self.pivot_floor, self.tolerance, self.rounds_left = Y, pivot_floor, tolerance, max_rounds
+            Y = self._padded(Y)
+        self.pivot_floor, self.tolerance, self.rounds_left = pivot_floor, tolerance, max_rounds
         scale = torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)
-        self.Q = (Y / scale).contiguous()             # working set; unit columns: the Gram matrix has a unit diagonal
+        if remake is not None and Y.is_contiguous():
+            self.Y, self.Q = None, Y.div_(scale)
+        else:
+            self.Y, self.Q = Y, (Y / scale).contiguous()   # working set; unit columns: the Gram matrix has a unit diagonal
         self.U = self.X = None                        # factors of the polishing rounds: allocated for the working set only
         self.info = torch.zeros(B, dtype=torch.int32, device=Y.device)
         self.final = None                             # allocated when the first matrix is done
@@ -624,7 +630,6 @@ class CholeskyQR:
         self.rounds = 0                               # factorisation rounds enqueued so far
         self.repairs = 0                              # matrices swept a second time (see _repair)
         self.repaired_ids = []                        # which matrices of the stack those were
-        self.presweep = None                          # (rows, their replacing sweep's result, event): see replace_rows below
         self.gram = self.far = None
         # The bookkeeping lives on the host (it waits once per round anyway), per working-set entry:
         # which matrix of the stack it is and whether it is within ||G - I||_F < 0.5.
@@ -642,27 +647,23 @@ class CholeskyQR:
             # fp32 rounding by construction; the rounds below are for the other matrices only.
             # replace_first: the caller knows the stack to be of low numerical rank (its last update needed the
             # replacing sweep for most matrices) and goes there directly
-            # replace_rows (list of matrix numbers): the caller knows these matrices to be of low numerical rank (their
-            # last updates ended in the replacing sweep).  Their replacing sweep -- a chain of some three hundred small
-            # launches whatever the number of matrices -- starts now, on side_stream, next to the sweep of the whole
-            # stack, instead of after the test and two stuck rounds; check() puts its result in their place.
-            if replace_rows and not replace_first:
-                rows = torch.as_tensor(sorted(set(int(r) for r in replace_rows)), dtype=torch.int64).to(Y.device)
-                sub = self.Q.index_select(0, rows)
-                sub_info = torch.zeros(rows.numel(), dtype=torch.int32, device=Y.device)
-                done = None
-                if side_stream is not None:
-                    side_stream.wait_stream(torch.cuda.current_stream(Y.device))
-                    with torch.cuda.stream(side_stream):
-                        block_gram_schmidt(sub, sub_info, pivot_floor, replace_dependent=True)
-                        done = torch.cuda.Event()
-                        done.record(side_stream)
-                else:
-                    block_gram_schmidt(sub, sub_info, pivot_floor, replace_dependent=True)
-                self.presweep = (rows, sub, done, sub_info)
             block_gram_schmidt(self.Q, self.info, pivot_floor, replace_dependent=replace_first)
             if replace_first:
                 self.mended[:] = True
+
+    def _padded(self, Y):
+        """Orders that are not a multiple of 64: diag(Y, I)."""
+        padded = torch.zeros(Y.shape[0], self.n, self.n, device=Y.device)
+        padded[:, :self.true_n, :self.true_n] = Y
+        padded.diagonal(dim1=1, dim2=2)[:, self.true_n:] = 1.0
+        return padded
+
+    def _original(self, ids):
+        """The matrices `ids` (int64 GPU vector) of the stack the object was made for."""
+        if self.Y is not None:
+            return self.Y.index_select(0, ids)
+        again = self.remake(ids)
+        return self._padded(again) if self.n != self.true_n else again
 
     def _index(self, positions):
         return torch.as_tensor(np.ascontiguousarray(positions), dtype=torch.int64).to(self.Q.device)
@@ -671,12 +672,12 @@ class CholeskyQR:
         """The working-set entries `where` (host positions) of `source` are final."""
         if where.size == 0:
             return
-        B = self.Y.shape[0]
+        B = self.batch
         if self.final is None and where.size == B and source.shape[0] == B and np.array_equal(self.ids, np.arange(B)):
             self.final = source                       # the whole stack at once: no copy
             return
         if self.final is None:
-            self.final = torch.empty_like(self.Y)
+            self.final = torch.empty(B, self.n, self.n, device=self.device)
         self.final.index_copy_(0, self._index(self.ids[where]), source.index_select(0, self._index(where)))
 
     def _keep(self, keep):
@@ -693,14 +694,6 @@ class CholeskyQR:
     def check(self):
         if self.swept:
             self.swept = False
-            if self.presweep is not None:
-                rows, sub, done, _ = self.presweep
-                if done is not None:
-                    torch.cuda.current_stream(self.Q.device).wait_event(done)
-                self.Q.index_copy_(0, rows, sub)
-                self.info.index_fill_(0, rows, 4)                               # (stand-in columns: tested and polished like the others)
-                self.mended[rows.cpu().numpy()] = True
-                self.presweep = None
             clean = self.info.cpu().numpy() == 0                                # (a host synchronisation)
             # the clean matrices are final where they are; only the flagged ones are copied out into a working
             # set of their own and written back when they are done
@@ -718,7 +711,7 @@ class CholeskyQR:
         cannot mend it (columns end unnormalised or parallel, and Cholesky QR rounds on such a matrix diverge).  They
         are swept again from their original columns, three passes, with every column that a pass finds dependent
         replaced by a stand-in column (block_gram_schmidt(replace_dependent=True))."""
-        original = self.Y.index_select(0, self._index(self.ids[where]))
+        original = self._original(self._index(self.ids[where]))
         scale = torch.linalg.vector_norm(original, dim=1, keepdim=True).clamp_min(1e-30)
         again = (original / scale).contiguous()
         info = torch.zeros(again.shape[0], dtype=torch.int32, device=again.device)
@@ -759,7 +752,7 @@ class CholeskyQR:
             # in a row did not bring nearer than half of before -- or a stack where every fourth matrix is far (eight
             # at least) -- is of low numerical rank: rounds diverge there, the replacing sweep does not.
             away = ~self.near
-            many = away.sum() >= 8 and away.sum() * 4 > self.Y.shape[0]
+            many = away.sum() >= 8 and away.sum() * 4 > self.batch
             with np.errstate(invalid="ignore"):
                 no_nearer = away & np.isfinite(self.far_before) & ~(distance < 0.5 * self.far_before)      # (NaN and inf count)
             self.stuck = np.where(no_nearer, self.stuck + 1, 0)
@@ -801,11 +794,11 @@ class CholeskyQR:
             bad, near, ids = self._failures()
             self.redo += ids[bad & near].tolist()
         if self.final is None:
-            self.final = torch.empty_like(self.Y)
+            self.final = torch.empty(self.batch, self.n, self.n, device=self.device)
         if self.redo:
-            redo = torch.tensor(sorted(set(self.redo)), device=self.Y.device)
+            redo = torch.tensor(sorted(set(self.redo)), device=self.device)
             torch.cuda.synchronize()              # the library routine is not trusted to be stream-ordered here
-            self.final[redo] = _householder_qr(self.Y[redo])[0]
+            self.final[redo] = _householder_qr(self._original(redo))[0]
             torch.cuda.synchronize()
         Q = self.final
         if Q.shape[1] != self.true_n:
