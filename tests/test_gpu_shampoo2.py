@@ -626,3 +626,46 @@ def test_column_dots_is_the_diagonal_of_the_product(mods, n, batch):
     assert torch.equal(got, X.column_dots(A.cuda(), B.cuda()))                 # fixed summation order
     with pytest.raises(ValueError):
         X.column_dots(A.cuda(), B[:, :, :32].contiguous().cuda())
+
+
+def test_a_clean_sweep_means_an_orthonormal_result(mods):
+    """CholeskyQR takes a swept matrix whose flags are all clear as final without testing it.  That rests on the sweep:
+    whenever it reports nothing (no pivot at the floor, no column replaced, no NaN) the result must be orthonormal to
+    fp32 rounding -- checked here over well and ill conditioned matrices, graded column scales, numerically dependent
+    columns and low rank, where the sweep has to raise a flag for whatever it cannot finish."""
+    _, E2 = mods
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(99)
+    n = 256
+    mats, kinds = [], []
+    for cond in (0.0, 2.0, 4.0, 6.0, 8.0):                                      # singular values 1 .. 10^-cond
+        u, _ = torch.linalg.qr(torch.randn(n, n, generator=g, dtype=torch.float64))
+        v, _ = torch.linalg.qr(torch.randn(n, n, generator=g, dtype=torch.float64))
+        mats.append(((u * torch.logspace(0, -cond, n, dtype=torch.float64)) @ v.T).float())
+        kinds.append("cond 1e%d" % cond)
+    graded = torch.randn(n, n, generator=g) * torch.logspace(0, -12, n)             # column scales over twelve decades
+    mats.append(graded); kinds.append("graded columns")
+    twin = torch.randn(n, n, generator=g)
+    twin[:, 100] = twin[:, 7] * (1 + 1e-7) + 1e-9 * torch.randn(n, generator=g)     # a column that repeats an earlier one
+    mats.append(twin); kinds.append("repeated column")
+    for rank in (n // 2, 8):
+        low = torch.randn(n, rank, generator=g) @ torch.randn(rank, n, generator=g)
+        mats.append(low + 1e-7 * torch.randn(n, n, generator=g)); kinds.append("rank %d plus noise" % rank)
+        mats.append(low); kinds.append("rank %d exactly" % rank)
+    Y = torch.stack(mats).cuda()
+    Q = (Y / torch.linalg.vector_norm(Y, dim=1, keepdim=True).clamp_min(1e-30)).contiguous()
+    info = torch.zeros(len(mats), dtype=torch.int32, device="cuda")
+    X.block_gram_schmidt(Q, info)
+    gram = Q.double().transpose(1, 2) @ Q.double()
+    off = (gram - torch.eye(n, dtype=torch.float64, device="cuda")).abs().amax(dim=(1, 2)).cpu()
+    flags = info.cpu().tolist()
+    for kind, flag, worst in zip(kinds, flags, off.tolist()):
+        print("%-22s flags %d  max |Q^T Q - I| %.2e" % (kind, flag, worst))
+        if flag == 0:
+            assert worst <= 2e-5, (kind, worst)
+    assert flags[0] == 0 and flags[1] == 0                                         # the easy ones are clean
+    assert all(f != 0 for f, k in zip(flags, kinds) if k.startswith("rank") or k == "repeated column")
+    # and the whole solver ends orthonormal for every one of them
+    final, redone = X.cholesky_qr(Y)
+    gram = final.double().transpose(1, 2) @ final.double()
+    assert float((gram - torch.eye(n, dtype=torch.float64, device="cuda")).abs().max()) <= 5e-5
