@@ -210,26 +210,50 @@ __global__ __launch_bounds__(256) void copy_flagged_kernel(float *dst, const flo
 
 // out[b][j] = sum_i A[b][i][j] B[b][i][j] for two stacks of n x n matrices: the diagonal of A^T B without the
 // product (the Rayleigh quotients diag(Q^T (L Q)) of a subspace iteration step).  A workgroup takes 64 columns of
-// one matrix; its four waves take every fourth row, eight rows in flight per thread, and add up in a fixed order.
+// one matrix: 16 lanes cover them with 16-byte loads, the 16 groups of lanes take every sixteenth row, four rows in
+// flight per thread, and the partial sums are added in a fixed order.
 __global__ __launch_bounds__(256) void column_dots_kernel(const float *A, const float *B, float *out, int n) {
-    const int c = blockIdx.x * 64 + (threadIdx.x & 63), g = threadIdx.x >> 6, b = blockIdx.y;
-    const float *pa = A + (long long)b * n * n + c, *pb = B + (long long)b * n * n + c;
-    float part8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const int c4 = (threadIdx.x & 15) * 4, g = threadIdx.x >> 4, b = blockIdx.y;
+    const long long base = (long long)b * n * n + blockIdx.x * 64 + c4;
+    const float *pa = A + base, *pb = B + base;
+    float4 part[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     int r = g;
-    for (; r + 28 < n; r += 32) {
-        float x[8], y[8];
+    for (; r + 48 < n; r += 64) {
+        float4 x[4], y[4];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) { x[i] = pa[(long long)(r + 4 * i) * n]; y[i] = pb[(long long)(r + 4 * i) * n]; }
+        for (int i = 0; i < 4; ++i) {
+            x[i] = *reinterpret_cast<const float4 *>(pa + (long long)(r + 16 * i) * n);
+            y[i] = *reinterpret_cast<const float4 *>(pb + (long long)(r + 16 * i) * n);
+        }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) part8[i] = __builtin_fmaf(x[i], y[i], part8[i]);
+        for (int i = 0; i < 4; ++i) {
+            part[i].x = __builtin_fmaf(x[i].x, y[i].x, part[i].x);
+            part[i].y = __builtin_fmaf(x[i].y, y[i].y, part[i].y);
+            part[i].z = __builtin_fmaf(x[i].z, y[i].z, part[i].z);
+            part[i].w = __builtin_fmaf(x[i].w, y[i].w, part[i].w);
+        }
     }
-    for (; r < n; r += 4) part8[0] = __builtin_fmaf(pa[(long long)r * n], pb[(long long)r * n], part8[0]);
-    __shared__ float part[4][64];
-    part[g][threadIdx.x & 63] = ((part8[0] + part8[1]) + (part8[2] + part8[3])) + ((part8[4] + part8[5]) + (part8[6] + part8[7]));
+    for (; r < n; r += 16) {
+        const float4 x = *reinterpret_cast<const float4 *>(pa + (long long)r * n), y = *reinterpret_cast<const float4 *>(pb + (long long)r * n);
+        part[0].x = __builtin_fmaf(x.x, y.x, part[0].x);
+        part[0].y = __builtin_fmaf(x.y, y.y, part[0].y);
+        part[0].z = __builtin_fmaf(x.z, y.z, part[0].z);
+        part[0].w = __builtin_fmaf(x.w, y.w, part[0].w);
+    }
+    __shared__ float sums[16][64];
+    sums[g][c4 + 0] = (part[0].x + part[1].x) + (part[2].x + part[3].x);
+    sums[g][c4 + 1] = (part[0].y + part[1].y) + (part[2].y + part[3].y);
+    sums[g][c4 + 2] = (part[0].z + part[1].z) + (part[2].z + part[3].z);
+    sums[g][c4 + 3] = (part[0].w + part[1].w) + (part[2].w + part[3].w);
     __syncthreads();
-    if (g == 0) {
+    if (threadIdx.x < 64) {
         const int l = threadIdx.x;
-        out[(long long)b * n + c] = (part[0][l] + part[1][l]) + (part[2][l] + part[3][l]);
+        float total = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) total += sums[k][l];
+        out[(long long)b * n + blockIdx.x * 64 + l] = total;
     }
 }
 
