@@ -376,3 +376,41 @@ def test_per_parameter_optimizer_checkpoint_is_flat(setup, monkeypatch):
     run(opt2, resumed, range(3, 5))
     for a, b in zip(straight, resumed):
         assert torch.equal(a.detach(), b.detach())
+
+
+def test_fused_step_with_parameters_the_bank_does_not_take(setup, monkeypatch):
+    """A bf16 matrix and a vector stay outside the bank (per-parameter preconditioner, torch's update rules with
+    per-parameter bias corrections) next to banked fp32 matrices; gradients are missing on some steps.  Against the
+    per-parameter optimizer; the checkpoint stays flat."""
+    import io
+    S1 = setup[0]
+    import optimizers.matrix_functions as MF
+    g = torch.Generator().manual_seed(23)
+    shapes = [(128, 192), (128, 64), (64,), (256, 64)]
+    dtypes = [torch.float32, torch.bfloat16, torch.float32, torch.float32]
+    init = [torch.rand(s, generator=g).to(d) for s, d in zip(shapes, dtypes)]
+    gs = [[(0.02 * torch.randn(s, generator=g)).to(d) for s, d in zip(shapes, dtypes)] for _ in range(5)]
+    present = [[True, st != 1, st != 3, st >= 1] for st in range(5)]
+    monkeypatch.setattr(MF.torch, "rand", lambda *size, **kw: torch.full(size, 0.75, **kw))
+    finals = []
+    for fused in (False, True):
+        params = [torch.nn.Parameter(t.clone().cuda()) for t in init]
+        opt = S1.ShampooAdamW(params, lr=1e-2, weight_decay=0.05, start_prec_step=2, stat_compute_steps=1, prec_compute_steps=2,
+                              fused=fused, **KW)
+        for st in range(5):
+            for p, gr, there in zip(params, gs[st], present[st]):
+                p.grad = gr.clone().cuda() if there else None
+            opt.step()
+        finals.append([p.detach().float().cpu() for p in params])
+        if fused:
+            assert "preconditioner" in opt.state[params[1]] and "preconditioner" in opt.state[params[2]]
+            assert "preconditioner" not in opt.state[params[0]] and "preconditioner" not in opt.state[params[3]]
+            sd = opt.state_dict()
+            assert sorted(sd["shampoo_preconditioners"]) == [1, 2]
+            buf = io.BytesIO()
+            torch.save(sd, buf)
+            buf.seek(0)
+            torch.load(buf, weights_only=True, map_location="cpu")
+        assert [opt.state[p]["step"] for p in params] == [sum(row[k] for row in present) for k in range(4)]
+    for k, (a, b) in enumerate(zip(*finals)):
+        assert rel(a, b) <= (2e-4 if dtypes[k] == torch.float32 else 2e-2), k

@@ -102,3 +102,64 @@ def test_low_bit_request_on_cpu_stays_dense_and_state_dict_round_trips():
     opt2.load_state_dict(sd)
     assert opt2.state[params[0]]["step"] == 1
     assert "Shampoo" in S1.ShampooSGD.__doc__ and "rect_t1" in S2.ShampooAdamW.__doc__
+
+
+@pytest.mark.parametrize("mod,kw", [(S1, {}), (S2, dict(inv_root_mode=0)), (S2, dict(inv_root_mode=1))])
+def test_checkpoint_holds_no_pickled_objects_and_resumes_bit_for_bit(mod, kw, tmp_path, monkeypatch):
+    """state_dict() writes the preconditioners in their flat form (tensors, numbers, lists) under
+    'shampoo_preconditioners', so torch.load(weights_only=True) reads the whole checkpoint (the reference pickles its
+    Preconditioner objects, optimizers/shampoo2.py:311-317); a run resumed from it continues exactly like the
+    uninterrupted one; a state that still holds the objects (the reference's form) loads as well."""
+    import io
+    monkeypatch.chdir(tmp_path)
+    g = torch.Generator().manual_seed(3)
+    shapes = [(12, 10), (7,), (9, 9)]
+    init = [torch.randn(s, generator=g) for s in shapes]
+    grads = [[torch.randn(s, generator=g) for s in shapes] for _ in range(6)]
+
+    def make(params):
+        return mod.ShampooAdamW(params, lr=1e-2, weight_decay=0.05, start_prec_step=2, stat_compute_steps=1, prec_compute_steps=2,
+                                stat_decay=0.9, prec_maxorder=8, prec_bits=32, **kw)
+
+    def run(opt, params, steps):
+        for st in steps:
+            for p, gr in zip(params, grads[st]):
+                p.grad = gr.clone()
+            torch.manual_seed(300 + st)
+            opt.step()
+
+    straight = [torch.nn.Parameter(t.clone()) for t in init]
+    run(make(straight), straight, range(6))
+    first = [torch.nn.Parameter(t.clone()) for t in init]
+    opt = make(first)
+    run(opt, first, range(3))
+    sd = opt.state_dict()
+    assert set(sd["shampoo_preconditioners"]) == {0, 1, 2}
+    assert not any("preconditioner" in one for one in sd["state"].values())
+    assert all("preconditioner" in opt.state[p] for p in first)                  # the live state keeps its objects
+    buf = io.BytesIO()
+    torch.save(sd, buf)
+    buf.seek(0)
+    loaded = torch.load(buf, weights_only=True)
+    resumed = [torch.nn.Parameter(p.detach().clone()) for p in first]
+    opt2 = make(resumed)
+    opt2.load_state_dict(loaded)
+    assert opt2.state[resumed[0]]["preconditioner"].is_active()
+    run(opt2, resumed, range(3, 6))
+    for a, b in zip(straight, resumed):
+        assert torch.equal(a.detach(), b.detach())
+    # the reference's form: objects inside 'state'
+    legacy = torch.optim.Optimizer.state_dict(opt)
+    assert any("preconditioner" in one for one in legacy["state"].values())
+    third = [torch.nn.Parameter(p.detach().clone()) for p in first]
+    opt3 = make(third)
+    opt3.load_state_dict(legacy)
+    run(opt3, third, range(3, 6))
+    for a, b in zip(straight, third):
+        assert torch.equal(a.detach(), b.detach())
+    # a flat state for another shape is refused
+    other = make([torch.nn.Parameter(torch.zeros(20, 3))])
+    bad = other.state_dict()
+    bad["state"], bad["shampoo_preconditioners"] = {0: {"step": 1}}, {0: loaded["shampoo_preconditioners"][0]}
+    with pytest.raises(ValueError):
+        other.load_state_dict(bad)
