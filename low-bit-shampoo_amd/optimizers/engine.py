@@ -48,7 +48,6 @@ class _Group:
 
 _SHARED_STREAMS = {}
 LANES = 2                                            # chains of launches the eigenbasis bank runs side by side
-BESIDE_SLOT = 9                                      # a stream no fan-out uses (at most 8 of those): work next to the sweeps
 
 
 def shared_stream(device, slot):
@@ -169,10 +168,11 @@ class ShampooBank:
             g.scratch[side] = torch.empty(len(g), order, order, device=self.device)
         return g.scratch[side]
 
-    def _fan_out(self, jobs, inline=False):
+    def _fan_out(self, jobs, inline=False, join=True):
         """Run the callables round-robin on the side streams, after everything already queued on the
-        current stream; the current stream then waits for all of them.  inline: one after the other on
-        the current stream (for a caller that is itself a side job next to another fan-out)."""
+        current stream; the current stream then waits for all of them (join=False: the caller does that
+        later, with _join).  inline: one after the other on the current stream (for a caller that is itself
+        a side job next to another fan-out)."""
         if inline or not self.streams:
             for job in jobs:
                 job()
@@ -186,16 +186,20 @@ class ShampooBank:
                 side.wait_event(start)
             with torch.cuda.stream(side):
                 job()
-        for side in self.streams[:len(jobs)]:
-            done = torch.cuda.Event()
-            done.record(side)
-            main.wait_event(done)
+        if join:
+            self._join(len(jobs))
 
-    def _run_on(self, slot, job, after_current=True):
+    def _join(self, count=None):
+        """The current stream waits for what the first `count` side streams (default: all) hold now."""
+        main = torch.cuda.current_stream(self.device)
+        for side in self.streams[:count]:
+            main.wait_stream(side)
+
+    def _run_on(self, slot, job, after_current=True, join=True):
         """Run one callable on side stream `slot` (the stream _fan_out gives job number `slot`), after what the
-        current stream holds; the current stream then waits for it.  after_current=False: only after what that
-        side stream holds itself -- for a job that goes on with the work of an earlier job on the same stream,
-        while the current stream has since been made to wait for other streams as well."""
+        current stream holds; the current stream then waits for it (join=False: the caller does that later, with
+        _join).  after_current=False: only after what that side stream holds itself -- for a job that goes on with
+        the work of an earlier job on the same stream, while the current stream has since moved on."""
         if not self.streams:
             job()
             return
@@ -205,7 +209,8 @@ class ShampooBank:
             side.wait_stream(main)
         with torch.cuda.stream(side):
             job()
-        main.wait_stream(side)
+        if join:
+            main.wait_stream(side)
 
     # ---- eligibility -----------------------------------------------------------------------------
     @staticmethod

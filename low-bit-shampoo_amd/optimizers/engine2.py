@@ -25,7 +25,7 @@ import time
 
 import torch
 
-from optimizers.engine import BESIDE_SLOT, LANES, ShampooBank, SideJob, shared_stream
+from optimizers.engine import LANES, ShampooBank, SideJob
 from optimizers.matrix_functions import ComputePowerBatched
 from qtensor import fused as X
 
@@ -34,9 +34,8 @@ cholesky_qr = X.cholesky_qr
 
 
 class ShampooBank2(ShampooBank):
-    # Measured on the ViT-B/32 shapes (three orders, four hardware queues per process): 22.5 ms per regular step with
-    # three or four side streams, 23.7 with two, 26.7 with five (the job that applies the stored roots then shares
-    # a hardware queue with the longest sweep).
+    # Measured on the ViT-B/32 shapes (four orders, four hardware queues per process): 22.3 ms per regular step with
+    # three or four side streams, 23.6 with two.
     DEFAULT_STREAMS = 4
 
     def __init__(self, params, name2qmap, code, *, rect_t1=1, rect_t2=4, inv_root_mode=0, **kwargs):
@@ -85,9 +84,6 @@ class ShampooBank2(ShampooBank):
         for row in repaired:
             period = min(2 * table[row][0], 256) if row in table else 8
             table[row] = [period, period]
-
-    def _beside_stream(self):
-        return shared_stream(self.device, BESIDE_SLOT)       # (the same stream as the fourth of the fan-out streams)
 
     def _init_statistics(self):
         """Basis = quantized identity, every kept quotient and the largest one = matrix_eps
@@ -153,7 +149,7 @@ class ShampooBank2(ShampooBank):
         for g in self.groups:
             self._grad_list(g, grads)
 
-        solver, redone, tick = {}, {}, {}
+        solver, redone, tick, begun = {}, {}, {}, {}
         # (a stack starts with the replacing sweep when most of it needed that sweep lately, or when it holds a matrix that did)
         direct = {o: bool(self._replace_first(o) + self._known_low_rank(o)) for o in orders}
 
@@ -181,6 +177,8 @@ class ShampooBank2(ShampooBank):
                     return X.gemm(stat[order].index_select(0, ids), self._rectified_basis(order, ids), trans_b=True)
 
                 product = X.gemm(stat[order], basis[order], trans_b=True)
+                begun[order] = torch.cuda.Event()
+                begun[order].record(torch.cuda.current_stream(self.device))
                 # (the rectified basis came from another stream's job: its memory must not be handed out again on that
                 # stream before this one has read it)
                 basis[order].record_stream(torch.cuda.current_stream(self.device))
@@ -226,10 +224,10 @@ class ShampooBank2(ShampooBank):
                        if only is None or any(pi in only for pi in g.param_index)])
         # The Cholesky QR of every order advances on its own stream; the host waits once per round.
         # (_fan_out gives job i the stream i % streams, so an order keeps its stream from call to call.)
-        # Two lanes for the sweeps and what follows them: a process has four hardware queues, the parameters outside
-        # the bank and the job that applies the stored roots take one each, and streams beyond that share a queue in
-        # the order of their launches -- a third stack on a stream of its own ran behind the second anyway, and held
-        # up what the second had to do after its sweep.  The stacks are dealt out by cost, the cheap ones of a lane first.
+        # Two lanes for the sweeps and what follows them, a third for stacks of a matrix or two: a process has four
+        # hardware queues, the current stream takes one, and streams beyond that share a queue in the order of their
+        # launches -- a third large stack on a stream of its own ran behind the second anyway, and held up what the
+        # second had to do after its sweep.  The stacks are dealt out by cost, the cheap ones of a lane first.
         cost = {o: o ** 3 * self.per_order[o] for o in orders}
         small = [o for o in orders if cost[o] * 50 < max(cost.values())]          # a matrix or two of a small order: a chain of tiny launches
         big = [o for o in orders if o not in small]
@@ -240,12 +238,18 @@ class ShampooBank2(ShampooBank):
         if small:                                                          # (they get a lane of their own: nothing big waits behind them)
             lanes.append(sorted(small, key=lambda x: cost[x]))
         slot = {o: i for i, lane in enumerate(lanes) for o in lane}
-        self._fan_out([(lambda lane=lane: [project(o)() for o in lane]) for lane in lanes])
-        # work of the caller that does not depend on the statistics (bank.alongside, consumed here) fills the device
-        # next to the factorisations, on a thread and a stream of its own
+        self._fan_out([(lambda lane=lane: [project(o)() for o in lane]) for lane in lanes], join=False)
+        # Work of the caller that does not depend on the statistics (bank.alongside, consumed here) fills the device
+        # next to the sweeps -- chains of launches that leave most of it idle -- and not next to the large products
+        # before them: it goes to the current stream, which has nothing else to do until all stacks are through (it
+        # waits for them at the very end), behind the point where the first lane's sweep begins, and is queued by a
+        # thread of its own.  (A further stream would share a hardware queue with one of the lanes and run behind
+        # that lane's sweep, and that lane's next step behind it.)
         beside, self.alongside = self.alongside, None
         if beside is not None:
-            beside = SideJob(self.device, self._beside_stream(), beside)
+            current = torch.cuda.current_stream(self.device)
+            current.wait_event(begun[lanes[0][0]])
+            beside = SideJob(self.device, current, beside)
         # Every stack goes on alone from here, on the stream that holds its sweep: the test after the sweep (the host
         # reads the sweep's flags, then the deviations of the flagged matrices), a polishing round where needed, and
         # as soon as it is finished its Rayleigh quotients and re-encoding -- none of it waits for the sweep of another
@@ -287,15 +291,16 @@ class ShampooBank2(ShampooBank):
                     continue
                 waiting_since = time.monotonic()
                 for o in sorted(ready, key=lambda x: -x ** 3 * self.per_order[x]):
-                    self._run_on(slot[o], look_at(o), after_current=False)
+                    self._run_on(slot[o], look_at(o), after_current=False, join=False)
                     if solver[o].finished:
                         unfinished.remove(o)
-                        self._run_on(slot[o], iterate(o), after_current=False)
+                        self._run_on(slot[o], iterate(o), after_current=False, join=False)
                     else:
                         tick[o] = tick_of(o)
         finally:
             if beside is not None:
                 beside.join()
+            self._join()
         self.qr_fallbacks += sum(redone.values())
         self.qr_rounds += sum(solver[o].rounds for o in orders)
         self.qr_repairs += sum(solver[o].repairs for o in orders)
