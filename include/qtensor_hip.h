@@ -285,15 +285,18 @@ void qtensor_hip_cholesky_upper_floor_batched(float *gram, float *u, float *x, i
                                               qtensor_stream_t stream);
 /* Block Gram-Schmidt with reorthogonalisation, in place: the columns of every q[b] (n x n, unit columns on entry) are
  * made orthonormal left to right in panels -- a panel has the finished columns taken out of it (W = Q_<^T Y_p,
- * Y_p -= Q_< W), its columns rescaled to unit length, is orthonormalised inside, and all of that once more; on
- * the outer level a panel is qtensor_hip_block_gram_schmidt_width() columns wide and "inside" is the same scheme
- * over its 64-column panels, where "inside" is Cholesky QR (pivot_floor as in cholesky_upper_floor).  Keeps span(q[:, :k]) for every k like the Cholesky
- * QR rounds above, but loses orthogonality only in proportion to fp32 rounding, not to the squared condition
- * number, so one sweep replaces their repetition; it replaces torch.linalg.qr of qtensor/utils.py:157 for a whole
- * stack.  fill (optional, [n, n], unit columns): a column that the first projection leaves shorter than
- * sqrt(null_norm2) -- rounding noise: it depends on the columns before it -- is replaced by the same column of
- * fill (bit 2 of info[b]) and then treated like any other.  w: scratch [batch, n, width]; gram, u, x: scratch
- * [batch, 64, 64] each; info as in cholesky_upper_floor (zeroed by the caller). */
+ * Y_p -= Q_< W), is orthonormalised inside, and all of that once more; on the outer level a panel is
+ * qtensor_hip_block_gram_schmidt_width() columns wide and "inside" is the same scheme over its 64-column panels,
+ * where "inside" is one Cholesky QR round in three launches: the Gram matrix of the panel as it is, its factorisation
+ * scaled to a unit diagonal (pivot_floor as in cholesky_upper_floor), and the panel times D^-1 U^-1.  Keeps
+ * span(q[:, :k]) for every k like the Cholesky QR rounds above, but loses orthogonality only in proportion to fp32
+ * rounding, not to the squared condition number, so one sweep replaces their repetition; it replaces torch.linalg.qr
+ * of qtensor/utils.py:157 for a whole stack.  fill (optional, [n, n], unit columns): a column that the projections of
+ * the first pass leave shorter than sqrt(null_norm2) -- rounding noise: it depends on the columns before it -- leaves
+ * that pass as a zero column and enters the second one as the same column of fill (bit 2 of info[b]); the last
+ * 4 * batch floats of w then hold which columns those are.  w: scratch [batch, n, width]; gram, x: scratch
+ * [batch, 64, 64] each; u: not used any more (kept in the signature); info as in cholesky_upper_floor (zeroed by the
+ * caller). */
 int qtensor_hip_block_gram_schmidt_width(void);
 void qtensor_hip_block_gram_schmidt_batched(float *q, float *w, float *gram, float *u, float *x, const float *fill, int *info,
                                             int n, int batch, float pivot_floor, float null_norm2, qtensor_stream_t stream);
@@ -301,9 +304,8 @@ void qtensor_hip_block_gram_schmidt_batched(float *q, float *w, float *gram, flo
  * dependent on the columns before it inside its 64-column panel (pivot at or below the floor) is replaced by its
  * stand-in column from fill before the second pass as well (bit 2 of info[b]), instead of being handed to the second pass
  * as it is (bit 1 if it is dependent there again).  For matrices of low numerical rank, where what a first pass leaves
- * of such a column is rounding noise: the plain sweep ends with columns that are not orthogonal there.  The last
- * 4 * batch floats of w then hold which columns were set aside.  (No counterpart in the reference: Householder QR
- * completes a rank-deficient basis by construction.) */
+ * of such a column is rounding noise: the plain sweep ends with columns that are not orthogonal there.  (No
+ * counterpart in the reference: Householder QR completes a rank-deficient basis by construction.) */
 void qtensor_hip_block_gram_schmidt_replacing_batched(float *q, float *w, float *gram, float *u, float *x, const float *fill,
                                                       int *info, int n, int batch, float pivot_floor, float null_norm2,
                                                       int replace_dependent, qtensor_stream_t stream);

@@ -52,20 +52,53 @@ __device__ __forceinline__ float lane_value(float x, int lane) {
     return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(x), lane));
 }
 
+//
+// SCALED: `gram` is the Gram matrix S = P^T P of a panel whose columns are not of unit length yet.  The kernel factors
+// D^-1 S D^-1 (D = the column lengths, from the diagonal of S) and `inv` receives D^-1 U^-1, so that P inv is the
+// orthonormalised panel without a pass that rescales it first; u and panel_inv are not written.  With stand_in != 0
+// a column whose squared length is not at least too_short (what projecting the earlier columns out has left of a
+// unit column is rounding noise; a NaN counts) is set aside like a dropped one -- it takes no part in the
+// factorisation, its column of inv is zero, its bit of set_aside is set -- whatever aside_pivots says; aside_pivots
+// == 0 keeps the columns dropped for their pivot where they are (bit 1 of info) and reports only the short ones.
+template <bool SCALED>
 __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long long g_stride, int ldg, float *u,
                                                         long long u_stride, int ldu, float *inv, long long inv_stride,
                                                         int ldi, float *panel_inv, int *info, float pivot_floor,
-                                                        unsigned long long *set_aside, int aside_stride) {
+                                                        unsigned long long *set_aside, int aside_stride, float too_short,
+                                                        int stand_in, int aside_pivots) {
     __shared__ __attribute__((aligned(16))) float cols[NB][LDC];
+    __shared__ float lengths[NB];
     const int b = blockIdx.x, lane = threadIdx.x;
     const float *G = gram + (long long)b * g_stride;
     for (int r = 0; r < NB; ++r) cols[r][lane] = G[(long long)r * ldg + lane];
     __syncthreads();
     float row[NB];                               // row `lane` of the symmetric matrix; ends as row `lane` of L
     float s[NB];                                 // right-hand side e_lane of the substitution; ends as column `lane` of L^-1
+    float own_scale = 1.0f;                      // SCALED: 1 / length of column `lane` (0 for a column set aside or of length 0)
+    unsigned long long early = 0;                // SCALED: the columns set aside for their length (uniform over the wave)
+    if constexpr (SCALED) {
+        const float norm2 = cols[lane][lane];
+        const bool aside = stand_in != 0 && !(norm2 >= too_short);
+        own_scale = 0.0f;
+        if (!aside) {
+            if (norm2 > 0.0f) {
+                const float r = __builtin_amdgcn_rsqf(norm2);
+                own_scale = r * __builtin_fmaf(-0.5f * norm2 * r, r, 1.5f);
+            } else if (norm2 != norm2) {
+                own_scale = norm2;               // a NaN column fails the factorisation, as it did when it was rescaled first
+            }
+        }
+        early = __ballot(aside);
+        lengths[lane] = own_scale;
+        __syncthreads();
+    }
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         row[j] = j >= lane ? cols[lane][j] : cols[j][lane];
+        if constexpr (SCALED) {
+            const bool out = ((early >> j) & 1ull) || ((early >> lane) & 1ull);
+            row[j] = out ? (j == lane ? 1.0f : 0.0f) : row[j] * own_scale * lengths[j];
+        }
         s[j] = j == lane ? 1.0f : 0.0f;
     }
     __syncthreads();
@@ -118,21 +151,28 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
         x_prev = xk;
         wave_lds_sync();                         // column k is readable in the next step
     }
-    float *U = u + (long long)b * u_stride;
     float *I = inv + (long long)b * inv_stride + (long long)lane * ldi;
+    if constexpr (!SCALED) {
+        float *U = u + (long long)b * u_stride;
 #pragma unroll
-    for (int r = 0; r < NB; ++r) U[(long long)r * ldu + lane] = r <= lane ? row[r] : 0.0f;        // U[r][lane] = L[lane][r]
+        for (int r = 0; r < NB; ++r) U[(long long)r * ldu + lane] = r <= lane ? row[r] : 0.0f;    // U[r][lane] = L[lane][r]
+    }
     if (set_aside != nullptr) {
+        const unsigned long long out = SCALED ? early | (aside_pivots != 0 ? dropped : 0ull) : dropped;
 #pragma unroll
         for (int c = 0; c < NB; ++c)
-            if ((dropped >> c) & 1ull) s[c] = 0.0f;
-        if (lane == 0) set_aside[(long long)b * aside_stride] = dropped;
-        dropped = 0;
+            if ((out >> c) & 1ull) s[c] = 0.0f;
+        if (lane == 0) set_aside[(long long)b * aside_stride] = out;
+        if (!SCALED || aside_pivots != 0) dropped = 0;
+    }
+    if constexpr (SCALED) {
+#pragma unroll
+        for (int c = 0; c < NB; ++c) s[c] *= own_scale;                                            // row `lane` of D^-1 U^-1
     }
 #pragma unroll
     for (int c = 0; c < NB; c += 4)              // U^-1[lane][c] = L^-1[c][lane] = s[c] of this lane (zero for c < lane)
         *reinterpret_cast<float4 *>(I + c) = make_float4(s[c], s[c + 1], s[c + 2], s[c + 3]);
-    if (panel_inv != nullptr) {
+    if (!SCALED && panel_inv != nullptr) {
         float *P = panel_inv + (long long)b * inv_stride + (long long)lane * ldi;
 #pragma unroll
         for (int c = 0; c < NB; c += 4) {
@@ -257,69 +297,80 @@ __global__ __launch_bounds__(256) void column_dots_kernel(const float *A, const 
     }
 }
 
-// One 64-column panel of every matrix of a stack: each column is scaled to unit length; with `fill` given, a
-// column whose squared length is below null_norm2 (what projecting out the earlier columns has left of a
-// unit column: rounding noise) is replaced by the same column of `fill` (unit columns in general position)
-// and bit 2 of info[b] is set.  The panel is n x 64 with leading dimension ld.  Two launches over
-// (kNormChunks row chunks, batch): squared lengths per chunk into partial [batch][kNormChunks][64], then
-// every chunk adds them up in the same order and rescales (or replaces) its rows.
+// out[b] (64 x 64, rows 64 floats apart) = A_b^T B_b for two panels of 64 columns and n rows (n a multiple of 64, rows
+// ld floats apart) of every matrix of a stack: the Gram matrix of a panel (A == B; upper_only: the block below the
+// diagonal is not computed) or the coefficients of a panel on its neighbour.  grid (32 x 32 blocks of the result,
+// batch); the four waves of a workgroup take a quarter of the rows each and add their blocks up in a fixed order.
+// The operands go from memory straight into the fp32 matrix instruction (v_mfma_f32_32x32x2f32: lane l supplies column
+// l % 32 of its block and row l / 32 of a pair of rows), 16 rows per group of loads, three groups in flight.
+// What bounds it is the number of half rows (128 bytes, 4 KB apart) it asks memory for -- 20 us for 99 panels of 1024
+// rows, where one pass over the same bytes in whole rows takes 5: sixteen waves per workgroup (23 us) or one
+// workgroup per matrix (33 us: rows 4 KB apart share a set of the first-level cache) do not change that.
 constexpr int kNormChunks = 8;
+constexpr int kPanelGroup = 8;                   // matrix instructions (pairs of rows) per group of loads
 
-__global__ __launch_bounds__(256) void panel_norms_kernel(const float *panel, long long stride, int ld, int n, float *partial) {
-    const int chunk = blockIdx.x, b = blockIdx.y, c = threadIdx.x & 63, g = threadIdx.x >> 6;
-    const float *P = panel + (long long)b * stride;
-    const int rows = (n + kNormChunks - 1) / kNormChunks, r0 = chunk * rows, r1 = min(r0 + rows, n);
-    // eight rows in flight per thread: the loop is bound by the latency of its loads, not by their number
-    float part8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    int r = r0 + g;
-    for (; r + 28 < r1; r += 32) {
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = P[(long long)(r + 4 * i) * ld + c];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) part8[i] = __builtin_fmaf(v[i], v[i], part8[i]);
-    }
-    for (; r < r1; r += 4) {
-        const float v = P[(long long)r * ld + c];
-        part8[0] = __builtin_fmaf(v, v, part8[0]);
-    }
-    const float sum = ((part8[0] + part8[1]) + (part8[2] + part8[3])) + ((part8[4] + part8[5]) + (part8[6] + part8[7]));
-    __shared__ float part[4][64];
-    part[g][c] = sum;
-    __syncthreads();
-    if (g == 0) partial[((long long)b * kNormChunks + chunk) * 64 + c] = (part[0][c] + part[1][c]) + (part[2][c] + part[3][c]);
-}
+typedef float qt_acc16 __attribute__((ext_vector_type(16)));
 
-__global__ __launch_bounds__(256) void panel_rescale_kernel(float *panel, long long stride, int ld, int n, const float *partial,
-                                                            const float *fill, int fill_ld, float null_norm2, int *info) {
-    const int chunk = blockIdx.x, b = blockIdx.y, c = threadIdx.x & 63, g = threadIdx.x >> 6;
-    float *P = panel + (long long)b * stride;
-    float norm2 = 0.0f;
+__global__ __launch_bounds__(256) void panel_product_kernel(const float *A, const float *B, long long stride, int ld, int n,
+                                                            float *out, long long out_stride, int upper_only) {
+    const int b = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int bi = upper_only ? (int)(blockIdx.x == 2) : (int)(blockIdx.x >> 1);
+    const int bj = upper_only ? (int)(blockIdx.x >= 1) : (int)(blockIdx.x & 1);
+    const int rows = n / 4, groups = rows / (2 * kPanelGroup);                 // (n is a multiple of 64)
+    const long long first = (long long)b * stride + (long long)(wave * rows + (lane >> 5)) * ld + (lane & 31);
+    const float *pa = A + first + 32 * bi, *pb = B + first + 32 * bj;
+    // (no branches between the loads and the matrix instructions: the compiler then counts the loads in flight exactly
+    // and waits for no more than the group it is about to use)
+    float a[4][kPanelGroup], c[4][kPanelGroup];
+    auto load = [&](int buf, int group) {
+        const long long at = (long long)min(group, groups - 1) * (2 * kPanelGroup) * ld;   // (past the end: a load nobody uses)
 #pragma unroll
-    for (int k = 0; k < kNormChunks; ++k) norm2 += partial[((long long)b * kNormChunks + k) * 64 + c];
-    const int rows = (n + kNormChunks - 1) / kNormChunks, r0 = chunk * rows, r1 = min(r0 + rows, n);
-    const bool replace = fill != nullptr && !(norm2 >= null_norm2);          // (a NaN column is replaced as well)
-    if (replace) {
-        for (int r = r0 + g; r < r1; r += 4) P[(long long)r * ld + c] = fill[(long long)r * fill_ld + c];
-        if (g == 0 && chunk == 0) atomicOr(info + b, 4);
-    } else if (norm2 > 0.0f) {
-        float scale = __builtin_amdgcn_rsqf(norm2);
-        scale = scale * __builtin_fmaf(-0.5f * norm2 * scale, scale, 1.5f);
-        int r = r0 + g;
-        for (; r + 28 < r1; r += 32) {               // eight rows in flight per thread
-            float v[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = P[(long long)(r + 4 * i) * ld + c];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) P[(long long)(r + 4 * i) * ld + c] = v[i] * scale;
+        for (int m = 0; m < kPanelGroup; ++m) {
+            a[buf][m] = pa[at + (long long)(2 * m) * ld];
+            c[buf][m] = pb[at + (long long)(2 * m) * ld];
         }
-        for (; r < r1; r += 4) P[(long long)r * ld + c] *= scale;
+    };
+    qt_acc16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    auto multiply = [&](int buf) {
+#pragma unroll
+        for (int m = 0; m < kPanelGroup; ++m) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[buf][m], c[buf][m], acc, 0, 0, 0);
+    };
+    load(0, 0);
+    load(1, 1);
+    load(2, 2);
+    int g = 0;
+    for (; g + 4 <= groups; g += 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            load((i + 3) & 3, g + i + 3);
+            multiply(i);
+        }
+    }
+    if (g < groups) {                                                          // up to three groups are left, in the buffers 0, 1, 2
+        multiply(0);
+        if (g + 1 < groups) {
+            multiply(1);
+            if (g + 2 < groups) multiply(2);
+        }
+    }
+    __shared__ float part[4][16][64];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part[wave][r][lane] = acc[r];
+    __syncthreads();
+    float *O = out + (long long)b * out_stride;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int r = 4 * wave + q;                                            // element r of a lane: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
+        const float sum = (part[0][r][lane] + part[1][r][lane]) + (part[2][r][lane] + part[3][r][lane]);
+        O[(32 * bi + 8 * wave + 4 * (lane >> 5) + q) * NB + 32 * bj + (lane & 31)] = sum;
     }
 }
 
 // The columns that the first pass over an outer panel set aside (bit j of aside[b * aside_stride + p]: column 64 p + j of
 // the panel, a zero column by now) take the same columns of `fill`; bit 2 of info[b] is set.  Launched over
-// (kNormChunks row chunks, batch) like the kernels above.
+// (kNormChunks row chunks, batch); threads take a column and every fourth row of the chunk.
 __global__ __launch_bounds__(256) void fill_aside_kernel(float *panel, long long stride, int ld, int n, int panels, int aside_stride,
                                                          const unsigned long long *aside, const float *fill, int fill_ld, int *info) {
     const int chunk = blockIdx.x, b = blockIdx.y, c = threadIdx.x & 63, g = threadIdx.x >> 6;
@@ -384,8 +435,8 @@ extern "C" void qtensor_hip_cholesky_upper_floor_batched(float *gram, float *u, 
             const long long corner = (long long)j0 * n + j0;
             // (the block of u right below the diagonal block is free: it takes the factor for the block row)
             float *panel_inv = rest > 0 ? u + (long long)j1 * n + j0 : nullptr;
-            hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram + corner, mat, n, u + corner, mat, n,
-                               x + corner, mat, n, panel_inv, info, pivot_floor, (unsigned long long *)nullptr, 0);
+            hipLaunchKernelGGL(cholesky64_kernel<false>, dim3(batch), dim3(NB), 0, stream, gram + corner, mat, n, u + corner, mat, n,
+                               x + corner, mat, n, panel_inv, info, pivot_floor, (unsigned long long *)nullptr, 0, 0.0f, 0, 0);
             if (!launch_ok("cholesky_upper_batched (diagonal block)")) return;
             if (rest == 0) break;
             const long long row = (long long)j0 * n + j1;
@@ -442,9 +493,9 @@ struct Sweep {
     hipStream_t stream;
     bool replace;                                             // columns a first pass finds dependent inside their panel are replaced too
     long long mat() const { return (long long)n * n; }
-    // replace: the tail of w holds, per matrix and 64-column panel of the current outer panel, which columns the
-    // first pass set aside (w_cols / 64 words of 64 bits per matrix)
-    long long w_floats() const { return (long long)batch * n * w_cols - (replace ? 2LL * batch * (w_cols / NB) : 0); }
+    // With stand-in columns the tail of w holds, per matrix and 64-column panel of the current outer panel, which
+    // columns the pass before set aside (w_cols / 64 words of 64 bits per matrix)
+    long long w_floats() const { return (long long)batch * n * w_cols - (fill != nullptr ? 2LL * batch * (w_cols / NB) : 0); }
     unsigned long long *aside_words() const { return reinterpret_cast<unsigned long long *>(w + w_floats()); }
 
     // columns [c0, c0 + width) -= Q[:, a0:c0] (Q[:, a0:c0]^T columns): the columns a0..c0 are orthonormal
@@ -479,44 +530,49 @@ struct Sweep {
     }
 
     // The 64 columns from c0 on, in pass `pass` of `passes` over their outer panel (which starts at column a0): take the
-    // columns a0..c0 out, unit columns, one Cholesky QR round inside.
-    // Stand-in columns: in the first pass a column shorter than sqrt(null_norm2) after the projections (it was a unit
-    // column before them: what is left is rounding noise) takes its column of `fill`.  In replace mode every pass but
-    // the last also sets aside the columns whose pivot inside the panel is at or below the floor -- they leave the
-    // pass as zero columns and come back as stand-in columns before the next one (fill_aside_kernel) -- and the
-    // passes between the first and the last replace a column that a projection shortens to less than half (it
-    // was orthonormalised a pass earlier: losing most of its length again means it was noise then).
+    // columns a0..c0 out, then one Cholesky QR round inside -- Gram matrix of the panel as it is (one launch that reads
+    // it once), factorisation of that matrix scaled to a unit diagonal (the columns' lengths are on the diagonal), and
+    // the panel times D^-1 U^-1: three launches, two passes over the panel.
+    // Stand-in columns: in every pass but the last a column that the projections have left shorter than a threshold
+    // -- sqrt(null_norm2) in the first pass, where it was a unit column before them and what is left is rounding
+    // noise; a half in the later ones, where it was orthonormalised a pass earlier and losing most of its length again
+    // means it was noise then -- leaves the pass as a zero column and comes back as its column of `fill` before the
+    // next pass (fill_aside_kernel).  In replace mode so do the columns whose pivot inside the panel is at or below
+    // the floor.
     bool panel(int a0, int c0, int pass, int passes) {
         float *panel_ptr = q + c0;
         const bool more = pass + 1 < passes;
+        const bool stand_in = fill != nullptr && more;
         // (word (c0 - a0) / 64 of the outer panel, matrices w_cols / 64 words apart -- see fill_aside_kernel)
-        unsigned long long *aside = replace && more ? aside_words() + (c0 - a0) / NB : nullptr;
-        const float *stand_in = fill == nullptr ? nullptr : pass == 0 || (replace && more) ? fill + c0 : nullptr;
+        unsigned long long *aside = stand_in ? aside_words() + (c0 - a0) / NB : nullptr;
         const float too_short = pass == 0 ? null_norm2 : 0.25f;
         // The last pass of replace mode normalises whatever has a pivot above the noise of the Gram matrix: a stand-in
         // column for one of the last columns of a matrix has little room left (the complement of a thousand columns in
         // a space of as many dimensions), which is a small pivot and no dependence.
         const float floor_here = replace && !more && pivot_floor > 1e-6f ? 1e-6f : pivot_floor;
         const long long small = (long long)NB * NB;
-        float *norms = u;                                     // [batch][kNormChunks][64]: u is free between factorisations
-        if (!project(a0, c0, NB)) return false;
-        hipLaunchKernelGGL(panel_norms_kernel, dim3(kNormChunks, batch), dim3(256), 0, stream, panel_ptr, mat(), n, n, norms);
-        hipLaunchKernelGGL(panel_rescale_kernel, dim3(kNormChunks, batch), dim3(256), 0, stream, panel_ptr, mat(), n, n, norms,
-                           stand_in, n, too_short, info);
-        if (!launch_ok("block_gram_schmidt_batched (normalize)")) return false;
-        qtensor_gemm_desc g = {};                             // S = Y_p^T Y_p
-        g.M = NB; g.N = NB; g.K = n; g.batch = batch;
-        g.kind_a = QTENSOR_DENSE_T; g.kind_b = QTENSOR_DENSE; g.epilogue = QTENSOR_EPI_STORE;
-        g.args.A = strided(panel_ptr, mat()); g.args.lda = n;
-        g.args.B = strided(panel_ptr, mat()); g.args.ldb = n;
-        g.args.C = strided(gram, small); g.args.ldc = NB;
-        g.args.workspace = w;                                 // one tile per matrix and a long k range: cut along k
-        g.args.workspace_floats = w_floats();
-        if (!run(g, stream)) return false;
-        hipLaunchKernelGGL(cholesky64_kernel, dim3(batch), dim3(NB), 0, stream, gram, small, NB, u, small, NB, x, small, NB,
-                           (float *)nullptr, info, floor_here, aside, w_cols / NB);
+        if (c0 - a0 == NB) {
+            // against the one neighbour inside the outer panel: coefficients in one launch, straight from the panels
+            hipLaunchKernelGGL(panel_product_kernel, dim3(4, batch), dim3(256), 0, stream, q + a0, panel_ptr, mat(), n, n, w, small, 0);
+            if (!launch_ok("block_gram_schmidt_batched (coefficients)")) return false;
+            qtensor_gemm_desc r = {};                         // Y -= Q_a W
+            r.M = n; r.N = NB; r.K = NB; r.batch = batch;
+            r.kind_a = QTENSOR_DENSE; r.kind_b = QTENSOR_DENSE; r.epilogue = QTENSOR_EPI_AXPBY_DENSE;
+            r.args.A = strided(q + a0, mat()); r.args.lda = n;
+            r.args.B = strided(w, small); r.args.ldb = NB;
+            r.args.C = strided(panel_ptr, mat()); r.args.ldc = n;
+            r.args.E = strided(panel_ptr, mat()); r.args.lde = n;
+            r.args.alpha = -1.0f; r.args.beta = 1.0f;
+            if (!run(r, stream)) return false;
+        } else if (!project(a0, c0, NB)) {
+            return false;
+        }
+        hipLaunchKernelGGL(panel_product_kernel, dim3(3, batch), dim3(256), 0, stream, panel_ptr, panel_ptr, mat(), n, n, gram, small, 1);
+        hipLaunchKernelGGL(cholesky64_kernel<true>, dim3(batch), dim3(NB), 0, stream, gram, small, NB, (float *)nullptr, small, NB, x,
+                           small, NB, (float *)nullptr, info, floor_here, aside, w_cols / NB, too_short, stand_in ? 1 : 0,
+                           replace && more ? 1 : 0);
         if (!launch_ok("block_gram_schmidt_batched (panel factor)")) return false;
-        qtensor_gemm_desc t = {};                             // Y_p <- Y_p U^-1 (one tile column: in place is safe)
+        qtensor_gemm_desc t = {};                             // Y_p <- Y_p D^-1 U^-1 (one tile column: in place is safe)
         t.M = n; t.N = NB; t.K = NB; t.batch = batch;
         t.kind_a = QTENSOR_DENSE; t.kind_b = QTENSOR_DENSE; t.epilogue = QTENSOR_EPI_STORE;
         t.args.A = strided(panel_ptr, mat()); t.args.lda = n;
@@ -582,8 +638,8 @@ extern "C" void qtensor_hip_block_gram_schmidt_replacing_batched(float *q, float
     for (int o0 = 0; o0 < n; o0 += outer) {
         const int width = n - o0 < outer ? n - o0 : outer;
         for (int pass = 0; pass < passes; ++pass) {
-            if (pass >= 1 && s.replace) {
-                // what the first pass set aside comes back as stand-in columns, ahead of everything the second pass does
+            if (pass >= 1 && fill != nullptr) {
+                // what the pass before set aside comes back as stand-in columns, ahead of everything this pass does
                 hipLaunchKernelGGL(fill_aside_kernel, dim3(kNormChunks, batch), dim3(256), 0, s.stream, q + o0, s.mat(), n, n, width / NB,
                                    outer / NB, s.aside_words(), fill + o0, n, info);
                 if (!launch_ok("block_gram_schmidt_batched (stand-in columns)")) return;
