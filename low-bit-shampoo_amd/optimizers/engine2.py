@@ -64,20 +64,33 @@ class ShampooBank2(ShampooBank):
             return False
         return True
 
+    APART_AT_MOST = 8                             # so many known low-rank matrices of a stack are still orthonormalised on their own
+
     def _known_low_rank(self, order):
-        """How many matrices of this stack are, for this update, taken to be of low numerical rank: those whose recent
+        """The matrices of this stack that are, for this update, taken to be of low numerical rank: those whose recent
         updates ended in the replacing sweep (the order-768 statistic of a 768 x 100 head: rank 100 plus the kept half).
-        A stack that holds one starts with the replacing sweep -- three passes instead of two for the whole stack, less
-        than the chain of some three hundred small launches that sweeping the one matrix again costs behind two stuck
-        polishing rounds (ViT-B/32: 23.2 ms per regular step, every step alike, against 21.5 to 26.5).  Every `period`
-        updates the stack gets the plain sweep again; the period doubles (8, 16, ... 256) each time that look ends in
-        the replacing sweep once more."""
-        known = 0
-        for state in self.low_rank_rows.setdefault(order, {}).values():
+        Up to APART_AT_MOST of them are orthonormalised apart from their stack, as a small stack of their own that starts
+        with the replacing sweep, on the lane of the small stacks, while the stack itself gets the plain sweep and
+        leaves their places alone; with more of them the whole stack starts with the replacing sweep.  Every `period`
+        updates such a matrix goes through the plain sweep with its stack again; the period doubles (8, 16, ... 256)
+        each time that look ends in the replacing sweep once more."""
+        known = []
+        for row, state in self.low_rank_rows.setdefault(order, {}).items():
             if state[1] > 0:
                 state[1] -= 1
-                known += 1
-        return known
+                known.append(row)
+        return sorted(known)
+
+    def _row_index(self, rows):
+        """int64 device vector of a short list of row numbers, kept: a copy from the host in the middle of an update
+        would make the host wait for the stream it is queued on."""
+        cache = self.__dict__.setdefault("_row_index_cache", {})
+        key = tuple(rows)
+        if key not in cache:
+            if len(cache) > 64:
+                cache.clear()
+            cache[key] = torch.tensor(list(rows), dtype=torch.int64, device=self.device)
+        return cache[key]
 
     def _note_repairs(self, order, repaired):
         table = self.low_rank_rows.setdefault(order, {})
@@ -150,8 +163,14 @@ class ShampooBank2(ShampooBank):
             self._grad_list(g, grads)
 
         solver, redone, tick, begun = {}, {}, {}, {}
-        # (a stack starts with the replacing sweep when most of it needed that sweep lately, or when it holds a matrix that did)
-        direct = {o: bool(self._replace_first(o) + self._known_low_rank(o)) for o in orders}
+        # (a stack starts with the replacing sweep when most of it needed that sweep lately, or when it holds many
+        # matrices that did; a few such matrices are orthonormalised apart from it)
+        direct, apart = {}, {}
+        for o in orders:
+            mostly, known = self._replace_first(o), self._known_low_rank(o)
+            direct[o] = mostly or len(known) > self.APART_AT_MOST
+            apart[o] = [] if direct[o] else known
+        apart_y, apart_event, apart_q, apart_back = {}, {}, {}, {}
 
         def rebuild(order):
             def run():
@@ -179,11 +198,16 @@ class ShampooBank2(ShampooBank):
                 product = X.gemm(stat[order], basis[order], trans_b=True)
                 begun[order] = torch.cuda.Event()
                 begun[order].record(torch.cuda.current_stream(self.device))
+                if apart[order]:
+                    # the columns of the matrices that go their own way, before the product is scaled in place
+                    apart_y[order] = product.index_select(0, self._row_index(apart[order]))
+                    apart_event[order] = torch.cuda.Event()
+                    apart_event[order].record(torch.cuda.current_stream(self.device))
                 # (the rectified basis came from another stream's job: its memory must not be handed out again on that
                 # stream before this one has read it)
                 basis[order].record_stream(torch.cuda.current_stream(self.device))
                 basis[order] = None
-                solver[order] = X.CholeskyQR(product, replace_first=direct[order], remake=remake)
+                solver[order] = X.CholeskyQR(product, replace_first=direct[order], remake=remake, leave=apart[order])
                 del product
                 # (the event that tells the host this stack's sweep is through goes right behind it: streams share
                 # hardware queues, and behind the launches of another stack's sweep it would wait for those as well)
@@ -195,6 +219,11 @@ class ShampooBank2(ShampooBank):
             def run():
                 L = stat[order]
                 Q, redone[order] = solver[order].result()
+                if apart[order]:                       # the matrices that went apart come back into their places
+                    torch.cuda.current_stream(self.device).wait_event(apart_back[order])
+                    own = apart_q.pop(order)
+                    Q.index_copy_(0, self._row_index(apart[order]), own)
+                    own.record_stream(torch.cuda.current_stream(self.device))
                 # Rayleigh quotients diag(Q^T L Q), the product L Q a few dozen matrices at a time
                 quotients = torch.empty(Q.shape[0], Q.shape[1], device=self.device)
                 per = max(1, self.QUOTIENT_PART_BYTES // (4 * order * order))
@@ -238,7 +267,42 @@ class ShampooBank2(ShampooBank):
         if small:                                                          # (they get a lane of their own: nothing big waits behind them)
             lanes.append(sorted(small, key=lambda x: cost[x]))
         slot = {o: i for i, lane in enumerate(lanes) for o in lane}
-        self._fan_out([(lambda lane=lane: [project(o)() for o in lane]) for lane in lanes], join=False)
+        # (index tensors of the matrices that go apart, made before anything is queued)
+        for o in orders:
+            if apart[o]:
+                self._row_index(apart[o])
+        # (a stream of their own, next to the lanes: behind their long chain of small launches the host would wait
+        # with every test of a small stack)
+        apart_lane = len(lanes)
+        keys = list(orders) + [(o, "apart") for o in orders if apart[o]]
+        for o in orders:
+            if apart[o]:
+                slot[(o, "apart")] = apart_lane
+
+        def sweep_apart(order):
+            def run():
+                # the known low-rank matrices of the stack as a stack of their own, replacing sweep first
+                current = torch.cuda.current_stream(self.device)
+                current.wait_event(apart_event[order])
+                y = apart_y.pop(order)
+                y.record_stream(current)                                   # (made on the stack's lane, used up on this one)
+                ids = self._row_index(apart[order])
+
+                def remake(which):
+                    rows = ids.index_select(0, which)
+                    return X.gemm(stat[order].index_select(0, rows), self._rectified_basis(order, rows), trans_b=True)
+
+                key = (order, "apart")
+                solver[key] = X.CholeskyQR(y, replace_first=True, remake=remake)
+                tick[key] = torch.cuda.Event()
+                tick[key].record(current)
+            return run
+
+        jobs = [(lambda lane=lane: [project(o)() for o in lane]) for lane in lanes]
+        if any(apart.values()):
+            own = [sweep_apart(o) for o in orders if apart[o]]
+            jobs.append(lambda: [job() for job in own])
+        self._fan_out(jobs, join=False)
         # Work of the caller that does not depend on the statistics (bank.alongside, consumed here) fills the device
         # next to the sweeps -- chains of launches that leave most of it idle -- and not next to the large products
         # before them: it goes to the current stream, which has nothing else to do until all stacks are through (it
@@ -255,34 +319,46 @@ class ShampooBank2(ShampooBank):
         # as soon as it is finished its Rayleigh quotients and re-encoding -- none of it waits for the sweep of another
         # stack (the current stream, which waits for all of them, is left out of it).  The host takes the stacks in the
         # order in which their streams get there: it polls an event per stack.
-        unfinished = sorted(orders, key=lambda o: o ** 3 * self.per_order[o])
+        def cost_of(key):
+            return key ** 3 * self.per_order[key] if not isinstance(key, tuple) else key[0] ** 3 * len(apart[key[0]])
+
+        unfinished = sorted(keys, key=cost_of)
         on_side = bool(self.streams)
 
-        def tick_of(order):
+        def tick_of(key):
             event = torch.cuda.Event()
-            event.record(self.streams[slot[order] % len(self.streams)] if on_side else torch.cuda.current_stream(self.device))
+            event.record(self.streams[slot[key] % len(self.streams)] if on_side else torch.cuda.current_stream(self.device))
             return event
 
-        tested = {o: False for o in orders}            # the test of the current iterate is queued, its outcome not read yet
+        tested = {k: False for k in keys}              # the test of the current iterate is queued, its outcome not read yet
 
-        def look_at(order):
+        def look_at(key):
             # one step of the stack's state machine; every read of the host in it finds its data there already,
             # because the step before it ended with the event that is now through
             def run():
-                s = solver[order]
-                if not tested[order]:
+                s = solver[key]
+                if not tested[key]:
                     s.check()
-                    tested[order] = not s.finished
+                    tested[key] = not s.finished
                 else:
-                    tested[order] = False
+                    tested[key] = False
                     if not s.poll():
                         s.advance()
             return run
 
+        def hand_back(order):
+            def run():
+                # (result() on the stream the solver lived on; the stack's lane waits for the event)
+                apart_q[order], redone[(order, "apart")] = solver[(order, "apart")].result()
+                apart_back[order] = torch.cuda.Event()
+                apart_back[order].record(torch.cuda.current_stream(self.device))
+            return run
+
         waiting_since = time.monotonic()
+        done = set()
         try:
             while unfinished:
-                ready = [o for o in unfinished if tick[o].query()]
+                ready = [k for k in unfinished if tick[k].query()]
                 if not ready:
                     if time.monotonic() - waiting_since > self.STALL_SECONDS:
                         raise RuntimeError(f"the statistics update of the orders {unfinished} made no progress on the device "
@@ -290,20 +366,26 @@ class ShampooBank2(ShampooBank):
                     time.sleep(2e-5)
                     continue
                 waiting_since = time.monotonic()
-                for o in sorted(ready, key=lambda x: -x ** 3 * self.per_order[x]):
-                    self._run_on(slot[o], look_at(o), after_current=False, join=False)
-                    if solver[o].finished:
-                        unfinished.remove(o)
-                        self._run_on(slot[o], iterate(o), after_current=False, join=False)
-                    else:
-                        tick[o] = tick_of(o)
+                for k in sorted(ready, key=lambda x: -cost_of(x)):
+                    self._run_on(slot[k], look_at(k), after_current=False, join=False)
+                    if not solver[k].finished:
+                        tick[k] = tick_of(k)
+                        continue
+                    unfinished.remove(k)
+                    done.add(k)
+                    order = k[0] if isinstance(k, tuple) else k
+                    if isinstance(k, tuple):
+                        self._run_on(slot[k], hand_back(order), after_current=False, join=False)
+                    # a stack goes on when it and the matrices that went apart from it are both through
+                    if order in done and (not apart[order] or (order, "apart") in done):
+                        self._run_on(slot[order], iterate(order), after_current=False, join=False)
         finally:
             if beside is not None:
                 beside.join()
             self._join()
         self.qr_fallbacks += sum(redone.values())
-        self.qr_rounds += sum(solver[o].rounds for o in orders)
-        self.qr_repairs += sum(solver[o].repairs for o in orders)
+        self.qr_rounds += sum(solver[k].rounds for k in keys)
+        self.qr_repairs += sum(solver[k].repairs for k in keys)
         for o in orders:
             if not direct[o]:
                 self.low_rank[o][0] = solver[o].repairs * 4 > self.per_order[o]

@@ -605,8 +605,10 @@ class CholeskyQR:
     library).  All calls for one object must be made with the same current stream."""
 
     def __init__(self, Y, max_rounds=12, pivot_floor=PIVOT_FLOOR, tolerance=2e-5, sweep=True, replace_first=False,
-                 remake=None):
-        """remake: optional callable, int64 GPU vector of matrix numbers -> those matrices of Y again.  With it Y is
+                 remake=None, leave=()):
+        """leave: matrices of the stack (their numbers) that the caller orthonormalises some other way: whatever the
+        sweep makes of them is final here, they are neither tested nor polished.
+        remake: optional callable, int64 GPU vector of matrix numbers -> those matrices of Y again.  With it Y is
         given up: its columns are scaled in place and it becomes the working set (one stack less held through the
         sweep); the few matrices whose original columns are needed again (_repair, the library fallback) are made anew."""
         if Y.dim() != 3 or Y.shape[1] != Y.shape[2] or Y.dtype != torch.float32 or not Y.is_cuda:
@@ -614,6 +616,7 @@ class CholeskyQR:
         B, self.true_n, _ = Y.shape
         n = -(-self.true_n // 64) * 64
         self.batch, self.n, self.device, self.remake = B, n, Y.device, remake
+        self.leave = np.asarray(sorted(leave), dtype=np.int64)
         if n != self.true_n:
             Y = self._padded(Y)
         self.pivot_floor, self.tolerance, self.rounds_left = pivot_floor, tolerance, max_rounds
@@ -650,6 +653,24 @@ class CholeskyQR:
             block_gram_schmidt(self.Q, self.info, pivot_floor, replace_dependent=replace_first)
             if replace_first:
                 self.mended[:] = True
+            self.info_host = self._to_host(self.info)
+
+    def _to_host(self, t):
+        """A copy of a small device tensor on its way into pinned host memory, queued on the current stream right
+        behind what produced it (read it with _landed_numpy).  The host never queues a copy at the moment it wants
+        the data: on a stream that shares a hardware queue with another stack's chain of launches such a copy, and the
+        host with it, would wait for that whole chain."""
+        host = torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
+        host.copy_(t, non_blocking=True)
+        landed = torch.cuda.Event()
+        landed.record(torch.cuda.current_stream(self.device))
+        return host, landed
+
+    @staticmethod
+    def _landed_numpy(pair):
+        host, landed = pair
+        landed.synchronize()
+        return host.numpy()
 
     def _padded(self, Y):
         """Orders that are not a multiple of 64: diag(Y, I)."""
@@ -666,7 +687,9 @@ class CholeskyQR:
         return self._padded(again) if self.n != self.true_n else again
 
     def _index(self, positions):
-        return torch.as_tensor(np.ascontiguousarray(positions), dtype=torch.int64).to(self.Q.device)
+        # (through pinned memory and without waiting: see _to_host)
+        host = torch.as_tensor(np.ascontiguousarray(positions), dtype=torch.int64).pin_memory()
+        return host.to(self.Q.device, non_blocking=True)
 
     def _finish(self, where, source):
         """The working-set entries `where` (host positions) of `source` are final."""
@@ -694,7 +717,8 @@ class CholeskyQR:
     def check(self):
         if self.swept:
             self.swept = False
-            clean = self.info.cpu().numpy() == 0                                # (a host synchronisation)
+            clean = self._landed_numpy(self.info_host) == 0                     # (waits for the sweep, if it is not through)
+            clean[self.leave] = True
             # the clean matrices are final where they are; only the flagged ones are copied out into a working
             # set of their own and written back when they are done
             self.final = self.Q
@@ -704,6 +728,7 @@ class CholeskyQR:
                 return
         self.gram = gemm(self.Q, self.Q, trans_a=True, symmetric=True)
         self.far = gram_deviation(self.gram)                                    # max |G - I|, ||G - I||_F^2
+        self.far_host = self._to_host(self.far)
 
     def _repair(self, where):
         """The working-set entries `where` (host positions) are far from orthonormal after the sweep: matrices of low
@@ -724,12 +749,12 @@ class CholeskyQR:
         """Host mask over the entries of the last round: the factorisation met a NaN."""
         info, near, ids = self.last
         self.last = None
-        return (info.cpu().numpy()[:ids.size] & 1) != 0, near, ids
+        return (self._landed_numpy(info)[:ids.size] & 1) != 0, near, ids
 
     def poll(self):
         if self.finished:
             return True
-        far = self.far.cpu().numpy()                                            # the host synchronisation
+        far = self._landed_numpy(self.far_host)                                 # the host synchronisation
         failed = np.zeros(self.ids.size, dtype=bool)
         if self.last is not None:
             bad, near, ids = self._failures()
@@ -779,7 +804,7 @@ class CholeskyQR:
         out = torch.empty_like(self.Q)
         solve_upper_right(self.Q, self.U[:k], self.X[:k], self.gram, out)      # the Gram matrix is used up: scratch
         self.Q, self.gram = out, None
-        self.last = (info, self.near.copy(), self.ids.copy())
+        self.last = (self._to_host(info), self.near.copy(), self.ids.copy())
         self.rounds_left -= 1
         self.rounds += 1
         if self.near.any():

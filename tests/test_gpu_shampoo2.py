@@ -669,3 +669,42 @@ def test_a_clean_sweep_means_an_orthonormal_result(mods):
     final, redone = X.cholesky_qr(Y)
     gram = final.double().transpose(1, 2) @ final.double()
     assert float((gram - torch.eye(n, dtype=torch.float64, device="cuda")).abs().max()) <= 5e-5
+
+
+def test_matrices_left_to_the_caller_are_neither_tested_nor_polished(mods):
+    """CholeskyQR(leave=...): the matrices a caller orthonormalises some other way (the eigenbasis bank sweeps its few
+    known low-rank matrices apart from their stack) cost the stack no test, no polishing round and no second sweep,
+    and the other matrices come out with the same bits as without them."""
+    _, E2 = mods
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(5)
+    n = 256
+    good = [torch.randn(n, n, generator=g) for _ in range(5)]
+    low = torch.randn(n, 24, generator=g) @ torch.randn(24, n, generator=g)                # rank 24: the plain sweep cannot finish it
+    Y = torch.stack(good[:2] + [low] + good[2:]).cuda()
+    with_it = X.CholeskyQR(Y.clone())
+    while not with_it.finished:
+        with_it.check()
+        if not with_it.poll():
+            with_it.advance()
+    q_all, _ = with_it.result()
+    assert with_it.repairs == 1 and with_it.repaired_ids == [2]
+    left = X.CholeskyQR(Y.clone(), leave=[2])
+    left.check()
+    assert left.finished and left.rounds == 0 and left.repairs == 0                         # nothing to test: the other sweeps are clean
+    q_left, redone = left.result()
+    keep = [0, 1, 3, 4, 5]
+    assert redone == 0 and torch.equal(q_left[keep], q_all[keep])
+    # and the matrix itself, as a stack of its own that starts with the replacing sweep, ends orthonormal
+    own = X.CholeskyQR(Y[2:3].clone(), replace_first=True)
+    while not own.finished:
+        own.check()
+        if not own.poll():
+            own.advance()
+    q_own, redone = own.result()
+    gram = q_own[0].double().T @ q_own[0].double()
+    assert redone == 0 and float((gram - torch.eye(n, dtype=torch.float64, device="cuda")).abs().max()) <= 5e-5
+    # its leading columns span what the matrix's leading columns span
+    lead = Y[2, :, :16].double()
+    proj = q_own[0, :, :16].double() @ (q_own[0, :, :16].double().T @ lead)
+    assert float((proj - lead).norm() / lead.norm()) <= 1e-4
