@@ -26,7 +26,7 @@ constexpr int NB = 64;
 constexpr int kFactorPanel = 256;      // rows factored between two updates of the whole trailing matrix
 constexpr int kSolvePanel = 256;       // diagonal blocks of the factor are inverted up to this size, then panels of that width are solved
 
-// One wave per matrix: upper Cholesky factor U (G = U^T U) of a 64 x 64 block and U^-1.
+// One workgroup of four waves per matrix: upper Cholesky factor U (G = U^T U) of a 64 x 64 block and U^-1.
 // Reads the upper triangle of G only.  A pivot that is not above `pivot_floor` is a column that depends on
 // the ones before it up to the rounding noise of the Gram matrix.  With pivot_floor > 0 such a column is
 // taken out of the factorisation: its pivot becomes the floor and the rest of its row of U zero (bit 1 of
@@ -40,18 +40,14 @@ constexpr int kSolvePanel = 256;       // diagonal blocks of the factor are inve
 // `set_aside`, if not null: the columns taken out are reported there (bit k of set_aside[b * aside_stride]) instead of in info, and
 // their columns of `inv` are zero, so that Q inv has zero columns in their place for the caller to fill.
 //
-// Lane i keeps row i of the (full, symmetric) trailing matrix in registers.  Step k scales column k
-// (one value per lane) into column k of L = U^T, parks it in LDS, and every lane reads it back as
-// 16-byte broadcasts: the same 64 values update the trailing matrix (a[i][j] -= L[i][k] L[j][k]) and
-// carry the forward substitution for column `lane` of L^-1 (s[j] -= L[j][k] x[k]), so the inverse
-// costs no second pass.  1 / sqrt(pivot) comes from v_rsq_f32 plus one Newton step.  One block = one
-// wave: the wave-level fence below is all the synchronisation the LDS copy needs.
-constexpr int LDC = NB + 4;                      // LDS row stride: rows stay 16-byte aligned
-
-__device__ __forceinline__ float lane_value(float x, int lane) {
-    return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(x), lane));
-}
-
+// Lane i of every wave stands for row i of the (full, symmetric) trailing matrix; wave w keeps the columns 16 w ..
+// 16 w + 15 of that row in registers, and the same columns of the right-hand side e_i of the forward substitution,
+// which ends as column i of L^-1 (L = U^T), so the inverse costs no second pass.  A right-looking factorisation in
+// four blocks of sixteen columns: the wave that owns a block factors it alone (1 / sqrt(pivot) from v_rsq_f32 plus one
+// Newton step; a[i][j] -= L[i][k] L[j][k], s[j] -= L[j][k] x[k] for its own columns j behind k), the waves behind it
+// apply the block's sixteen steps to their columns from the copy in LDS.  (With one wave per matrix and all 64 columns
+// in a lane's registers a step costs twice 64 - k multiply-adds per lane and the kernel 25-29 us; a barrier per step
+// between four waves costs as much in waiting.)
 //
 // SCALED: `gram` is the Gram matrix S = P^T P of a panel whose columns are not of unit length yet.  The kernel factors
 // D^-1 S D^-1 (D = the column lengths, from the diagonal of S) and `inv` receives D^-1 U^-1, so that P inv is the
@@ -60,22 +56,32 @@ __device__ __forceinline__ float lane_value(float x, int lane) {
 // unit column is rounding noise; a NaN counts) is set aside like a dropped one -- it takes no part in the
 // factorisation, its column of inv is zero, its bit of set_aside is set -- whatever aside_pivots says; aside_pivots
 // == 0 keeps the columns dropped for their pivot where they are (bit 1 of info) and reports only the short ones.
+constexpr int LDC = NB + 4;                      // LDS row stride: rows stay 16-byte aligned
+constexpr int kCholWaves = 4, kCholCols = NB / kCholWaves;
+
+__device__ __forceinline__ float lane_value(float x, int lane) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(x), lane));
+}
+
 template <bool SCALED>
-__global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long long g_stride, int ldg, float *u,
-                                                        long long u_stride, int ldu, float *inv, long long inv_stride,
-                                                        int ldi, float *panel_inv, int *info, float pivot_floor,
-                                                        unsigned long long *set_aside, int aside_stride, float too_short,
-                                                        int stand_in, int aside_pivots) {
+__global__ __launch_bounds__(NB * kCholWaves) void cholesky64_kernel(const float *gram, long long g_stride, int ldg, float *u,
+                                                                     long long u_stride, int ldu, float *inv, long long inv_stride,
+                                                                     int ldi, float *panel_inv, int *info, float pivot_floor,
+                                                                     unsigned long long *set_aside, int aside_stride,
+                                                                     float too_short, int stand_in, int aside_pivots) {
     __shared__ __attribute__((aligned(16))) float cols[NB][LDC];
+    __shared__ __attribute__((aligned(16))) float handed[NB][2][NB];      // [k][column k of L | x[k] of every row][row]
     __shared__ float lengths[NB];
-    const int b = blockIdx.x, lane = threadIdx.x;
+    __shared__ unsigned long long s_dropped[kCholWaves];
+    __shared__ int s_failed[kCholWaves];
+    const int b = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c0 = wave * kCholCols;
     const float *G = gram + (long long)b * g_stride;
-    for (int r = 0; r < NB; ++r) cols[r][lane] = G[(long long)r * ldg + lane];
+    for (int r = wave; r < NB; r += kCholWaves) cols[r][lane] = G[(long long)r * ldg + lane];
     __syncthreads();
-    float row[NB];                               // row `lane` of the symmetric matrix; ends as row `lane` of L
-    float s[NB];                                 // right-hand side e_lane of the substitution; ends as column `lane` of L^-1
+    float row[kCholCols];                        // columns c0 .. c0 + 15 of row `lane` of the symmetric matrix; end as L[lane][c0 ..]
+    float s[kCholCols];                          // the same columns of the right-hand side e_lane; end as L^-1[c0 ..][lane]
     float own_scale = 1.0f;                      // SCALED: 1 / length of column `lane` (0 for a column set aside or of length 0)
-    unsigned long long early = 0;                // SCALED: the columns set aside for their length (uniform over the wave)
+    unsigned long long early = 0;                // SCALED: the columns set aside for their length (uniform over the workgroup)
     if constexpr (SCALED) {
         const float norm2 = cols[lane][lane];
         const bool aside = stand_in != 0 && !(norm2 >= too_short);
@@ -89,100 +95,113 @@ __global__ __launch_bounds__(NB) void cholesky64_kernel(const float *gram, long 
             }
         }
         early = __ballot(aside);
-        lengths[lane] = own_scale;
+        if (wave == 0) lengths[lane] = own_scale;
         __syncthreads();
     }
 #pragma unroll
-    for (int j = 0; j < NB; ++j) {
-        row[j] = j >= lane ? cols[lane][j] : cols[j][lane];
+    for (int jj = 0; jj < kCholCols; ++jj) {
+        const int j = c0 + jj;
+        row[jj] = j >= lane ? cols[lane][j] : cols[j][lane];
         if constexpr (SCALED) {
             const bool out = ((early >> j) & 1ull) || ((early >> lane) & 1ull);
-            row[j] = out ? (j == lane ? 1.0f : 0.0f) : row[j] * own_scale * lengths[j];
+            row[jj] = out ? (j == lane ? 1.0f : 0.0f) : row[jj] * own_scale * lengths[j];
         }
-        s[j] = j == lane ? 1.0f : 0.0f;
+        s[jj] = j == lane ? 1.0f : 0.0f;
     }
-    __syncthreads();
     bool ok = true;
-    unsigned long long dropped = 0;              // columns taken out of the factorisation (uniform over the wave)
-    // Step k: pivot, column k of L, then the two next columns at once through v_readlane (they carry the
-    // chain from one pivot to the next); all further columns get the update of step k one step later, from
-    // the copy of column k parked in LDS, so that no pivot ever waits for an LDS round trip.
-    float l_prev = 0.0f, x_prev = 0.0f;
+    uint32_t taken_out = 0;                      // which of its sixteen columns this wave took out of the factorisation (uniform over the wave)
+    // Four phases.  In phase p wave p factors its sixteen columns on its own -- step k: pivot, column k of L, then its
+    // columns behind k at once, their L[j][k] through v_readlane -- and leaves every column of L, with the
+    // substitution's x[k] of every row, in LDS; behind the barrier the waves after it bring their columns up to date
+    // with those sixteen steps (the same multiply-adds in the same order as step by step), and the next one goes on.
 #pragma unroll
-    for (int k = 0; k < NB; ++k) {
-        float4 far[NB / 4];                      // column k-1 of L for the columns from k+2 on
-        if (k >= 1) {
+    for (int p = 0; p < kCholWaves; ++p) {
+        if (wave == p) {                         // (uniform over the wave)
 #pragma unroll
-            for (int j = (k + 2) & ~3; j < NB; j += 4) far[j / 4] = *reinterpret_cast<const float4 *>(&cols[k - 1][j]);
-        }
-        float d = lane_value(row[k], k);
-        bool drop = false;
-        if (!(d > pivot_floor)) {
-            if (pivot_floor > 0.0f && d == d) { drop = true; dropped |= 1ull << k; d = pivot_floor; }
-            else { ok = false; d = 1.0f; }
-        }
-        float r = __builtin_amdgcn_rsqf(d);
-        r = r * __builtin_fmaf(-0.5f * d * r, r, 1.5f);
-        float l = row[k] * r;                    // L[lane][k] (lanes above k: unused values)
-        if (drop) l = lane == k ? d * r : 0.0f;  // sqrt(floor) on the diagonal, nothing below it
-        row[k] = l;
-        s[k] *= r;                               // x[k] = s[k] / L[k][k]
-        const float xk = s[k];
-        cols[k][lane] = l;
+            for (int kk = 0; kk < kCholCols; ++kk) {
+                const int k = p * kCholCols + kk;
+                float d = lane_value(row[kk], k);
+                bool drop = false;
+                if (!(d > pivot_floor)) {
+                    if (pivot_floor > 0.0f && d == d) { drop = true; taken_out |= 1u << kk; d = pivot_floor; }
+                    else { ok = false; d = 1.0f; }
+                }
+                float r = __builtin_amdgcn_rsqf(d);
+                r = r * __builtin_fmaf(-0.5f * d * r, r, 1.5f);
+                float l = row[kk] * r;           // L[lane][k] (lanes above k: unused values)
+                if (drop) l = lane == k ? d * r : 0.0f;   // sqrt(floor) on the diagonal, nothing below it
+                row[kk] = l;
+                s[kk] *= r;                      // x[k] = s[k] / L[k][k]
+                const float xk = s[kk];
+                handed[k][0][lane] = l;
+                handed[k][1][lane] = xk;
 #pragma unroll
-        for (int j = k + 1; j <= k + 2 && j < NB; ++j) {
-            const float v = lane_value(l, j);    // L[j][k]
-            row[j] = __builtin_fmaf(-l, v, row[j]);
-            s[j] = __builtin_fmaf(-v, xk, s[j]);
-        }
-        if (k >= 1) {
-#pragma unroll
-            for (int j = (k + 2) & ~3; j < NB; j += 4) {
-                const float v[4] = {far[j / 4].x, far[j / 4].y, far[j / 4].z, far[j / 4].w};
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (j + e >= k + 2) {
-                        row[j + e] = __builtin_fmaf(-l_prev, v[e], row[j + e]);
-                        s[j + e] = __builtin_fmaf(-v[e], x_prev, s[j + e]);
-                    }
+                for (int jj = kk + 1; jj < kCholCols; ++jj) {
+                    const float v = lane_value(l, p * kCholCols + jj);     // L[j][k]
+                    row[jj] = __builtin_fmaf(-l, v, row[jj]);
+                    s[jj] = __builtin_fmaf(-v, xk, s[jj]);
+                }
             }
         }
-        l_prev = l;
-        x_prev = xk;
-        wave_lds_sync();                         // column k is readable in the next step
+        if (p + 1 == kCholWaves) break;
+        __syncthreads();
+        if (wave > p) {
+#pragma unroll
+            for (int kk = 0; kk < kCholCols; ++kk) {
+                const int k = p * kCholCols + kk;
+                const float l = handed[k][0][lane], xk = handed[k][1][lane];
+#pragma unroll
+                for (int q = 0; q < kCholCols; q += 4) {
+                    const float4 v4 = *reinterpret_cast<const float4 *>(&handed[k][0][c0 + q]);     // L[j][k] for four columns j
+                    const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        row[q + e] = __builtin_fmaf(-l, v[e], row[q + e]);
+                        s[q + e] = __builtin_fmaf(-v[e], xk, s[q + e]);
+                    }
+                }
+            }
+        }
     }
-    float *I = inv + (long long)b * inv_stride + (long long)lane * ldi;
+    if (lane == 0) { s_dropped[wave] = (unsigned long long)taken_out << c0; s_failed[wave] = ok ? 0 : 1; }
+    __syncthreads();
+    unsigned long long dropped = 0;
+    int failed = 0;
+#pragma unroll
+    for (int w = 0; w < kCholWaves; ++w) { dropped |= s_dropped[w]; failed |= s_failed[w]; }
+    float *I = inv + (long long)b * inv_stride + (long long)lane * ldi + c0;
     if constexpr (!SCALED) {
         float *U = u + (long long)b * u_stride;
 #pragma unroll
-        for (int r = 0; r < NB; ++r) U[(long long)r * ldu + lane] = r <= lane ? row[r] : 0.0f;    // U[r][lane] = L[lane][r]
+        for (int jj = 0; jj < kCholCols; ++jj)                                      // U[r][lane] = L[lane][r]
+            U[(long long)(c0 + jj) * ldu + lane] = c0 + jj <= lane ? row[jj] : 0.0f;
     }
     if (set_aside != nullptr) {
         const unsigned long long out = SCALED ? early | (aside_pivots != 0 ? dropped : 0ull) : dropped;
 #pragma unroll
-        for (int c = 0; c < NB; ++c)
-            if ((out >> c) & 1ull) s[c] = 0.0f;
-        if (lane == 0) set_aside[(long long)b * aside_stride] = out;
+        for (int jj = 0; jj < kCholCols; ++jj)
+            if ((out >> (c0 + jj)) & 1ull) s[jj] = 0.0f;
+        if (threadIdx.x == 0) set_aside[(long long)b * aside_stride] = out;
         if (!SCALED || aside_pivots != 0) dropped = 0;
     }
     if constexpr (SCALED) {
 #pragma unroll
-        for (int c = 0; c < NB; ++c) s[c] *= own_scale;                                            // row `lane` of D^-1 U^-1
+        for (int jj = 0; jj < kCholCols; ++jj) s[jj] *= own_scale;                 // row `lane` of D^-1 U^-1
     }
 #pragma unroll
-    for (int c = 0; c < NB; c += 4)              // U^-1[lane][c] = L^-1[c][lane] = s[c] of this lane (zero for c < lane)
-        *reinterpret_cast<float4 *>(I + c) = make_float4(s[c], s[c + 1], s[c + 2], s[c + 3]);
+    for (int jj = 0; jj < kCholCols; jj += 4)    // U^-1[lane][c] = L^-1[c][lane] = s[c] of this lane (zero for c < lane)
+        *reinterpret_cast<float4 *>(I + jj) = make_float4(s[jj], s[jj + 1], s[jj + 2], s[jj + 3]);
     if (!SCALED && panel_inv != nullptr) {
-        float *P = panel_inv + (long long)b * inv_stride + (long long)lane * ldi;
+        float *P = panel_inv + (long long)b * inv_stride + (long long)lane * ldi + c0;
 #pragma unroll
-        for (int c = 0; c < NB; c += 4) {
+        for (int jj = 0; jj < kCholCols; jj += 4) {
             float v[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = (dropped >> (c + e)) & 1ull ? 0.0f : s[c + e];
-            *reinterpret_cast<float4 *>(P + c) = make_float4(v[0], v[1], v[2], v[3]);
+            for (int e = 0; e < 4; ++e) v[e] = (dropped >> (c0 + jj + e)) & 1ull ? 0.0f : s[jj + e];
+            *reinterpret_cast<float4 *>(P + jj) = make_float4(v[0], v[1], v[2], v[3]);
         }
     }
-    if ((!ok || dropped != 0) && lane == 0) info[b] |= (ok ? 0 : 1) | (dropped != 0 ? 2 : 0);
+    if ((failed != 0 || dropped != 0) && threadIdx.x == 0) info[b] |= (failed != 0 ? 1 : 0) | (dropped != 0 ? 2 : 0);
 }
 
 // How far a stack of Gram matrices is from the identity: per matrix max |G - I| and ||G - I||_F^2, in
@@ -435,7 +454,7 @@ extern "C" void qtensor_hip_cholesky_upper_floor_batched(float *gram, float *u, 
             const long long corner = (long long)j0 * n + j0;
             // (the block of u right below the diagonal block is free: it takes the factor for the block row)
             float *panel_inv = rest > 0 ? u + (long long)j1 * n + j0 : nullptr;
-            hipLaunchKernelGGL(cholesky64_kernel<false>, dim3(batch), dim3(NB), 0, stream, gram + corner, mat, n, u + corner, mat, n,
+            hipLaunchKernelGGL(cholesky64_kernel<false>, dim3(batch), dim3(NB * kCholWaves), 0, stream, gram + corner, mat, n, u + corner, mat, n,
                                x + corner, mat, n, panel_inv, info, pivot_floor, (unsigned long long *)nullptr, 0, 0.0f, 0, 0);
             if (!launch_ok("cholesky_upper_batched (diagonal block)")) return;
             if (rest == 0) break;
@@ -568,7 +587,7 @@ struct Sweep {
             return false;
         }
         hipLaunchKernelGGL(panel_product_kernel, dim3(3, batch), dim3(256), 0, stream, panel_ptr, panel_ptr, mat(), n, n, gram, small, 1);
-        hipLaunchKernelGGL(cholesky64_kernel<true>, dim3(batch), dim3(NB), 0, stream, gram, small, NB, (float *)nullptr, small, NB, x,
+        hipLaunchKernelGGL(cholesky64_kernel<true>, dim3(batch), dim3(NB * kCholWaves), 0, stream, gram, small, NB, (float *)nullptr, small, NB, x,
                            small, NB, (float *)nullptr, info, floor_here, aside, w_cols / NB, too_short, stand_in ? 1 : 0,
                            replace && more ? 1 : 0);
         if (!launch_ok("block_gram_schmidt_batched (panel factor)")) return false;
