@@ -116,6 +116,8 @@ def precond_step_gpu(torch, variant="shampoo1"):
     import importlib
     S = importlib.import_module("optimizers." + variant)
 
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()               # what earlier parts of this run still hold: not this workload's
     g = torch.Generator(device="cuda").manual_seed(1)
     params = [torch.nn.Parameter(0.02 * torch.randn(s, device="cuda", generator=g)) for s in vit_b32_shapes()]
     grad_sets = [[0.02 * torch.randn(p.shape, device="cuda", generator=g) for p in params] for _ in range(4)]
@@ -181,10 +183,11 @@ def precond_step_gpu(torch, variant="shampoo1"):
         "ms_per_step_amortized_over_10": round((9 * reg + new) / 10, 3),
         "device_ms_regular": round(mean(regular, 1), 3),
         "device_ms_with_inverse_roots": round(mean(newton, 1), 3),
-        "device_memory_gib": {"allocated_between_steps": round(resident / 2 ** 30, 2),
-                              "peak_inside_a_step": round(max(peak.values()) / 2 ** 30, 2),
-                              "peak_inside_a_regular_step": round(peak["regular"] / 2 ** 30, 2),
-                              "peak_inside_a_step_with_inverse_roots": round(peak["roots"] / 2 ** 30, 2),
+        "device_memory_gib": {"allocated_between_steps": round((resident - before) / 2 ** 30, 2),
+                              "peak_inside_a_step": round((max(peak.values()) - before) / 2 ** 30, 2),
+                              "peak_inside_a_regular_step": round((peak["regular"] - before) / 2 ** 30, 2),
+                              "peak_inside_a_step_with_inverse_roots": round((peak["roots"] - before) / 2 ** 30, 2),
+                              "held_by_earlier_parts_of_the_run_and_left_out": round(before / 2 ** 30, 2),
                               "of_which_parameters_and_the_four_gradient_sets": round(5 * sum(p.numel() for p in params) * 4 / 2 ** 30, 2)},
         "product_gflop_per_regular_step": round(2 * gram_flop / 1e9, 1),
         "product_tflops_regular": round(2 * gram_flop / (mean(regular, 1) * 1e-3) / 1e12, 1),
