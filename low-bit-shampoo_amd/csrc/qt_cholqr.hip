@@ -4,7 +4,7 @@
 // (torch.linalg.qr at qtensor/utils.py:157 of the reference).
 //
 // The only arithmetic done outside the matrix-core GEMM (qtensor_hip_gemm) is the 64 x 64 diagonal
-// block: one wave per matrix factors it in registers and also inverts the factor.
+// block: four waves per matrix factor it in registers and also invert the factor.
 //   factor:  for each block row j:  U_jj = chol(G_jj);  U_j,> = U_jj^-T G_j,>;  G_>,> -= U_j,>^T U_j,>
 //            (the last step for the rows of the current 256-row panel at once, for the rest per panel)
 //   solve :  the inverted diagonal blocks are doubled up to 256 x 256 -- with blocks A, C already
