@@ -485,33 +485,42 @@ _COMPLETION = {}                 # (device index, order) -> fixed matrix of unit
 NULL_COLUMN_NORM2 = 1e-11        # what a projection leaves of a unit column that depends on the earlier ones: rounding noise
 
 
-def completion_columns(device: torch.device, n: int) -> Tensor:
+def completion_columns(device: torch.device, n: int, true_n: int = None) -> Tensor:
     """[n, n] fixed pseudo-random unit columns (the same for every call): stand-ins for the columns of a
-    rank-deficient matrix that are rounding noise once the columns before them are taken out."""
-    key = (device.index, n)
+    rank-deficient matrix that are rounding noise once the columns before them are taken out.  true_n < n: the
+    matrices are diag(Y, I) with Y of order true_n (orders padded to a multiple of 64) and so are the stand-ins,
+    diag(F, I): a stand-in for a column of Y has nothing in the padding rows, or the part of Q that is handed back,
+    its leading true_n x true_n block, would not be orthonormal."""
+    true_n = n if true_n is None else true_n
+    key = (device.index, n, true_n)
     if key not in _COMPLETION:
         gen = torch.Generator(device=device).manual_seed(0x5eed + n)
         r = torch.randn(n, n, device=device, generator=gen)
+        if true_n < n:
+            r[true_n:, :true_n] = 0.0
+            r[:, true_n:] = 0.0
+            r.diagonal()[true_n:] = 1.0
         _COMPLETION[key] = (r / torch.linalg.vector_norm(r, dim=0, keepdim=True)).contiguous()
     return _COMPLETION[key]
 
 
 def block_gram_schmidt(q: Tensor, info: Tensor, pivot_floor: float = 2e-4, null_norm2: float = NULL_COLUMN_NORM2,
-                       complete: bool = True, replace_dependent: bool = False) -> Tensor:
+                       complete: bool = True, replace_dependent: bool = False, true_n: int = None) -> Tensor:
     """Orthonormalise the columns of every matrix of the stack q [B, n, n] (unit columns, n a multiple of 64)
     in place, left to right in panels of 64 columns: block Gram-Schmidt with reorthogonalisation, Cholesky QR
     inside a panel.  span(q[:, :, :k]) is kept for every k.  complete: columns that depend on the earlier ones
     up to rounding noise are replaced by fixed unit columns in general position (bit 2 of info[b]); info int32
     [B], zeroed by the caller, bits as in cholesky_upper.  replace_dependent (needs complete): a column that the
     first pass finds dependent inside its 64-column panel (pivot at or below pivot_floor) is replaced as well,
-    instead of being handed to the second pass as it is -- for matrices of low numerical rank."""
+    instead of being handed to the second pass as it is -- for matrices of low numerical rank.  true_n < n: the
+    matrices are diag(Y, I) with Y of order true_n, and the stand-in columns keep that form (completion_columns)."""
     B, n, _ = q.shape
     _stack(q, "q", (B, n, n))
     if info.dtype != torch.int32 or info.numel() != B or not info.is_cuda:
         raise ValueError("info must be an int32 GPU vector with one entry per matrix")
     w = torch.empty(B, n, F.lib.qtensor_hip_block_gram_schmidt_width(), device=q.device)
     small = torch.empty(3, B, 64, 64, device=q.device)
-    fill = completion_columns(q.device, n) if complete else None
+    fill = completion_columns(q.device, n, true_n) if complete else None
     if replace_dependent and fill is None:
         raise ValueError("replace_dependent needs complete=True")
     F._call(F.lib.qtensor_hip_block_gram_schmidt_replacing_batched, q.device, q.data_ptr(), w.data_ptr(), small[0].data_ptr(),
@@ -650,7 +659,7 @@ class CholeskyQR:
             # fp32 rounding by construction; the rounds below are for the other matrices only.
             # replace_first: the caller knows the stack to be of low numerical rank (its last update needed the
             # replacing sweep for most matrices) and goes there directly
-            block_gram_schmidt(self.Q, self.info, pivot_floor, replace_dependent=replace_first)
+            block_gram_schmidt(self.Q, self.info, pivot_floor, replace_dependent=replace_first, true_n=self.true_n)
             if replace_first:
                 self.mended[:] = True
             self.info_host = self._to_host(self.info)
@@ -740,7 +749,7 @@ class CholeskyQR:
         scale = torch.linalg.vector_norm(original, dim=1, keepdim=True).clamp_min(1e-30)
         again = (original / scale).contiguous()
         info = torch.zeros(again.shape[0], dtype=torch.int32, device=again.device)
-        block_gram_schmidt(again, info, self.pivot_floor, replace_dependent=True)
+        block_gram_schmidt(again, info, self.pivot_floor, replace_dependent=True, true_n=self.true_n)
         self.Q.index_copy_(0, self._index(where), again)
         self.repairs += int(where.size)
         self.repaired_ids += [int(i) for i in self.ids[where]]

@@ -708,3 +708,24 @@ def test_matrices_left_to_the_caller_are_neither_tested_nor_polished(mods):
     lead = Y[2, :, :16].double()
     proj = q_own[0, :, :16].double() @ (q_own[0, :, :16].double().T @ lead)
     assert float((proj - lead).norm() / lead.norm()) <= 1e-4
+
+
+@pytest.mark.parametrize("n", [100, 200, 832])
+def test_stand_in_columns_of_a_padded_order_stay_inside_the_matrix(mods, n):
+    """Orders that are not a multiple of 64 are factored as diag(Y, I).  A stand-in column for a dependent column of Y
+    must have nothing in the padding rows, or the leading n x n block that is handed back is not orthonormal (a
+    stand-in in general position of the padded space loses n / n_padded of its length there)."""
+    _, E2 = mods
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(n)
+    dep = torch.randn(2, n, n, generator=g)
+    dep[:, :, n // 2] = dep[:, :, 1] * 2.0                                     # one column repeats an earlier one
+    low = torch.randn(2, n, n // 4, generator=g) @ torch.randn(2, n // 4, n, generator=g)   # and a stack of rank n / 4
+    for Y in (dep.cuda(), low.cuda()):
+        Q, redone = X.cholesky_qr(Y)
+        gram = Q.double().transpose(1, 2) @ Q.double()
+        assert float((gram - torch.eye(n, dtype=torch.float64, device="cuda")).abs().max()) <= 5e-5
+        k = n // 8                                                             # the leading columns still span what Y's span
+        lead = Y[:, :, :k].double()
+        proj = Q[:, :, :k].double() @ (Q[:, :, :k].double().transpose(1, 2) @ lead)
+        assert float((proj - lead).norm() / lead.norm()) <= 1e-4
