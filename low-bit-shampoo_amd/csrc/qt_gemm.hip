@@ -1605,8 +1605,10 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
     // to the caller's workspace and are summed in order afterwards.  Same cost model, with a fixed cost per
     // workgroup (prologue, epilogue, the extra pass over the output) worth about 64 k steps.
     a.split_k = 1;
+    // (not with skip flags: the launch that adds the slices up would write the sum of slices nobody computed into the
+    // results that are to be left alone)
     if (ep == kStore && !a.symmetric && a.batch_inner <= 1 && a.triangular == 0 && a.workspace != nullptr && d->K % 16 == 0 &&
-        is_aligned(a.workspace, 16)) {
+        is_aligned(a.workspace, 16) && a.skip == nullptr) {
         const Shape &sh = shapes[pick];
         const double units = compute_units();
         const long long tm = (d->M + sh.bm - 1) / sh.bm, tn = (d->N + sh.bn - 1) / sh.bn;

@@ -179,8 +179,9 @@ def gemm(A, B, *, trans_a=False, trans_b=False, out: Optional[Tensor] = None, al
          upper_a: bool = False, upper_b: bool = False, requantize: bool = False, pipe: Optional[str] = None):
     """out[b] = epilogue(op(A[b]) @ op(B[b])).
 
-    A, B: fp32 tensors ([m,k] / [batch,m,k]; with trans_x the stored matrix is the transpose) or a
-    `Quantized` (square; then the other operand must be dense).
+    A, B: fp32 tensors ([m,k] / [batch,m,k]; with trans_x the stored matrix is the transpose; trans_a together
+    with trans_b is not built: that product is the transpose of B A) or a `Quantized` (square; then the other
+    operand must be dense).
     addend: None, a dense tensor E or a `Quantized` E: out = beta*E + alpha*product.
     newton: None or (T_out, w, err): also writes T_out = (1-w) I + w*product and folds
     max|product - I| into err[b] (fp32 [batch], zeroed by the caller).

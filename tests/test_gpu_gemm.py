@@ -513,3 +513,24 @@ def test_split_pipe_at_the_top_of_the_fp32_range(mods):
     out = X.gemm(A, Bm, pipe="split")
     assert bool(out[0, 5].isnan().all()) and bool(torch.isfinite(out[0, 4]).all()) and bool(torch.isfinite(out[0, 9]).all())
     assert bool(torch.isfinite(X.gemm(A, Bm, pipe="f32")).all())
+
+
+@pytest.mark.parametrize("m,n,k,batch", [(17, 63, 768, 1), (500, 63, 640, 3), (64, 1000, 512, 2), (5, 5, 1024, 5)])
+def test_skipped_entries_stay_untouched_when_k_is_long(mods, m, n, k, batch):
+    """Plain-store products with few output tiles and a long k range are cut along k into slices that a second launch
+    adds up.  With skip flags that second launch would write sums of slices nobody computed into the entries that are
+    to be left alone, so such products are not cut."""
+    _, X = mods
+    g = torch.Generator().manual_seed(m + n + k)
+    A, B = torch.randn(batch, m, k, generator=g).cuda(), torch.randn(batch, k, n, generator=g).cuda()
+    want = (A.double() @ B.double()).cpu()
+    for pipe in ("f32", "split"):
+        for pattern in (0, 1):
+            skip = torch.tensor([(b + pattern) % 2 for b in range(batch)], dtype=torch.int32).cuda()
+            out = torch.full((batch, m, n), 7.0, device="cuda")
+            X.gemm(A, B, out=out, skip=skip, pipe=pipe)
+            for b in range(batch):
+                if int(skip[b]):
+                    assert bool((out[b] == 7.0).all()), (pipe, b)
+                else:
+                    assert rel_err(out[b], want[b]) <= TOL, (pipe, b)
