@@ -296,7 +296,8 @@ void qtensor_hip_cholesky_upper_floor_batched(float *gram, float *u, float *x, i
  * that pass as a zero column and enters the second one as the same column of fill (bit 2 of info[b]); the last
  * 4 * batch floats of w then hold which columns those are.  w: scratch [batch, n, width]; gram, x: scratch
  * [batch, 64, 64] each; u: not used any more (kept in the signature); info as in cholesky_upper_floor (zeroed by the
- * caller). */
+ * caller), where bit 1 also stands for a column that the last pass over its panel found shortened to less than half and
+ * lifted back to unit length: such a matrix can be off by the rounding error over what was left and wants a test. */
 int qtensor_hip_block_gram_schmidt_width(void);
 void qtensor_hip_block_gram_schmidt_batched(float *q, float *w, float *gram, float *u, float *x, const float *fill, int *info,
                                             int n, int batch, float pivot_floor, float null_norm2, qtensor_stream_t stream);

@@ -82,6 +82,7 @@ __global__ __launch_bounds__(NB * kCholWaves) void cholesky64_kernel(const float
     float s[kCholCols];                          // the same columns of the right-hand side e_lane; end as L^-1[c0 ..][lane]
     float own_scale = 1.0f;                      // SCALED: 1 / length of column `lane` (0 for a column set aside or of length 0)
     unsigned long long early = 0;                // SCALED: the columns set aside for their length (uniform over the workgroup)
+    bool shrunk = false;                         // SCALED: a column kept although the projections left little of it
     if constexpr (SCALED) {
         const float norm2 = cols[lane][lane];
         const bool aside = stand_in != 0 && !(norm2 >= too_short);
@@ -95,6 +96,12 @@ __global__ __launch_bounds__(NB * kCholWaves) void cholesky64_kernel(const float
             }
         }
         early = __ballot(aside);
+        // Without stand-ins (the last pass over a panel) a column that the projections have shortened that much is
+        // kept and lifted back to unit length, and whatever rounding left in it with it: the result can be off by
+        // the rounding error over what was left, so the matrix is flagged (bit 1 of info) and the caller tests it.
+        // (A column that depends on the ones before it gets here when an earlier pass could not tell: next to an
+        // ill-conditioned panel that one Cholesky QR round had not made orthonormal yet.)
+        shrunk = stand_in == 0 && __ballot(!(norm2 >= too_short)) != 0;
         if (wave == 0) lengths[lane] = own_scale;
         __syncthreads();
     }
@@ -201,7 +208,7 @@ __global__ __launch_bounds__(NB * kCholWaves) void cholesky64_kernel(const float
             *reinterpret_cast<float4 *>(P + jj) = make_float4(v[0], v[1], v[2], v[3]);
         }
     }
-    if ((failed != 0 || dropped != 0) && threadIdx.x == 0) info[b] |= (failed != 0 ? 1 : 0) | (dropped != 0 ? 2 : 0);
+    if ((failed != 0 || dropped != 0 || shrunk) && threadIdx.x == 0) info[b] |= (failed != 0 ? 1 : 0) | (dropped != 0 || shrunk ? 2 : 0);
 }
 
 // How far a stack of Gram matrices is from the identity: per matrix max |G - I| and ||G - I||_F^2, in

@@ -729,3 +729,37 @@ def test_stand_in_columns_of_a_padded_order_stay_inside_the_matrix(mods, n):
         lead = Y[:, :, :k].double()
         proj = Q[:, :, :k].double() @ (Q[:, :, :k].double().transpose(1, 2) @ lead)
         assert float((proj - lead).norm() / lead.norm()) <= 1e-4
+
+
+def test_a_dependent_column_next_to_an_ill_conditioned_panel_is_flagged(mods):
+    """A column that depends on the 64 columns before it sits in the second 64-column panel of its 128-column outer
+    panel.  In the first pass that first panel has had one Cholesky QR round only (orthonormal to rounding times its
+    squared conditioning), so what the projection leaves of the column is far above rounding noise and nobody can
+    tell that it is dependent; the last pass then finds next to nothing left of it, lifts that back to unit length,
+    and the result is off by rounding over what was left.  The sweep must flag such a matrix (so that it is tested
+    and polished): whatever it reports clean is orthonormal, and the solver's result always is."""
+    _, E2 = mods
+    import qtensor.fused as X
+    g = torch.Generator().manual_seed(64)
+    mats = []
+    for n, r in ((65, 64), (65, 64), (128, 64), (100, 70), (130, 64)):
+        for _ in range(6):
+            mats.append((n, torch.randn(n, r, generator=g) @ torch.randn(r, n, generator=g)))
+    flagged = 0
+    for n, Y in mats:
+        Y = Y.unsqueeze(0).cuda()
+        s = X.CholeskyQR(Y)
+        info = int(s.info.cpu()[0])
+        swept = s.Q[0].double()
+        off = float((swept.T @ swept - torch.eye(swept.shape[0], dtype=torch.float64, device="cuda")).abs().max())
+        if info == 0:
+            assert off <= 2e-5, (n, off)
+        flagged += info != 0
+        while not s.finished:
+            s.check()
+            if not s.poll():
+                s.advance()
+        Q, redone = s.result()
+        gram = Q[0].double().T @ Q[0].double()
+        assert float((gram - torch.eye(n, dtype=torch.float64, device="cuda")).abs().max()) <= 5e-5
+    assert flagged >= len(mats) // 2                                        # these matrices are rank deficient: most must be flagged
