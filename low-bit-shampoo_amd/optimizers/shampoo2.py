@@ -54,7 +54,6 @@ class Preconditioner(PreconditionerBase):
 
 class _Fused2(_FusedStep):
     bank_keys = ('rect_t1', 'rect_t2', 'inv_root_mode')
-    overlap_unbatched_statistics = True      # a statistics update here is a QR: rounds with a device wait each
     overlap_precondition = True              # the stored roots are applied to the gradients next to the factorisations
 
     @staticmethod
