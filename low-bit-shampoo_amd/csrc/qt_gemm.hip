@@ -622,7 +622,7 @@ constexpr int kWavesPerSimd = (PREC == kPipeSplit && BM == 128 && BN == 128 &&
                                (KA >= kQuant4 || KB >= kQuant4 || EPI == kRequant8)) ? 2 : 3;   // (the 256-entry tables of the 8-bit re-encoding leave LDS for two)
 
 template <int BM, int BN, int KA, int KB, int EPI, int PREC = kPipeF32>
-__global__ __launch_bounds__(256, (kWavesPerSimd<BM, BN, KA, KB, EPI, PREC>)) void gemm_kernel(const GemmArgs args) {   // three waves per SIMD: at most 168 registers
+__global__ __launch_bounds__(256, (kWavesPerSimd<BM, BN, KA, KB, EPI, PREC>)) void gemm_kernel(const GemmArgs args) {   // three waves per SIMD mean at most 168 registers, two 256
     constexpr int WM = BM / 2, WN = BN / 2, MI = WM / 32, NI = WN / 32;
     // Workgroups are dealt round-robin to the 8 accelerator dies, each with its own L2.  Renumber
     // them so that every die works through one contiguous run of (batch entry, tile row, tile
