@@ -34,8 +34,9 @@ cholesky_qr = X.cholesky_qr
 
 
 class ShampooBank2(ShampooBank):
-    # Measured on the ViT-B/32 shapes (four orders, four hardware queues per process): 22.3 ms per regular step with
-    # three or four side streams, 23.6 with two.
+    # Two lanes for the large stacks, one for the small ones, one for the few matrices that are swept apart from
+    # their stack (a process has four hardware queues; on the ViT-B/32 shapes fewer side streams cost a millisecond
+    # or two per regular step, more gain nothing).
     DEFAULT_STREAMS = 4
 
     def __init__(self, params, name2qmap, code, *, rect_t1=1, rect_t2=4, inv_root_mode=0, **kwargs):
@@ -70,7 +71,7 @@ class ShampooBank2(ShampooBank):
         """The matrices of this stack that are, for this update, taken to be of low numerical rank: those whose recent
         updates ended in the replacing sweep (the order-768 statistic of a 768 x 100 head: rank 100 plus the kept half).
         Up to APART_AT_MOST of them are orthonormalised apart from their stack, as a small stack of their own that starts
-        with the replacing sweep, on the lane of the small stacks, while the stack itself gets the plain sweep and
+        with the replacing sweep, on a stream next to the lanes, while the stack itself gets the plain sweep and
         leaves their places alone; with more of them the whole stack starts with the replacing sweep.  Every `period`
         updates such a matrix goes through the plain sweep with its stack again; the period doubles (8, 16, ... 256)
         each time that look ends in the replacing sweep once more."""
