@@ -64,8 +64,9 @@ def shared_stream(device, slot):
 
 
 class SideJob:
-    """Runs fn() on a thread and a stream of its own, ordered after what the current stream holds now;
-    join() makes the current stream wait for it and passes an exception on."""
+    """Runs fn() on a thread of its own with `stream` as that thread's current stream, ordered after what the
+    caller's current stream holds now (`stream` may be that very stream: then only the queueing is done
+    elsewhere); join() makes the caller's stream wait for it and passes an exception on."""
 
     def __init__(self, device, stream, fn):
         self.main, self.side, self.error = torch.cuda.current_stream(device), stream, None
