@@ -204,9 +204,6 @@ class ShampooBank2(ShampooBank):
                     apart_y[order] = product.index_select(0, self._row_index(apart[order]))
                     apart_event[order] = torch.cuda.Event()
                     apart_event[order].record(torch.cuda.current_stream(self.device))
-                # (the rectified basis came from another stream's job: its memory must not be handed out again on that
-                # stream before this one has read it)
-                basis[order].record_stream(torch.cuda.current_stream(self.device))
                 basis[order] = None
                 solver[order] = X.CholeskyQR(product, replace_first=direct[order], remake=remake, leave=apart[order])
                 del product
@@ -249,9 +246,11 @@ class ShampooBank2(ShampooBank):
                     self.basis[order].put(rows, X.store_stack(chosen, self.basis[order].select(rows), transposed=True))
             return run
 
-        self._fan_out([rebuild(o) for o in orders])
-        self._fan_out([accumulate(g, side) for g in self.groups for side in (0, 1)
-                       if only is None or any(pi in only for pi in g.param_index)])
+        gradient_terms = {o: [] for o in orders}              # order -> the products G G^T / G^T G that go into its stack
+        for g in self.groups:
+            if only is None or any(pi in only for pi in g.param_index):
+                for side in (0, 1):
+                    gradient_terms[g.slot[side][0]].append(accumulate(g, side))
         # The Cholesky QR of every order advances on its own stream; the host waits once per round.
         # (_fan_out gives job i the stream i % streams, so an order keeps its stream from call to call.)
         # Two lanes for the sweeps and what follows them, a third for stacks of a matrix or two: a process has four
@@ -299,7 +298,20 @@ class ShampooBank2(ShampooBank):
                 tick[key].record(current)
             return run
 
-        jobs = [(lambda lane=lane: [project(o)() for o in lane]) for lane in lanes]
+        def chain(lane):
+            def run():
+                # a stack is rebuilt, takes its gradient terms, is multiplied out and swept on its lane, one stack of
+                # the lane after the other; the lanes start together and nothing waits for another lane on the way
+                # (the second lane held back until the first one's large products are through, so that they fill the
+                # device next to the other lane's sweep and not next to each other, is a millisecond slower per step)
+                for o in lane:
+                    rebuild(o)()
+                    for job in gradient_terms[o]:
+                        job()
+                    project(o)()
+            return run
+
+        jobs = [chain(lane) for lane in lanes]
         if any(apart.values()):
             own = [sweep_apart(o) for o in orders if apart[o]]
             jobs.append(lambda: [job() for job in own])
