@@ -1608,8 +1608,12 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
     a.split_k = 1;
     // (not with skip flags: the launch that adds the slices up would write the sum of slices nobody computed into the
     // results that are to be left alone)
+    // (nor a quantized left factor with k up to 1024: measured on 36 to 144 output tiles, the product that is not cut
+    // -- smaller tiles, three workgroups per unit -- takes 31-55 us where runs of k tiles and the launch that sums the
+    // pieces take 35-57; from k = 1536 on the cut wins by a quarter and more, and so it does for a quantized right factor)
+    const bool short_left = ka >= kQuant4 && d->K <= 1024;
     if (ep == kStore && !a.symmetric && a.batch_inner <= 1 && a.triangular == 0 && a.workspace != nullptr && d->K % 16 == 0 &&
-        is_aligned(a.workspace, 16) && a.skip == nullptr) {
+        is_aligned(a.workspace, 16) && a.skip == nullptr && !short_left) {
         const Shape &sh = shapes[pick];
         const double units = compute_units();
         const long long tm = (d->M + sh.bm - 1) / sh.bm, tn = (d->N + sh.bn - 1) / sh.bn;
