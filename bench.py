@@ -233,7 +233,7 @@ PRODUCT_TRAFFIC_SOURCE = ("profiles/dense_stack_product_99x1024_kernel_stats_and
 
 def fused_gemm_gpu(torch, code):
     """deq(Lq) @ G @ deq(Rq) for G 768 x 3072, Lq 768^2 and Rq 3072^2 stored 4-bit / blocksize 64 with exact
-    diagonals: the two fused products, timed with events on the launch stream."""
+    diagonals: the two fused products (three launches), timed with events on the launch stream."""
     import qtensor.fused as X
     g = torch.Generator(device="cuda").manual_seed(3)
     m, n = 768, 3072
@@ -256,16 +256,18 @@ def fused_gemm_gpu(torch, code):
     flop = 2.0 * m * m * n + 2.0 * m * n * n
 
     def rate():
-        for _ in range(10):
+        # (a hundred untimed runs first: the products are short, and the clock takes tens of milliseconds to settle;
+        # then fifty runs back to back between one pair of events, as a step would issue them)
+        for _ in range(100):
             run()
-        reps = 20
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
-        ev[0].record()
-        for i in range(reps):
+        reps = 50
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
             run()
-            ev[i + 1].record()
+        e1.record()
         torch.cuda.synchronize()
-        ms = sum(ev[i].elapsed_time(ev[i + 1]) for i in range(reps)) / reps
+        ms = e0.elapsed_time(e1) / reps
         return ms, flop / (ms * 1e-3) / 1e12
 
     before = X.gemm_pipe("f32")
