@@ -20,6 +20,7 @@
 #include <initializer_list>
 
 namespace qt {
+void gemm_with_tile(const qtensor_gemm_desc *d, hipStream_t stream, int tile);     // qt_gemm.hip
 namespace {
 
 constexpr int NB = 64;
@@ -426,6 +427,13 @@ bool run(qtensor_gemm_desc &d, hipStream_t stream) {
     return qtensor_hip_last_error() == 0;
 }
 
+// The same with the tile shape chosen here (0 = 128 x 128, 2 = 64 x 128): for the sweep's projections, where measured
+// times and the product kernel's cost model part ways.
+bool run_tiled(qtensor_gemm_desc &d, hipStream_t stream, int tile) {
+    gemm_with_tile(&d, stream, tile);
+    return qtensor_hip_last_error() == 0;
+}
+
 bool stack_args_ok(const char *what, int n, int batch, std::initializer_list<const void *> ptrs) {
     for (const void *p : ptrs)
         if (!p) { set_error(kNullPointer, "%s: null pointer", what); return false; }
@@ -543,7 +551,13 @@ struct Sweep {
             p.args.workspace = w + w_used;
             p.args.workspace_floats = w_all - w_used;
         }
-        if (!run(p, stream)) return false;
+        // Tile shapes by measurement (a stack of 99 matrices of order 1024, seven outer panels of a pass): the coefficients
+        // -- few output tiles, a long k -- take 685 us with tiles of 128 x 128 (cut along k where that shape leaves units
+        // idle) against 773 with what the product's cost model picks; the application 771 us with tiles of 64 rows and the
+        // panel's full width against 800 (136 of order 768: 389 against 441 and 424 against 448; 50 of order 1024: 384
+        // against 419 and 388 against 435).  Smaller stacks are left to the model, which is as good or better there.
+        const bool wide = width == 2 * NB && (long long)batch * n >= 49152;
+        if (!(wide ? run_tiled(p, stream, 0) : run(p, stream))) return false;
         qtensor_gemm_desc r = {};                             // Y -= Q_a W
         r.M = n; r.N = width; r.K = k; r.batch = batch;
         r.kind_a = QTENSOR_DENSE; r.kind_b = QTENSOR_DENSE; r.epilogue = QTENSOR_EPI_AXPBY_DENSE;
@@ -552,7 +566,7 @@ struct Sweep {
         r.args.C = strided(q + c0, mat()); r.args.ldc = n;
         r.args.E = strided(q + c0, mat()); r.args.lde = n;
         r.args.alpha = -1.0f; r.args.beta = 1.0f;
-        return run(r, stream);
+        return wide ? run_tiled(r, stream, 2) : run(r, stream);
     }
 
     // The 64 columns from c0 on, in pass `pass` of `passes` over their outer panel (which starts at column a0): take the

@@ -1419,7 +1419,7 @@ StaticScratch *static_scratch() {
     return &slot;
 }
 
-void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream);
+void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream, int tile_hint = -1);
 
 // Process-wide choice of the matrix pipe (qtensor_hip_gemm_pipe); starts from the
 // environment variable QT_GEMM_PIPE ("f32" or "split"), else the split pipe.
@@ -1508,8 +1508,19 @@ extern "C" void qtensor_hip_gemm_static(const qtensor_gemm_desc *d, void *stream
     }
 }
 
+// For callers inside the library that know their shapes better than the cost model below (the sweep's narrow
+// projections): the product with the tile shape given, 0..3 = 128 x 128, 128 x 64, 64 x 128, 64 x 64.  The bits of a
+// product do not depend on its tiles, only on whether k is cut, which is still decided for that shape.
+namespace qt {
+void gemm_with_tile(const qtensor_gemm_desc *d, hipStream_t stream, int tile);
+}
+void qt::gemm_with_tile(const qtensor_gemm_desc *d, hipStream_t stream, int tile) {
+    qt::clear_error();
+    gemm_dispatch(d, stream, tile);
+}
+
 namespace {
-void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
+void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream, int tile_hint) {
     using namespace qt;
     if (!d) { set_error(kNullPointer, "gemm: null descriptor"); return; }
     GemmArgs a = d->args;
@@ -1584,6 +1595,8 @@ void gemm_dispatch(const qtensor_gemm_desc *d, hipStream_t stream) {
         int fm = 0, fn = 0;
         if (sscanf(forced, "%dx%d", &fm, &fn) == 2)
             for (int i = 0; i < 4; ++i) if (shapes[i].bm == fm && shapes[i].bn == fn) pick = i;
+    } else if (tile_hint >= 0 && tile_hint < 4) {
+        pick = tile_hint;
     } else {
         const double units = compute_units();
         double best = 0.0;
