@@ -48,6 +48,20 @@ class ShampooBank2(ShampooBank):
         self.low_rank = {}                        # order -> [most of the stack needed the replacing sweep, updates since the plain one was tried]
         self.low_rank_rows = {}                   # order -> {row: [updates between two looks at the plain sweep, updates until the next look]}
         super().__init__(params, name2qmap, code, **kwargs)
+        # Statistics that cannot have full rank, whatever the gradients: the update of a block's statistic of order n is
+        # b * (its kept half: rank n // 2) + (1 - b) * G G^T with G n x m, so its rank is at most n // 2 + m -- the order-768
+        # statistic of a 768 x 256 block has a null space of 128 dimensions in every update.  order -> rows of its stack
+        self.rank_deficient = self._rank_deficient_rows(self.groups)
+
+    @staticmethod
+    def _rank_deficient_rows(groups):
+        rows = {}
+        for g in groups:
+            for side, (order, other) in enumerate(((g.bm, g.bn), (g.bn, g.bm))):
+                if max(1, order // 2) + other < order:
+                    first = g.slot[side][1]
+                    rows.setdefault(order, []).extend(range(first, first + len(g)))
+        return {order: sorted(r) for order, r in rows.items()}
 
     QUOTIENT_PART_BYTES = 128 << 20               # L Q for the Rayleigh quotients is formed this much at a time
     LOOK_AGAIN = 8                                # updates after which a stack of low numerical rank tries the plain sweep again
@@ -65,21 +79,22 @@ class ShampooBank2(ShampooBank):
             return False
         return True
 
-    APART_AT_MOST = 8                             # so many known low-rank matrices of a stack are still orthonormalised on their own
+    APART_AT_MOST = 32                            # so many known low-rank matrices of a stack are still orthonormalised on their own
 
     def _known_low_rank(self, order):
-        """The matrices of this stack that are, for this update, taken to be of low numerical rank: those whose recent
-        updates ended in the replacing sweep (the order-768 statistic of a 768 x 100 head: rank 100 plus the kept half).
-        Up to APART_AT_MOST of them are orthonormalised apart from their stack, as a small stack of their own that starts
-        with the replacing sweep, on a stream next to the lanes, while the stack itself gets the plain sweep and
-        leaves their places alone; with more of them the whole stack starts with the replacing sweep.  Every `period`
-        updates such a matrix goes through the plain sweep with its stack again; the period doubles (8, 16, ... 256)
-        each time that look ends in the replacing sweep once more."""
-        known = []
+        """The matrices of this stack that are, for this update, taken to be of low numerical rank: those that cannot
+        have full rank by the shape of their block (rank_deficient: the order-768 statistics of a 768 x 100 head and of
+        the 768 x 256 blocks of a 768 x 2304 weight), and those whose recent updates ended in the replacing sweep.
+        Up to APART_AT_MOST of them (and at most a quarter of the stack) are orthonormalised apart from their stack, as a
+        small stack of their own that starts with the replacing sweep, on a stream next to the lanes, while the stack
+        itself gets the plain sweep and leaves their places alone; with more of them the whole stack starts with the
+        replacing sweep.  Every `period` updates a matrix of the second kind goes through the plain sweep with its stack
+        again; the period doubles (8, 16, ... 256) each time that look ends in the replacing sweep once more."""
+        known = set(self.rank_deficient.get(order, ()))
         for row, state in self.low_rank_rows.setdefault(order, {}).items():
             if state[1] > 0:
                 state[1] -= 1
-                known.append(row)
+                known.add(row)
         return sorted(known)
 
     def _row_index(self, rows):
@@ -169,7 +184,7 @@ class ShampooBank2(ShampooBank):
         direct, apart = {}, {}
         for o in orders:
             mostly, known = self._replace_first(o), self._known_low_rank(o)
-            direct[o] = mostly or len(known) > self.APART_AT_MOST
+            direct[o] = mostly or len(known) > self.APART_AT_MOST or 4 * len(known) > self.per_order[o]
             apart[o] = [] if direct[o] else known
         apart_y, apart_event, apart_q, apart_back = {}, {}, {}, {}
 

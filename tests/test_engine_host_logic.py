@@ -5,7 +5,7 @@ rank."""
 import pytest
 import torch
 
-from optimizers.engine import ShampooBank
+from optimizers.engine import ShampooBank, _Group
 from optimizers.engine2 import ShampooBank2
 from optimizers.shampoo_common import BlockPartitioner
 
@@ -51,7 +51,7 @@ def test_the_set_of_parameters_of_a_call_is_normalised():
 
 def bare_bank():
     bank = object.__new__(ShampooBank2)
-    bank.low_rank, bank.low_rank_rows = {}, {}
+    bank.low_rank, bank.low_rank_rows, bank.rank_deficient = {}, {}, {}
     return bank
 
 
@@ -102,3 +102,28 @@ def test_low_rank_memory_travels_with_the_checkpoint(monkeypatch):
     ShampooBank2.load_state_dict(other, {"low_rank": low_rank, "low_rank_rows": rows})
     assert other.low_rank == {1024: [True, 3]}
     assert other.low_rank_rows == {768: {5: [16, 15]}}
+
+
+def test_statistics_that_cannot_have_full_rank_are_known_from_the_block_shapes():
+    # ViT-B/32 with blocks of at most 1024: the order-768 statistics of the 768 x 256 blocks (rank <= 384 + 256) and of the
+    # 768 x 100 head (rank <= 384 + 100); every other statistic can have full rank
+    shapes = {(768, 1024): 60, (768, 256): 12, (768, 768): 12, (1024, 768): 39, (768, 100): 1}
+    groups, rows_of = [], {}
+    for (bm, bn), count in shapes.items():
+        g = _Group(bm, bn, bn)
+        g.param_index = list(range(count))
+        for side, order in enumerate((bm, bn)):
+            g.slot[side] = (order, rows_of.get(order, 0))
+            rows_of[order] = rows_of.get(order, 0) + count
+        groups.append(g)
+    found = ShampooBank2._rank_deficient_rows(groups)
+    assert set(found) == {768}
+    first_256 = groups[1].slot[0][1]
+    head = groups[4].slot[0][1]
+    assert found[768] == sorted(list(range(first_256, first_256 + 12)) + [head])
+    bank = bare_bank()
+    bank.rank_deficient = found
+    assert bank._known_low_rank(768) == found[768] and bank._known_low_rank(768) == found[768]     # every update, no countdown
+    bank._note_repairs(768, [0])
+    assert bank._known_low_rank(768) == sorted(found[768] + [0])
+    assert bank._known_low_rank(1024) == []
