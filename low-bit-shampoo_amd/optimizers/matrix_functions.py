@@ -143,7 +143,8 @@ def ComputePowerBatched(mats, p=4, iter_count=10, error_tolerance=1e-6, ridge_ep
     mats.diagonal(dim1=1, dim2=2).add_((ridge_epsilon * top).unsqueeze(1))
     z = (1 + p) / (2 * torch.linalg.matrix_norm(mats))                       # [B]
     R = [torch.zeros(B, n, n, device=dev), torch.empty(B, n, n, device=dev)]
-    R[0].diagonal(dim1=1, dim2=2).copy_(torch.pow(z, 1.0 / p).unsqueeze(1).expand(B, n))
+    first_root = torch.pow(z, 1.0 / p)                                       # the root starts as this multiple of the identity
+    R[0].diagonal(dim1=1, dim2=2).copy_(first_root.unsqueeze(1).expand(B, n))
     M = [mats * z.view(B, 1, 1), torch.empty(B, n, n, device=dev)]
     T = [(1 - w) * eye + w * M[0], torch.empty(B, n, n, device=dev)]
     T2 = torch.empty(B, n, n, device=dev)
@@ -160,14 +161,18 @@ def ComputePowerBatched(mats, p=4, iter_count=10, error_tolerance=1e-6, ridge_ep
 
     R_ptr, M_ptr, T_ptr = table(R), table(M), table(T)
     side = torch.zeros(B, dtype=torch.bool, device=dev)                     # False: buffer 0 holds the state
-    for _ in range(iter_count):
+    for round_number in range(iter_count):
         skip = done.to(torch.int32)
         cur = lambda tab: torch.where(side, tab[1], tab[0])                   # noqa: E731
         oth = lambda tab: torch.where(side, tab[0], tab[1])                   # noqa: E731
         Rc, Ro, Mc, Mo, Tc, To = cur(R_ptr), oth(R_ptr), cur(M_ptr), oth(M_ptr), cur(T_ptr), oth(T_ptr)
         shape = (B, n, n)
-        X.gemm(X.PtrList(Rc, shape), X.PtrList(Tc, shape), out=X.PtrList(Ro, shape), skip=skip,
-               symmetric=symmetric)                                          # candidate root
+        if round_number == 0:
+            # candidate root of the first round: (c I) T = c T, every matrix still in its first buffer
+            torch.mul(T[0], first_root.view(B, 1, 1), out=R[1])
+        else:
+            X.gemm(X.PtrList(Rc, shape), X.PtrList(Tc, shape), out=X.PtrList(Ro, shape), skip=skip,
+                   symmetric=symmetric)                                      # candidate root
         power = X.PtrList(Tc, shape)                                         # T^p by repeated squaring
         done_p = 1
         while done_p < p:
